@@ -1,0 +1,382 @@
+"""Cache manager: pages of keys and values, a block table for each request, and
+slots for per-request state of fixed size.  Pure host code, no tensors.
+
+Layers with the same need form a *group* (all earlier keys, or a window of the
+most recent ones).  A group has its own page pool; a page id addresses the same
+page in the storage of every layer of the group.  A request holds, per group, a
+table from page index (position // page_size) to page id, with -1 where it holds
+no page (never allocated, or given back because a window has passed it).
+
+What the reference does and this keeps: a LIFO free list that hands out page 0
+first (src/engine/kvcache.py:67,149-154,166), reference counts with retain and
+release (kvcache.py:127-147), and a hash chain over full pages for sharing a
+common prefix between requests (kvcache.py:81-125).  What differs: pages go back
+when a request ends (the reference waits for the whole queue, llm_engine.py:147-152);
+a page is registered for sharing only once all its tokens are computed, and the map
+from page to hash is kept, so that a freed page leaves the registry
+(kvcache.py:163-165 pops a map that nothing fills); a reservation is all or nothing.
+"""
+from __future__ import annotations
+
+import hashlib
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+
+class CacheError(RuntimeError):
+    """A request for pages or slots that cannot be met, or a misuse of the manager."""
+
+
+class OutOfPages(CacheError):
+    pass
+
+
+@dataclass(frozen=True)
+class GroupSpec:
+    """The need of a group of layers: ``window`` None keeps every key, an int
+    keeps the ``window`` most recent positions (the current one included)."""
+    window: Optional[int] = None
+
+
+class PagePool:
+    """Pages of one group: LIFO free list and reference counts."""
+
+    def __init__(self, num_pages: int):
+        if num_pages <= 0:
+            raise CacheError("a page pool needs at least one page")
+        self.num_pages = num_pages
+        self.free: List[int] = list(range(num_pages - 1, -1, -1))  # pop() hands out 0 first
+        self.refcount: List[int] = [0] * num_pages
+
+    @property
+    def num_free(self) -> int:
+        return len(self.free)
+
+    def allocate(self) -> int:
+        if not self.free:
+            raise OutOfPages("no free page")
+        page = self.free.pop()
+        if self.refcount[page] != 0:
+            raise CacheError(f"free page {page} has reference count {self.refcount[page]}")
+        self.refcount[page] = 1
+        return page
+
+    def retain(self, page: int) -> None:
+        self._check_id(page)
+        if self.refcount[page] <= 0:
+            raise CacheError(f"cannot retain page {page}: it is free")
+        self.refcount[page] += 1
+
+    def release(self, page: int) -> bool:
+        """Drop one reference; True if the page became free."""
+        self._check_id(page)
+        if self.refcount[page] <= 0:
+            raise CacheError(f"cannot release page {page}: it is free already")
+        self.refcount[page] -= 1
+        if self.refcount[page] == 0:
+            self.free.append(page)
+            return True
+        return False
+
+    def _check_id(self, page: int) -> None:
+        if not 0 <= page < self.num_pages:
+            raise CacheError(f"page id {page} is outside 0..{self.num_pages - 1}")
+
+
+class StateSlots:
+    """Slots for per-request state of fixed size: one index per live request."""
+
+    def __init__(self, num_slots: int):
+        if num_slots <= 0:
+            raise CacheError("at least one state slot is needed")
+        self.num_slots = num_slots
+        self.free: List[int] = list(range(num_slots - 1, -1, -1))
+        self.owner: List[Optional[Hashable]] = [None] * num_slots
+
+    @property
+    def num_free(self) -> int:
+        return len(self.free)
+
+    def take(self, owner: Hashable) -> int:
+        if not self.free:
+            raise CacheError("no free state slot")
+        slot = self.free.pop()
+        self.owner[slot] = owner
+        return slot
+
+    def give_back(self, slot: int) -> None:
+        if not 0 <= slot < self.num_slots or self.owner[slot] is None:
+            raise CacheError(f"state slot {slot} is not held")
+        self.owner[slot] = None
+        self.free.append(slot)
+
+
+def chain_hash(parent: int, tokens: Sequence[int]) -> int:
+    """64-bit hash of a page's tokens chained to the hash of the page before it
+    (the construction of src/engine/kvcache.py:81-86)."""
+    h = hashlib.blake2b(digest_size=8)
+    h.update(int(parent).to_bytes(8, "little", signed=False))
+    for tok in tokens:
+        h.update(int(tok).to_bytes(8, "little", signed=True))
+    return int.from_bytes(h.digest(), "little", signed=False)
+
+
+@dataclass
+class RequestCache:
+    """What one live request holds."""
+    req_id: Hashable
+    state_slot: int
+    tables: List[List[int]]            # per group: page index -> page id or -1
+    num_tokens: int = 0                # positions whose keys are in the cache
+    tokens: List[int] = field(default_factory=list)   # their token ids (for page hashes)
+    hashes: List[int] = field(default_factory=list)   # chain hashes of the full pages so far
+    shared_len: int = 0                # tokens taken over from other requests at admission
+    new_request: bool = True           # no step has run yet: fixed-size state must be cleared
+
+
+@dataclass
+class _SharedEntry:
+    pages: Tuple[int, ...]   # one page id per group
+    tokens: Tuple[int, ...]
+
+
+class CacheManager:
+    def __init__(self, groups: Sequence[GroupSpec], num_pages, page_size: int, max_requests: int,
+                 prefix_sharing: bool = False):
+        if page_size <= 0:
+            raise CacheError("page_size must be positive")
+        self.groups = list(groups)
+        if isinstance(num_pages, int):
+            num_pages = [num_pages] * len(self.groups)
+        if len(num_pages) != len(self.groups):
+            raise CacheError("one page count per group is needed")
+        for g in self.groups:
+            if g.window is not None and g.window <= 0:
+                raise CacheError("a window must be positive")
+        self.page_size = page_size
+        self.pools = [PagePool(n) for n in num_pages]
+        self.slots = StateSlots(max_requests)
+        self.requests: Dict[Hashable, RequestCache] = {}
+        # a prefix can only be shared when every group keeps all keys
+        self.prefix_sharing = bool(prefix_sharing) and bool(self.groups) and \
+            all(g.window is None for g in self.groups)
+        self._shared: Dict[int, _SharedEntry] = {}
+        self._page_hash: Dict[int, int] = {}   # page id of group 0 -> hash it is registered under
+        self.stats = {"pages_allocated": 0, "pages_freed": 0, "shared_page_hits": 0}
+
+    # ---- requests -------------------------------------------------------------
+    def add_request(self, req_id: Hashable) -> RequestCache:
+        if req_id in self.requests:
+            raise CacheError(f"request {req_id!r} is live already")
+        slot = self.slots.take(req_id)
+        rc = RequestCache(req_id=req_id, state_slot=slot, tables=[[] for _ in self.groups])
+        self.requests[req_id] = rc
+        return rc
+
+    def get(self, req_id: Hashable) -> RequestCache:
+        try:
+            return self.requests[req_id]
+        except KeyError:
+            raise CacheError(f"request {req_id!r} is not live") from None
+
+    def free_request(self, req_id: Hashable) -> None:
+        rc = self.get(req_id)
+        for g, table in enumerate(rc.tables):
+            for page in table:
+                if page >= 0:
+                    self._release(g, page)
+            table.clear()
+        self.slots.give_back(rc.state_slot)
+        del self.requests[req_id]
+
+    # ---- pages ------------------------------------------------------------------
+    def _first_live_page(self, g: int, next_pos: int) -> int:
+        """Index of the first page that a query at position >= next_pos can still see."""
+        w = self.groups[g].window
+        if w is None:
+            return 0
+        first_key = max(0, next_pos - w + 1)
+        return first_key // self.page_size
+
+    def pages_needed(self, req_id: Hashable, new_len: int) -> List[int]:
+        """New pages per group for the request to hold positions up to new_len - 1,
+        given that the next step starts at its current length."""
+        rc = self.get(req_id)
+        need = []
+        for g, table in enumerate(rc.tables):
+            lo = self._first_live_page(g, rc.num_tokens)
+            hi = (new_len + self.page_size - 1) // self.page_size
+            n = 0
+            for i in range(lo, hi):
+                if i >= len(table) or table[i] < 0:
+                    n += 1
+            need.append(n)
+        return need
+
+    def can_reserve(self, wants: Sequence[Tuple[Hashable, int]]) -> bool:
+        """True if all of (request, new length) can get their pages together."""
+        total = [0] * len(self.groups)
+        for req_id, new_len in wants:
+            for g, n in enumerate(self.pages_needed(req_id, new_len)):
+                total[g] += n
+        return all(total[g] <= self.pools[g].num_free for g in range(len(self.groups)))
+
+    def reserve(self, req_id: Hashable, new_len: int) -> None:
+        """Give the request pages for every position it will hold up to new_len - 1.
+        All or nothing: raises OutOfPages and changes nothing if a pool is short."""
+        rc = self.get(req_id)
+        if new_len < rc.num_tokens:
+            raise CacheError("a request's length cannot shrink")
+        need = self.pages_needed(req_id, new_len)
+        for g, n in enumerate(need):
+            if n > self.pools[g].num_free:
+                raise OutOfPages(f"group {g} needs {n} pages for request {req_id!r}, "
+                                 f"{self.pools[g].num_free} are free")
+        hi = (new_len + self.page_size - 1) // self.page_size
+        for g, table in enumerate(rc.tables):
+            lo = self._first_live_page(g, rc.num_tokens)
+            while len(table) < hi:
+                table.append(-1)
+            for i in range(lo, hi):
+                if table[i] < 0:
+                    table[i] = self.pools[g].allocate()
+                    self.stats["pages_allocated"] += 1
+
+    def commit(self, req_id: Hashable, tokens: Sequence[int]) -> None:
+        """The step has written these tokens' keys: lengthen the request, register pages
+        that became full for sharing, and give back pages that a window has passed."""
+        rc = self.get(req_id)
+        new_len = rc.num_tokens + len(tokens)
+        for g, table in enumerate(rc.tables):
+            if len(table) * self.page_size < new_len:
+                raise CacheError(f"request {req_id!r} has no pages reserved up to {new_len}")
+        rc.tokens.extend(int(t) for t in tokens)
+        rc.num_tokens = new_len
+        rc.new_request = False
+        if self.prefix_sharing:
+            self._register_full_pages(rc)
+        for g, table in enumerate(rc.tables):
+            if self.groups[g].window is None:
+                continue
+            live_from = self._first_live_page(g, new_len)
+            for i in range(min(live_from, len(table))):
+                if table[i] >= 0:
+                    self._release(g, table[i])
+                    table[i] = -1
+
+    def _release(self, g: int, page: int) -> None:
+        if self.pools[g].release(page):
+            self.stats["pages_freed"] += 1
+            if g == 0:
+                h = self._page_hash.pop(page, None)
+                if h is not None:
+                    self._shared.pop(h, None)
+
+    # ---- tables and slots for a step ------------------------------------------------
+    def block_table(self, req_id: Hashable, group: int) -> List[int]:
+        return self.get(req_id).tables[group]
+
+    def token_slots(self, req_id: Hashable, group: int, start: int, count: int) -> List[int]:
+        """page * page_size + offset for positions start .. start + count - 1."""
+        table = self.get(req_id).tables[group]
+        P = self.page_size
+        out = []
+        for pos in range(start, start + count):
+            page = table[pos // P]
+            if page < 0:
+                raise CacheError(f"request {req_id!r} holds no page for position {pos} in group {group}")
+            out.append(page * P + pos % P)
+        return out
+
+    # ---- prefix sharing ----------------------------------------------------------
+    def match_prefix(self, req_id: Hashable, prompt: Sequence[int]) -> int:
+        """For a request that holds nothing yet: take over the pages of the longest
+        registered run of full pages that equals the prompt's beginning.  At least one
+        prompt token is always left to compute.  Returns the number of tokens taken over."""
+        rc = self.get(req_id)
+        if rc.num_tokens or any(rc.tables[g] for g in range(len(self.groups))):
+            raise CacheError("a prefix can only be matched for a request that holds nothing")
+        if not self.prefix_sharing:
+            return 0
+        P = self.page_size
+        max_pages = (len(prompt) - 1) // P if prompt else 0
+        parent = 0
+        taken: List[_SharedEntry] = []
+        hashes = []
+        for i in range(max_pages):
+            toks = tuple(int(t) for t in prompt[i * P:(i + 1) * P])
+            h = chain_hash(parent, toks)
+            entry = self._shared.get(h)
+            if entry is None or entry.tokens != toks:   # the token test guards against collisions
+                break
+            taken.append(entry)
+            hashes.append(h)
+            parent = h
+        for entry in taken:
+            for g, page in enumerate(entry.pages):
+                self.pools[g].retain(page)
+                rc.tables[g].append(page)
+        n = len(taken) * P
+        rc.num_tokens = n
+        rc.shared_len = n
+        rc.tokens = [int(t) for t in prompt[:n]]
+        rc.hashes = hashes
+        self.stats["shared_page_hits"] += len(taken)
+        return n
+
+    def _register_full_pages(self, rc: RequestCache) -> None:
+        P = self.page_size
+        full = rc.num_tokens // P
+        while len(rc.hashes) < full:
+            i = len(rc.hashes)
+            toks = tuple(rc.tokens[i * P:(i + 1) * P])
+            parent = rc.hashes[-1] if rc.hashes else 0
+            h = chain_hash(parent, toks)
+            rc.hashes.append(h)
+            pages = tuple(rc.tables[g][i] for g in range(len(self.groups)))
+            if h not in self._shared and pages[0] not in self._page_hash:
+                self._shared[h] = _SharedEntry(pages=pages, tokens=toks)
+                self._page_hash[pages[0]] = h
+
+    # ---- whole-manager views -------------------------------------------------------
+    def num_free_pages(self, group: int = 0) -> int:
+        return self.pools[group].num_free
+
+    def reset(self) -> None:
+        for req_id in list(self.requests):
+            self.free_request(req_id)
+        self._shared.clear()
+        self._page_hash.clear()
+
+    def check_invariants(self) -> None:
+        """No page lost, held twice without a count, or both free and held."""
+        for g, pool in enumerate(self.pools):
+            held: Dict[int, int] = {}
+            for rc in self.requests.values():
+                seen = set()
+                for page in rc.tables[g]:
+                    if page < 0:
+                        continue
+                    if page in seen:
+                        raise CacheError(f"request {rc.req_id!r} holds page {page} twice in group {g}")
+                    seen.add(page)
+                    held[page] = held.get(page, 0) + 1
+            free = set(pool.free)
+            if len(free) != len(pool.free):
+                raise CacheError(f"group {g}: a page is in the free list twice")
+            for page in range(pool.num_pages):
+                rcnt = pool.refcount[page]
+                if rcnt != held.get(page, 0):
+                    raise CacheError(f"group {g}: page {page} has count {rcnt}, "
+                                     f"{held.get(page, 0)} requests hold it")
+                if (rcnt == 0) != (page in free):
+                    raise CacheError(f"group {g}: page {page} count {rcnt}, in free list: {page in free}")
+        for h, entry in self._shared.items():
+            for g, page in enumerate(entry.pages):
+                if self.pools[g].refcount[page] <= 0:
+                    raise CacheError(f"registered page {page} of group {g} is free")
+            if self._page_hash.get(entry.pages[0]) != h:
+                raise CacheError("the two maps of the prefix registry disagree")
+        owners = [o for o in self.slots.owner if o is not None]
+        if sorted(map(repr, owners)) != sorted(map(repr, self.requests)):
+            raise CacheError("state slots and live requests disagree")

@@ -1,0 +1,93 @@
+// Shared device helpers for the gfx950 kernels: element types, conversions,
+// wave64 reductions and the error convention of the C entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define QE_WAVE 64
+
+// Element type codes used across the C ABI.
+enum QeDtype { QE_F32 = 0, QE_BF16 = 1 };
+
+// bfloat16 held as its 16 bits; conversions are explicit so that every rounding
+// point is visible in the kernels.
+struct bf16_t { uint16_t bits; };
+
+__device__ __forceinline__ float bf16_to_float(bf16_t v) {
+    return __uint_as_float(((uint32_t)v.bits) << 16);
+}
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t bits16) {
+    return __uint_as_float(bits16 << 16);
+}
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t float_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    bf16_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) { r.bits = (uint16_t)((u >> 16) | 0x0040u); return r; }
+    u += 0x7fffu + ((u >> 16) & 1u);
+    r.bits = (uint16_t)(u >> 16);
+    return r;
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static __device__ __forceinline__ float load(const float* p) { return *p; }
+    static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <> struct Elem<bf16_t> {
+    static __device__ __forceinline__ float load(const bf16_t* p) { return bf16_to_float(*p); }
+    static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = float_to_bf16(v); }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Block-wide sum for blocks of up to 1024 threads (a multiple of 64).
+// `scratch` holds at least 16 floats of shared memory.  All threads get the sum.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) scratch[wid] = v;
+    __syncthreads();
+    float r = 0.f;
+    for (int i = 0; i < nw; ++i) r += scratch[i];
+    return r;
+}
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) scratch[wid] = v;
+    __syncthreads();
+    float r = scratch[0];
+    for (int i = 1; i < nw; ++i) r = fmaxf(r, scratch[i]);
+    return r;
+}
+
+// ---- host side ---------------------------------------------------------------
+// Entry points return 0 on success, a positive hipError_t, or -1 for an argument
+// the kernels do not take; qe_last_error() then holds the reason.
+extern "C" const char* qe_last_error();
+void qe_set_error(const char* fmt, ...);
+
+#define QE_REQUIRE(cond, ...)                         \
+    do {                                              \
+        if (!(cond)) { qe_set_error(__VA_ARGS__); return -1; } \
+    } while (0)
+
+#define QE_LAUNCH_CHECK()                             \
+    do {                                              \
+        hipError_t e_ = hipGetLastError();            \
+        if (e_ != hipSuccess) { qe_set_error("%s: %s", __func__, hipGetErrorString(e_)); return (int)e_; } \
+    } while (0)
+
+static inline int qe_cdiv(long a, long b) { return (int)((a + b - 1) / b); }

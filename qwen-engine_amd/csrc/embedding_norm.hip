@@ -1,0 +1,123 @@
+// Embedding gather into the 32-bit residual stream, and RMSNorm with an optional
+// fused residual add and an optional row gather.
+#include "common.h"
+
+// out[t, :] = float(table[ids[t], :]).  One block per token.
+template <typename TW>
+__global__ void embedding_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
+                                 float* __restrict__ out, int H) {
+    const long t = blockIdx.x;
+    const TW* row = table + (long)ids[t] * H;
+    float* o = out + t * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) o[c] = Elem<TW>::load(row + c);
+}
+
+extern "C" int qe_embedding(const int* ids, const void* table, float* out, int T, int V, int H,
+                            int dt_w, hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && V > 0 && H > 0, "embedding: bad sizes T=%d V=%d H=%d", T, V, H);
+    if (T == 0) return 0;
+    const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+    if (dt_w == QE_F32)
+        embedding_kernel<float><<<T, threads, 0, stream>>>(ids, (const float*)table, out, H);
+    else if (dt_w == QE_BF16)
+        embedding_kernel<bf16_t><<<T, threads, 0, stream>>>(ids, (const bf16_t*)table, out, H);
+    else
+        QE_REQUIRE(false, "embedding: unknown table dtype %d", dt_w);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// One block per output row r.  src row = rows ? rows[r] : r.
+//   v = h[src] (+ delta[src]);  if delta and !rows: h[src] = v  (the residual sum, in 32-bit)
+//   out[r] = v * rsqrt(mean(v^2) + eps) * w        (all in 32-bit, one rounding at the store)
+// Two passes over the row; the second re-reads h (and delta) instead of keeping
+// the row in registers, so any H is taken.
+template <typename TA>
+__global__ void rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__ delta,
+                               const int* __restrict__ rows, const float* __restrict__ w,
+                               TA* __restrict__ out, int H, float eps) {
+    __shared__ float red[16];
+    const long r = blockIdx.x;
+    const long src = rows ? (long)rows[r] : r;
+    float* hr = h + src * H;
+    const TA* dr = delta ? delta + src * H : nullptr;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = hr[c];
+        if (dr) v += Elem<TA>::load(dr + c);
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float rstd = rsqrtf(ss / (float)H + eps);
+    TA* o = out + r * H;
+    const bool write_back = dr && !rows;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = hr[c];
+        if (dr) v += Elem<TA>::load(dr + c);
+        if (write_back) hr[c] = v;
+        Elem<TA>::store(o + c, v * rstd * w[c]);
+    }
+}
+
+extern "C" int qe_rmsnorm(float* h, const void* delta, const int* rows, const float* w, void* out,
+                          int n_out_rows, int H, float eps, int dt_a, hipStream_t stream) {
+    QE_REQUIRE(n_out_rows >= 0 && H > 0, "rmsnorm: bad sizes rows=%d H=%d", n_out_rows, H);
+    if (n_out_rows == 0) return 0;
+    const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
+    if (dt_a == QE_F32)
+        rmsnorm_kernel<float><<<n_out_rows, threads, 0, stream>>>(h, (const float*)delta, rows, w, (float*)out, H, eps);
+    else if (dt_a == QE_BF16)
+        rmsnorm_kernel<bf16_t><<<n_out_rows, threads, 0, stream>>>(h, (const bf16_t*)delta, rows, w, (bf16_t*)out, H, eps);
+    else
+        QE_REQUIRE(false, "rmsnorm: unknown dtype %d", dt_a);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// h[t, :] += delta[t, :]  (for blocks whose norm does not fuse the residual sum)
+template <typename TA>
+__global__ void residual_add_kernel(float* __restrict__ h, const TA* __restrict__ delta, long n) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        h[i] += Elem<TA>::load(delta + i);
+}
+
+extern "C" int qe_residual_add(float* h, const void* delta, long n, int dt_a, hipStream_t stream) {
+    if (n <= 0) return 0;
+    const int blocks = (int)((n + 255) / 256 > 4096 ? 4096 : (n + 255) / 256);
+    if (dt_a == QE_F32)
+        residual_add_kernel<float><<<blocks, 256, 0, stream>>>(h, (const float*)delta, n);
+    else if (dt_a == QE_BF16)
+        residual_add_kernel<bf16_t><<<blocks, 256, 0, stream>>>(h, (const bf16_t*)delta, n);
+    else
+        QE_REQUIRE(false, "residual_add: unknown dtype %d", dt_a);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// out[t, i] = silu(gu[t, i]) * gu[t, I + i], the product formed in 32-bit.
+template <typename TA>
+__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int T, int I) {
+    const long n = (long)T * I;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (long)gridDim.x * blockDim.x) {
+        const long t = idx / I;
+        const int i = (int)(idx - t * I);
+        const float g = Elem<TA>::load(gu + t * 2 * I + i);
+        const float u = Elem<TA>::load(gu + t * 2 * I + I + i);
+        Elem<TA>::store(out + idx, g / (1.f + expf(-g)) * u);
+    }
+}
+
+extern "C" int qe_silu_mul(const void* gu, void* out, int T, int I, int dt_a, hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && I > 0, "silu_mul: bad sizes T=%d I=%d", T, I);
+    if (T == 0) return 0;
+    const long n = (long)T * I;
+    const int blocks = (int)((n + 255) / 256 > 8192 ? 8192 : (n + 255) / 256);
+    if (dt_a == QE_F32)
+        silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, T, I);
+    else if (dt_a == QE_BF16)
+        silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, T, I);
+    else
+        QE_REQUIRE(false, "silu_mul: unknown dtype %d", dt_a);
+    QE_LAUNCH_CHECK();
+    return 0;
+}

@@ -1,0 +1,37 @@
+"""The flat batch that one step runs: portions of prompts beside single decoded
+tokens.  The same description serves every mixer; each consumes what it needs."""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional
+
+import torch
+
+from ..parts.base import Runtime
+
+
+@dataclass
+class SeqInfo:
+    """One request's share of the step (host side)."""
+    req_id: Hashable
+    q_start: int        # first row of the request's tokens in the flat batch
+    q_len: int          # number of its tokens in this step
+    kv_before: int      # tokens already in its cache = position of its first new token
+    state_slot: int
+    new_request: bool   # its first step: fixed-size state starts from zero
+
+
+@dataclass
+class StepContext:
+    rt: Runtime
+    page_size: int
+    num_tokens: int
+    seqs: List[SeqInfo]
+    token_ids: torch.Tensor            # int32 [T]
+    positions: torch.Tensor            # int32 [T] absolute position of each token
+    tok_seq: torch.Tensor              # int32 [T] index into seqs / rows of the block tables
+    block_tables: List[torch.Tensor]   # per cache group: int32 [B, max_blocks], -1 where no page
+    slots: List[torch.Tensor]          # per cache group: int32 [T] page * page_size + offset
+    logit_rows: torch.Tensor           # int32 [R] rows whose logits are wanted
+    state_slots: torch.Tensor          # int32 [B]
+    max_position: int = 0              # largest position in the batch (host)

@@ -1,0 +1,287 @@
+"""Python bindings of the HIP kernels: each function checks on the host that the
+operands have the shapes, element types, layout and device that the kernel and
+its grid assume, then launches on the current HIP stream.
+
+There is no fallback: if the library cannot be built or loaded, or no GPU is
+present, importing the kernels fails with the reason.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+ALGO_AUTO, ALGO_GENERIC = 0, 1
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def load_library():
+    """Load (building first if need be) the kernel library.  Raises if there is no GPU."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not torch.cuda.is_available():
+        raise KernelError("no GPU is visible: the engine has no CPU path")
+    path = _build.library_path()
+    lib = ctypes.CDLL(str(path))
+    lib.qe_last_error.restype = ctypes.c_char_p
+    vp, i32, f32, i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_long
+    sigs = {
+        "qe_embedding": [vp, vp, vp, i32, i32, i32, i32, vp],
+        "qe_rmsnorm": [vp, vp, vp, vp, vp, i32, i32, f32, i32, vp],
+        "qe_residual_add": [vp, vp, i64, i32, vp],
+        "qe_silu_mul": [vp, vp, i32, i32, i32, vp],
+        "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp],
+        "qe_qk_rope_store": [vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
+        "qe_attention": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp],
+        "qe_argmax": [vp, vp, i32, i32, vp],
+        "qe_sample": [vp, vp, vp, vp, i32, i32, vp],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = ctypes.c_int
+    _lib = lib
+    return lib
+
+
+def library_file() -> str:
+    load_library()
+    return str(_build.library_path(verbose=False))
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = _lib.qe_last_error().decode(errors="replace")
+        raise KernelError(f"{what}: {msg} (code {rc})")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, shape=None, device=None) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name} is no tensor")
+    if not t.is_cuda:
+        raise KernelError(f"{name} is not on the GPU")
+    if device is not None and t.device != device:
+        raise KernelError(f"{name} is on {t.device}, expected {device}")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} is not contiguous")
+    if dtype is not None:
+        ok = t.dtype in dtype if isinstance(dtype, (tuple, list)) else t.dtype == dtype
+        if not ok:
+            raise KernelError(f"{name} has element type {t.dtype}, expected {dtype}")
+    if shape is not None:
+        if t.dim() != len(shape) or any(s is not None and int(s) != int(a) for s, a in zip(shape, t.shape)):
+            raise KernelError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+
+_ACT = (torch.float32, torch.bfloat16)
+
+
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = float32(table[ids[t]]).  ids int32 [T] with 0 <= id < V (the caller checks the range)."""
+    lib = load_library()
+    _need(ids, "ids", torch.int32, (None,))
+    _need(table, "table", _ACT, (None, None), ids.device)
+    T, (V, H) = ids.shape[0], table.shape
+    if out is None:
+        out = torch.empty((T, H), dtype=torch.float32, device=ids.device)
+    _need(out, "out", torch.float32, (T, H), ids.device)
+    _check(lib.qe_embedding(ids.data_ptr(), table.data_ptr(), out.data_ptr(), T, V, H,
+                            _DT[table.dtype], _stream()), "embedding")
+    return out
+
+
+def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMSNorm of the 32-bit stream h [T, H] into out_dtype.
+
+    With ``delta`` the residual sum h + delta is normed; it is written back to h
+    unless ``rows`` is given.  With ``rows`` (int32 [R]) only those rows are normed
+    and the result is [R, H].
+    """
+    lib = load_library()
+    _need(h, "h", torch.float32, (None, None))
+    T, H = h.shape
+    _need(weight, "weight", torch.float32, (H,), h.device)
+    if delta is not None:
+        _need(delta, "delta", out_dtype, (T, H), h.device)
+    n = T
+    if rows is not None:
+        _need(rows, "rows", torch.int32, (None,), h.device)
+        n = rows.shape[0]
+    if out is None:
+        out = torch.empty((n, H), dtype=out_dtype, device=h.device)
+    _need(out, "out", out_dtype, (n, H), h.device)
+    _check(lib.qe_rmsnorm(h.data_ptr(), _ptr(delta), _ptr(rows), weight.data_ptr(), out.data_ptr(),
+                          n, H, float(eps), _DT[out_dtype], _stream()), "rmsnorm")
+    return out
+
+
+def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
+    """h += delta, h in 32-bit."""
+    lib = load_library()
+    _need(h, "h", torch.float32)
+    _need(delta, "delta", _ACT, tuple(h.shape), h.device)
+    _check(lib.qe_residual_add(h.data_ptr(), delta.data_ptr(), h.numel(), _DT[delta.dtype], _stream()),
+           "residual_add")
+
+
+def silu_mul(gu: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """gu [T, 2 I] = gate | up  ->  silu(gate) * up  [T, I]."""
+    lib = load_library()
+    _need(gu, "gu", _ACT, (None, None))
+    T, I2 = gu.shape
+    if I2 % 2:
+        raise KernelError(f"silu_mul: the width {I2} of gate|up is odd")
+    I = I2 // 2
+    if out is None:
+        out = torch.empty((T, I), dtype=gu.dtype, device=gu.device)
+    _need(out, "out", gu.dtype, (T, I), gu.device)
+    _check(lib.qe_silu_mul(gu.data_ptr(), out.data_ptr(), T, I, _DT[gu.dtype], _stream()), "silu_mul")
+    return out
+
+
+def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+         out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
+         algo: int = ALGO_AUTO) -> torch.Tensor:
+    """x [M, K] . w [N, K]^T (+ bias [N], 32-bit) -> [M, N] in out_dtype (default: x's)."""
+    lib = load_library()
+    _need(x, "x", _ACT, (None, None))
+    M, K = x.shape
+    _need(w, "w", _ACT, (None, K), x.device)
+    N = w.shape[0]
+    if x.dtype == torch.float32 and w.dtype != torch.float32:
+        raise KernelError("gemm: 32-bit activations need 32-bit weights")
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (N,), x.device)
+    out_dtype = out_dtype or x.dtype
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _need(out, "out", out_dtype, (M, N), x.device)
+    _check(lib.qe_gemm(x.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), M, N, K,
+                       _DT[x.dtype], _DT[w.dtype], _DT[out_dtype], algo, _stream()), "gemm")
+    return out
+
+
+def qk_rope_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                  positions: Optional[torch.Tensor], q_weight: Optional[torch.Tensor],
+                  k_weight: Optional[torch.Tensor], eps: float, table: Optional[torch.Tensor],
+                  slots: Optional[torch.Tensor], cache: Optional[torch.Tensor], page_size: int,
+                  q_out: Optional[torch.Tensor] = None, packed: bool = False) -> torch.Tensor:
+    """Per-head q/k norm (if weights), rotation (if table), cache write (if slots) of qkv
+    [T, (Hq + 2 Hkv) D].  cache: one layer's pages [pages, 2, Hkv, P, D].  Returns q [T, Hq, D];
+    with ``packed`` it returns all heads [T, Hq + 2 Hkv, D] instead and writes no cache.
+    The caller guarantees positions < table rows and slots < pages * P."""
+    lib = load_library()
+    T = qkv.shape[0]
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _need(qkv, "qkv", _ACT, (T, width))
+    dev = qkv.device
+    if positions is not None:
+        _need(positions, "positions", torch.int32, (T,), dev)
+    if (q_weight is None) != (k_weight is None):
+        raise KernelError("qk_rope_store: q and k norm weights come together")
+    if q_weight is not None:
+        _need(q_weight, "q_weight", torch.float32, (head_dim,), dev)
+        _need(k_weight, "k_weight", torch.float32, (head_dim,), dev)
+    rotary_dim = 0
+    if table is not None:
+        _need(table, "table", torch.float32, (None, None), dev)
+        rotary_dim = table.shape[1]
+        if positions is None:
+            raise KernelError("qk_rope_store: a rotation needs positions")
+    if slots is not None:
+        _need(slots, "slots", torch.int32, (T,), dev)
+        if cache is None:
+            raise KernelError("qk_rope_store: slots without a cache")
+        _need(cache, "cache", qkv.dtype, (None, 2, num_kv_heads, page_size, head_dim), dev)
+    packed_out = None
+    if packed:
+        if slots is not None:
+            raise KernelError("qk_rope_store: the packed form writes no cache")
+        packed_out = torch.empty((T, num_heads + 2 * num_kv_heads, head_dim), dtype=qkv.dtype, device=dev)
+    else:
+        if q_out is None:
+            q_out = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=dev)
+        _need(q_out, "q_out", qkv.dtype, (T, num_heads, head_dim), dev)
+    _check(lib.qe_qk_rope_store(qkv.data_ptr(), _ptr(positions), _ptr(q_weight), _ptr(k_weight),
+                                float(eps), _ptr(table), rotary_dim, _ptr(slots), _ptr(cache),
+                                _ptr(q_out), _ptr(packed_out), T, num_heads, num_kv_heads, head_dim,
+                                page_size, _DT[qkv.dtype], _stream()), "qk_rope_store")
+    return packed_out if packed else q_out
+
+
+def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
+              block_table: torch.Tensor, scale: float, window: int = 0,
+              out: Optional[torch.Tensor] = None, algo: int = ALGO_AUTO) -> torch.Tensor:
+    """q [T, Hq, D]; cache [pages, 2, Hkv, P, D]; positions, tok_seq int32 [T];
+    block_table int32 [B, max_blocks].  Token t sees the keys at positions
+    max(0, p - window + 1) .. p of request tok_seq[t] (window 0: all).  The caller
+    guarantees that those positions have pages in the table."""
+    lib = load_library()
+    _need(q, "q", _ACT, (None, None, None))
+    T, Hq, D = q.shape
+    dev = q.device
+    _need(cache, "cache", q.dtype, (None, 2, None, None, D), dev)
+    Hkv, P = cache.shape[2], cache.shape[3]
+    _need(positions, "positions", torch.int32, (T,), dev)
+    _need(tok_seq, "tok_seq", torch.int32, (T,), dev)
+    _need(block_table, "block_table", torch.int32, (None, None), dev)
+    if out is None:
+        out = torch.empty_like(q)
+    _need(out, "out", q.dtype, (T, Hq, D), dev)
+    _check(lib.qe_attention(q.data_ptr(), out.data_ptr(), cache.data_ptr(), positions.data_ptr(),
+                            tok_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, Hq,
+                            Hkv, D, P, float(scale), int(window), _DT[q.dtype], algo, _stream()),
+           "attention")
+    return out
+
+
+def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Lowest index of the largest logit per row; logits float32 [R, V] -> int32 [R]."""
+    lib = load_library()
+    _need(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    if out is None:
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _need(out, "out", torch.int32, (R,), logits.device)
+    _check(lib.qe_argmax(logits.data_ptr(), out.data_ptr(), R, V, _stream()), "argmax")
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Inverse-CDF draw from softmax(logits / temperature) per row with uniform[r] in [0, 1).
+    Every temperature must be positive."""
+    lib = load_library()
+    _need(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    _need(temperature, "temperature", torch.float32, (R,), logits.device)
+    _need(uniform, "uniform", torch.float32, (R,), logits.device)
+    if out is None:
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _need(out, "out", torch.int32, (R,), logits.device)
+    _check(lib.qe_sample(logits.data_ptr(), temperature.data_ptr(), uniform.data_ptr(), out.data_ptr(),
+                         R, V, _stream()), "sample")
+    return out

@@ -1,0 +1,53 @@
+"""A pre-norm residual block: x += mixer(norm(x)); x += ffn(norm(x))
+(src/models/qwen3/model.py:278-298).  The residual stream is kept in 32-bit and each
+residual sum is fused into the norm that follows it, so the block hands its last
+branch output on as ``pending`` instead of adding it itself."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .base import CacheBinding, Runtime, TensorInfo
+from .registry import build_part, part_class, register_part
+
+# checkpoint names of the four parts inside a layer's prefix
+_NAMES = ("input_layernorm", "self_attn", "post_attention_layernorm", "mlp")
+
+
+def _names(spec):
+    return getattr(spec, "part_names", _NAMES)
+
+
+class PreNormBlock:
+    def __init__(self, spec, hidden_size: int):
+        self.spec = spec
+        self.hidden = int(hidden_size)
+        self.mixer_norm = build_part(spec.mixer_norm, hidden_size)
+        self.mixer = build_part(spec.mixer, hidden_size)
+        self.ffn_norm = build_part(spec.ffn_norm, hidden_size)
+        self.ffn = build_part(spec.ffn, hidden_size)
+
+    @staticmethod
+    def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
+        out: Dict[str, TensorInfo] = {}
+        for name, sub in zip(_names(spec), (spec.mixer_norm, spec.mixer, spec.ffn_norm, spec.ffn)):
+            for rel, info in part_class(sub.kind).expected_tensors(sub, hidden).items():
+                out[f"{name}.{rel}"] = info
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        for name, part in zip(_names(self.spec), (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)):
+            pre = name + "."
+            part.load({k[len(pre):]: v for k, v in tensors.items() if k.startswith(pre)}, rt)
+
+    def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], ctx, binding: CacheBinding) -> torch.Tensor:
+        """h: 32-bit residual stream (updated in place).  pending: branch output not yet
+        added to h, or None.  Returns the feed-forward output, to be added by whoever norms next."""
+        x = self.mixer_norm.forward(h, ctx.rt, delta=pending)
+        a = self.mixer.forward(x, ctx, binding)
+        x = self.ffn_norm.forward(h, ctx.rt, delta=a)
+        return self.ffn.forward(x, ctx)
+
+
+register_part("prenorm_block", PreNormBlock)

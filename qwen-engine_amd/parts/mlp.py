@@ -1,0 +1,44 @@
+"""Dense gated feed-forward: down(silu(gate x) * up x), no biases
+(src/models/qwen3/model.py:232-237; silu.mul as src/layers/fused_ops/silumul.py:46-53,
+with the product formed in 32-bit before the one rounding).  gate and up are one
+product with the two weights stacked."""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..kernels import ops
+from .base import Runtime, TensorInfo
+from .registry import register_part
+
+
+class SwiGLU:
+    def __init__(self, spec, hidden_size: int):
+        self.hidden = int(hidden_size)
+        self.inter = int(spec.intermediate_size)
+        self.w_gu = self.w_down = None
+
+    @staticmethod
+    def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
+        i = spec.intermediate_size
+        return {
+            "gate_proj.weight": TensorInfo((i, hidden)),
+            "up_proj.weight": TensorInfo((i, hidden)),
+            "down_proj.weight": TensorInfo((hidden, i)),
+        }
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        if g.dtype != u.dtype:
+            g, u = g.float(), u.float()
+        self.w_gu = rt.place_matrix(torch.cat([g, u], dim=0))
+        self.w_down = rt.place_matrix(tensors["down_proj.weight"])
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        gu = ops.gemm(x, self.w_gu)
+        a = ops.silu_mul(gu)
+        return ops.gemm(a, self.w_down)
+
+
+register_part("swiglu", SwiGLU)

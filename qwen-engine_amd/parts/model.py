@@ -1,0 +1,99 @@
+"""The decoder: embedding, the layers in the order of the schedule, final norm on
+the wanted rows, head (src/models/qwen3/model.py:349-359,420-422; the head is applied
+only where logits are asked for, and gives 32-bit logits)."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..cache.plan import CachePlan, plan_cache
+from ..config.spec import ModelSpec
+from ..kernels import ops
+from .base import CacheBinding, Runtime, TensorInfo
+from .registry import build_part, part_class
+
+
+def expected_tensors(spec: ModelSpec) -> Dict[str, TensorInfo]:
+    """Every tensor the model folder must hold, by checkpoint name."""
+    out: Dict[str, TensorInfo] = {spec.embed_name: TensorInfo((spec.vocab_size, spec.hidden_size), "normal", "matrix")}
+    for layer in spec.layers:
+        for rel, info in part_class(layer.kind).expected_tensors(layer, spec.hidden_size).items():
+            out[f"{layer.prefix}.{rel}"] = info
+    norm_rel = part_class(spec.final_norm.kind).expected_tensors(spec.final_norm, spec.hidden_size)
+    base = spec.final_norm_name[:-len(".weight")] if spec.final_norm_name.endswith(".weight") else spec.final_norm_name
+    for rel, info in norm_rel.items():
+        out[f"{base}.{rel}"] = info
+    if not spec.tie_head:
+        out[spec.head_name] = TensorInfo((spec.vocab_size, spec.hidden_size), "normal", "matrix")
+    return out
+
+
+def cache_plan(spec: ModelSpec) -> CachePlan:
+    needs = []
+    for entry in spec.schedule:
+        mixer_spec = spec.layers[entry.layer].mixer
+        cls = part_class(mixer_spec.kind)
+        kv = cls.cache_need(mixer_spec) if hasattr(cls, "cache_need") else None
+        state = cls.state_need(mixer_spec, spec.hidden_size) if hasattr(cls, "state_need") else None
+        needs.append((kv, state, entry.cache_from))
+    return plan_cache(needs)
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec):
+        spec.validate()
+        self.spec = spec
+        self.blocks = [build_part(layer, spec.hidden_size) for layer in spec.layers]
+        self.final_norm = build_part(spec.final_norm, spec.hidden_size)
+        self.embed: Optional[torch.Tensor] = None
+        self.head: Optional[torch.Tensor] = None
+        self.rt: Optional[Runtime] = None
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        spec = self.spec
+        self.rt = rt
+        self.embed = rt.place_matrix(tensors[spec.embed_name])
+        for layer, block in zip(spec.layers, self.blocks):
+            pre = layer.prefix + "."
+            block.load({k[len(pre):]: v for k, v in tensors.items() if k.startswith(pre)}, rt)
+        base = spec.final_norm_name[:-len(".weight")] if spec.final_norm_name.endswith(".weight") else spec.final_norm_name
+        self.final_norm.load({k[len(base) + 1:]: v for k, v in tensors.items() if k.startswith(base + ".")}, rt)
+        self.head = self.embed if spec.tie_head else rt.place_matrix(tensors[spec.head_name])
+
+    def weight_bytes_read_per_step(self) -> int:
+        """Bytes of every weight a step uses once (the embedding table only where it is the head)."""
+        seen, total = set(), 0
+
+        def add(t):
+            nonlocal total
+            if isinstance(t, torch.Tensor) and t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                total += t.numel() * t.element_size()
+
+        counts: Dict[int, int] = {}
+        for e in self.spec.schedule:
+            counts[e.layer] = counts.get(e.layer, 0) + 1
+        for idx, n in counts.items():
+            b = self.blocks[idx]
+            before = total
+            for part in (b.mixer_norm, b.mixer, b.ffn_norm, b.ffn):
+                for v in vars(part).values():
+                    add(v)
+            total += (n - 1) * (total - before)
+        for v in vars(self.final_norm).values():
+            add(v)
+        add(self.head)
+        return total
+
+    def forward(self, ctx, bindings: List[CacheBinding]) -> torch.Tensor:
+        """Runs the tokens of ctx through the schedule; returns float32 logits [R, V]."""
+        h = ops.embedding(ctx.token_ids, self.embed)
+        pending = None
+        for i, entry in enumerate(self.spec.schedule):
+            pending = self.blocks[entry.layer].forward(h, pending, ctx, bindings[i])
+        R = ctx.logit_rows.shape[0]
+        if R == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=h.device)
+        x = self.final_norm.forward(h, ctx.rt, delta=pending, rows=ctx.logit_rows)
+        return ops.gemm(x, self.head, out_dtype=torch.float32)
