@@ -1,0 +1,192 @@
+"""What pins the plain implementation beside the reference's text (CPU): the vectors
+of the reference's own operator tests, special cases that reduce to a library routine,
+and invariants; each chosen so that a plausible mistake fails it."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from plain import qwen3_plain as P
+from tiny import TINY_A, TINY_B, make_folder
+
+
+def rand(*shape, seed=0, dtype=torch.float32):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=dtype)
+
+
+# ---- RMSNorm ----------------------------------------------------------------------------
+def test_rms_norm_is_the_library_routine_at_the_reference_test_shape():
+    x = torch.rand(32, 2048, generator=torch.Generator().manual_seed(1))     # layernorm.py:216-226,270
+    w = rand(2048, seed=2)
+    got = P.rms_norm(x, w, 1e-6)
+    want = F.rms_norm(x, (2048,), weight=w, eps=1e-6)                      # layernorm.py:209-214
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_rms_norm_invariants():
+    x = rand(5, 3, 48, seed=3)
+    ones = torch.ones(48)
+    y = P.rms_norm(x, ones, 1e-12)
+    torch.testing.assert_close((y * y).mean(-1), torch.ones(5, 3), rtol=1e-5, atol=1e-6)   # rows have RMS 1
+    torch.testing.assert_close(P.rms_norm(7.5 * x, ones, 1e-12), y, rtol=1e-5, atol=1e-6)  # scale invariant
+    w = rand(48, seed=4)
+    flat = P.rms_norm(x.reshape(15, 48), w, 1e-6).reshape(5, 3, 48)
+    torch.testing.assert_close(P.rms_norm(x, w, 1e-6), flat)              # 3-D = rows sharing w
+    # eps sits inside the root, next to the mean: a zero row stays zero and finite
+    assert torch.equal(P.rms_norm(torch.zeros(2, 8), torch.ones(8), 1e-6), torch.zeros(2, 8))
+    big_eps = P.rms_norm(torch.full((1, 4), 2.0), torch.ones(4), 5.0)
+    torch.testing.assert_close(big_eps, torch.full((1, 4), 2.0 / 3.0))     # 2 / sqrt(4 + 5)
+
+
+# ---- linear, embedding, silu.mul --------------------------------------------------------------
+def test_linear_embedding_silu_reduce_to_library_routines():
+    x, w = rand(256, 512, seed=5), rand(1024, 512, seed=6)                 # linear.py:188-201,255
+    torch.testing.assert_close(P.linear(x, w), F.linear(x, w), rtol=1e-4, atol=1e-4)
+    b = rand(1024, seed=7)
+    torch.testing.assert_close(P.linear(x, w, b), F.linear(x, w, b), rtol=1e-4, atol=1e-4)
+    ids = torch.randint(0, 1024, (32,), generator=torch.Generator().manual_seed(8))
+    table = rand(1024, 2048, seed=9)                                       # embedding.py:140-151,196
+    assert torch.equal(P.embedding(ids, table), F.embedding(ids, table))
+    g, u = rand(256, 2048, seed=10), rand(256, 2048, seed=11)              # silumul.py:160-176,225
+    torch.testing.assert_close(P.silu_mul(g, u), F.silu(g) * u, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(P.silu_mul(g, torch.ones_like(g)), F.silu(g), rtol=1e-5, atol=1e-6)
+    assert torch.equal(P.silu_mul(torch.zeros(3), u[0, :3]), torch.zeros(3))
+
+
+# ---- rotation -------------------------------------------------------------------------------
+def test_rope_table_rows():
+    t = P.rope_table(10000.0, 8, 16)
+    assert t.shape == (16, 8)
+    torch.testing.assert_close(t[0], torch.tensor([1., 1, 1, 1, 0, 0, 0, 0]))
+    freqs = torch.tensor([1.0, 10000 ** -0.25, 10000 ** -0.5, 10000 ** -0.75])
+    torch.testing.assert_close(t[5, :4], torch.cos(5 * freqs))
+    torch.testing.assert_close(t[5, 4:], torch.sin(5 * freqs))
+
+
+def test_rope_pairs_feature_i_with_i_plus_half_and_turns_counterclockwise():
+    d = 8
+    t = P.rope_table(10000.0, d, 4)
+    x = torch.zeros(1, 1, d)
+    x[0, 0, 0] = 1.0
+    y = P.apply_rope(t, torch.tensor([1]), x)[0, 0]
+    want = torch.zeros(d)
+    want[0], want[d // 2] = math.cos(1.0), math.sin(1.0)   # interleaved pairing would put sin at index 1,
+    torch.testing.assert_close(y, want)                     # a wrong sign would give -sin
+    x = torch.zeros(1, 1, d)
+    x[0, 0, d // 2 + 1] = 1.0
+    y = P.apply_rope(t, torch.tensor([2]), x)[0, 0]
+    f1 = 10000 ** -0.25
+    want = torch.zeros(d)
+    want[1], want[d // 2 + 1] = -math.sin(2 * f1), math.cos(2 * f1)
+    torch.testing.assert_close(y, want)
+
+
+def test_rope_invariants_at_the_reference_test_shape():
+    d = 128
+    t = P.rope_table(1e6, d, 2048)
+    pos = torch.randint(0, 2048, (32,), generator=torch.Generator().manual_seed(12))   # rope.py:276-300,359-364
+    q, k = rand(32, 32, d, seed=13), rand(32, 16, d, seed=14)
+    rq, rk = P.apply_rope(t, pos, q), P.apply_rope(t, pos, k)
+    assert torch.equal(P.apply_rope(t, torch.zeros(32, dtype=torch.long), q), q)       # position 0: identity
+    pair = lambda z: z[..., :d // 2] ** 2 + z[..., d // 2:] ** 2
+    torch.testing.assert_close(pair(rq), pair(q), rtol=1e-4, atol=1e-5)                # each pair keeps its length
+    # <rope(q, m), rope(k, n)> depends on m - n only
+    a, b = rand(1, 1, d, seed=15), rand(1, 1, d, seed=16)
+    dot = lambda m, n: (P.apply_rope(t, torch.tensor([m]), a) * P.apply_rope(t, torch.tensor([n]), b)).sum()
+    torch.testing.assert_close(dot(17, 5), dot(1012, 1000), rtol=1e-3, atol=1e-3)
+    assert abs(dot(17, 5) - dot(17, 6)) > 1e-3
+
+
+# ---- attention --------------------------------------------------------------------------------
+def test_attention_without_mask_is_the_library_routine():
+    q, k, v = rand(7, 4, 16, seed=20), rand(7, 4, 16, seed=21), rand(7, 4, 16, seed=22)
+    got = P.attention(q, k, v, 0.3, causal=False)
+    want = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None],
+                                          v.transpose(0, 1)[None], scale=0.3)[0].transpose(0, 1)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_causal_attention_with_cached_prefix_is_the_reference_twin():
+    # 5 new tokens after 6 cached ones, explicit mask q_abs_pos >= k_abs_pos (attn.py:767-780)
+    hq, hkv, d = 6, 2, 16
+    q, k, v = rand(5, hq, d, seed=23), rand(11, hkv, d, seed=24), rand(11, hkv, d, seed=25)
+    got = P.attention(q, k, v, 0.25)
+    mask = (6 + torch.arange(5))[:, None] >= torch.arange(11)[None, :]
+    want = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None],
+                                          v.transpose(0, 1)[None], attn_mask=mask[None, None],
+                                          scale=0.25, enable_gqa=True)[0].transpose(0, 1)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+    # grouped = each kv head repeated for the heads of its group, in blocks (h // group)
+    rep = P.attention(q, k.repeat_interleave(3, dim=1), v.repeat_interleave(3, dim=1), 0.25)
+    torch.testing.assert_close(got, rep)
+
+
+def test_attention_edge_cases():
+    q, k, v = rand(3, 2, 8, seed=26), rand(3, 1, 8, seed=27), rand(3, 1, 8, seed=28)
+    out = P.attention(q, k, v, 1.0)
+    torch.testing.assert_close(out[0], v[0].expand(2, 8))          # the first token sees one key: itself
+    one_head = P.attention(q[:, :1], k, v, 1.0)
+    torch.testing.assert_close(one_head, out[:, :1])
+    # a window of 1 returns each token's own value; a window as long as the sequence changes nothing
+    torch.testing.assert_close(P.attention(q, k, v, 1.0, window=1), v.expand(3, 2, 8))
+    torch.testing.assert_close(P.attention(q, k, v, 1.0, window=3), out)
+    w2 = P.attention(q, k, v, 1.0, window=2)
+    torch.testing.assert_close(w2[:2], out[:2])
+    assert not torch.allclose(w2[2], out[2])
+
+
+# ---- whole model ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_logits_depend_on_distances_only(tmp_path, which):
+    folder = make_folder(tmp_path, which, dtype=torch.float32, std=0.05)
+    cfg, w = P.read_folder(folder)
+    toks = torch.randint(0, cfg["vocab_size"], (20,), generator=torch.Generator().manual_seed(3)).tolist()
+    base = P.forward_logits(cfg, w, toks)
+    assert base.shape == (20, cfg["vocab_size"])
+    shifted = P.forward_logits(cfg, w, toks, position_offset=37)
+    torch.testing.assert_close(shifted, base, rtol=1e-3, atol=2e-4)
+    # causal: a later token does not change earlier logits
+    other = P.forward_logits(cfg, w, toks[:12] + [(toks[12] + 1) % cfg["vocab_size"]] + toks[13:])
+    torch.testing.assert_close(other[:12], base[:12])
+    assert not torch.allclose(other[12:], base[12:])
+    f64 = P.forward_logits(cfg, w, toks, compute=torch.float64)
+    torch.testing.assert_close(base.double(), f64, rtol=1e-4, atol=1e-5)
+
+
+def test_tied_head_is_the_embedding_table(tmp_path):
+    folder = make_folder(tmp_path, "A", dtype=torch.float32, std=0.05)
+    cfg, w = P.read_folder(folder)
+    assert "lm_head.weight" not in w
+    toks = [1, 2, 3, 4]
+    base = P.forward_logits(cfg, w, toks)
+    untied = dict(cfg, tie_word_embeddings=False)
+    w2 = dict(w)
+    w2["lm_head.weight"] = w["model.embed_tokens.weight"]
+    torch.testing.assert_close(P.forward_logits(untied, w2, toks), base)
+
+
+def test_norm_comes_before_rotation_and_only_without_bias(tmp_path):
+    folder = make_folder(tmp_path, "B", dtype=torch.float32, std=0.05)
+    cfg, w = P.read_folder(folder)
+    x = rand(6, cfg["hidden_size"], seed=30)
+    pos = torch.arange(6)
+    table = P.rope_table(P.rope_theta_of(cfg), cfg["head_dim"], 64)
+    w = dict(w)
+    base = P.attention_block(x, pos, w, "model.layers.0", cfg, table)
+    # scaling q_proj changes nothing when q is normalised per head afterwards (up to eps = 1e-5
+    # beside a mean square near 0.2: a relative change of some 1e-5 in the scores)
+    w["model.layers.0.self_attn.q_proj.weight"] = 3.0 * w["model.layers.0.self_attn.q_proj.weight"]
+    torch.testing.assert_close(P.attention_block(x, pos, w, "model.layers.0", cfg, table), base, rtol=1e-3, atol=2e-5)
+    # with bias there is no q/k norm (model.py:204-206): the same scaling now matters
+    biased = dict(cfg, attention_bias=True)
+    for n, width in (("q", 192), ("k", 32), ("v", 32)):
+        w[f"model.layers.0.self_attn.{n}_proj.bias"] = torch.zeros(width)
+    a = P.attention_block(x, pos, w, "model.layers.0", biased, table)
+    w["model.layers.0.self_attn.q_proj.weight"] = w["model.layers.0.self_attn.q_proj.weight"] / 3.0
+    b = P.attention_block(x, pos, w, "model.layers.0", biased, table)
+    assert not torch.allclose(a, b, rtol=1e-3, atol=1e-5)
+
+
+def test_greedy_takes_the_lowest_index_on_ties():
+    assert P.greedy(torch.tensor([[1.0, 3.0, 3.0, 2.0], [0.0, 0.0, 0.0, 0.0]])) == [1, 0]

@@ -1,0 +1,201 @@
+"""The scheduler's decisions (CPU), against the real cache manager and a stand-in for
+the step function whose "model" makes the next token a hash of all tokens so far."""
+import hashlib
+
+import pytest
+
+import qwen_engine_amd  # noqa: F401
+from qwen_engine_amd.cache import CacheManager, GroupSpec
+from qwen_engine_amd.engine.scheduler import Request, Scheduler
+from qwen_engine_amd.sampling import SamplingParams
+
+
+def fake_next(tokens):
+    h = hashlib.blake2b(repr(list(tokens)).encode(), digest_size=4).digest()
+    return int.from_bytes(h, "little") % 97 + 3          # never 0..2 (used as eos below)
+
+
+def drive(sched, cache, log=None, max_steps=10_000):
+    """What LLMEngine.step does, with the fake model: reserve, commit, sample, update."""
+    steps = 0
+    while sched.has_work():
+        planned = sched.plan()
+        if not planned:
+            break
+        assert len({p.request.req_id for p in planned}) == len(planned)
+        assert sum(len(p.tokens) for p in planned) <= sched.max_step_tokens
+        assert cache.can_reserve([(p.request.req_id, p.request.num_computed + len(p.tokens)) for p in planned])
+        sampled = []
+        for p in planned:
+            r = p.request
+            assert p.tokens == r.known[r.num_computed:r.num_computed + len(p.tokens)]
+            assert cache.get(r.req_id).num_tokens == r.num_computed
+            cache.reserve(r.req_id, r.num_computed + len(p.tokens))
+            cache.commit(r.req_id, p.tokens)
+            if p.sample:
+                sampled.append(fake_next(r.known))
+        if log is not None:
+            log.append([(p.request.req_id, len(p.tokens), p.sample) for p in planned])
+        sched.update(planned, sampled)
+        cache.check_invariants()
+        steps += 1
+        assert steps < max_steps
+    return steps
+
+
+def make(num_pages=64, page=4, max_num_seqs=4, max_model_len=256, budget=64, chunk=16, eos=(), sharing=False):
+    cache = CacheManager([GroupSpec()], num_pages, page_size=page, max_requests=max_num_seqs, prefix_sharing=sharing)
+    return Scheduler(cache, max_num_seqs, max_model_len, budget, chunk, eos), cache
+
+
+def expected_output(prompt, n):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        t = fake_next(toks)
+        out.append(t)
+        toks.append(t)
+    return out
+
+
+PROMPTS = [[5, 6, 7, 8, 9], list(range(10, 19)), list(range(20, 33)), [40] * 30]
+
+
+def test_every_request_gets_exactly_its_tokens():
+    sched, cache = make()
+    reqs = [Request(i, p, SamplingParams(max_new_tokens=8)) for i, p in enumerate(PROMPTS)]
+    for r in reqs:
+        sched.add(r)
+    drive(sched, cache)
+    for r in reqs:
+        assert r.finish_reason == "length" and r.output == expected_output(r.prompt, 8)
+    assert all(pool.num_free == pool.num_pages for pool in cache.pools)      # freed at finish
+    assert cache.slots.num_free == 4
+
+
+def test_outputs_do_not_depend_on_sizes_of_the_engine():
+    want = [expected_output(p, 10) for p in PROMPTS]
+    for kw in (dict(max_num_seqs=1), dict(budget=3, chunk=2), dict(budget=7, chunk=6), dict(num_pages=14),
+               dict(page=1, num_pages=60), dict(sharing=True), dict(num_pages=11, budget=5, chunk=4)):
+        sched, cache = make(**kw)
+        reqs = [Request(i, p, SamplingParams(max_new_tokens=10)) for i, p in enumerate(PROMPTS)]
+        for r in reqs:
+            sched.add(r)
+        drive(sched, cache)
+        assert [r.output for r in reqs] == want, kw
+        assert all(pool.num_free == pool.num_pages for pool in cache.pools)
+
+
+def test_prompts_are_cut_under_the_budget_and_mixed_with_decodes():
+    sched, cache = make(budget=8, chunk=6)
+    a = Request(0, list(range(3, 8)), SamplingParams(max_new_tokens=6))
+    b = Request(1, list(range(30, 50)), SamplingParams(max_new_tokens=2))
+    sched.add(a)
+    sched.add(b)
+    log = []
+    drive(sched, cache, log)
+    # step 0: a's whole prompt (5), then b's first portion cut to the 3 tokens that are left
+    assert log[0] == [(0, 5, True), (1, 3, False)]
+    # step 1: a decodes one token beside b's next portion of 6 (the chunk size)
+    assert log[1] == [(0, 1, True), (1, 6, False)]
+    assert log[2] == [(0, 1, True), (1, 6, False)]
+    assert log[3] == [(0, 1, True), (1, 5, True)]        # b's last portion gives its first token
+    assert all(sum(n for _, n, _ in step) <= 8 for step in log)
+
+
+def test_admission_is_first_in_first_out_and_bounded():
+    sched, cache = make(max_num_seqs=2)
+    reqs = [Request(i, [7 + i] * 6, SamplingParams(max_new_tokens=3)) for i in range(5)]
+    for r in reqs:
+        sched.add(r)
+    log = []
+    drive(sched, cache, log)
+    first_seen = {}
+    for s, step in enumerate(log):
+        assert len(step) <= 2
+        for rid, _, _ in step:
+            first_seen.setdefault(rid, s)
+    assert [first_seen[i] for i in range(5)] == sorted(first_seen[i] for i in range(5))
+
+
+def test_stops_on_eos_unless_told_not_to():
+    prompt = [5, 6, 7]
+    out = expected_output(prompt, 12)
+    eos = out[4]
+    first = out.index(eos)
+    sched, cache = make(eos=(eos,))
+    r = Request(0, prompt, SamplingParams(max_new_tokens=12))
+    r2 = Request(1, prompt, SamplingParams(max_new_tokens=12, ignore_eos=True))
+    sched.add(r)
+    sched.add(r2)
+    drive(sched, cache)
+    assert r.finish_reason == "stop" and r.output == out[:first + 1]
+    assert r2.finish_reason == "length" and r2.output == out
+
+
+def test_length_is_capped_by_max_model_len():
+    sched, cache = make(max_model_len=12)
+    r = Request(0, list(range(3, 11)), SamplingParams(max_new_tokens=50))
+    sched.add(r)
+    drive(sched, cache)
+    assert r.finish_reason == "length" and len(r.prompt) + len(r.output) == 12
+    too_long = Request(1, [4] * 12, SamplingParams())
+    sched.add(too_long)
+    assert too_long.finish_reason == "error" and "max_model_len" in too_long.error
+
+
+def test_when_pages_run_out_the_newest_request_is_preempted_and_recomputed():
+    # 3 requests of 8 + 12 tokens need 5 pages each at the end; 9 pages cannot hold them all
+    sched, cache = make(num_pages=9, page=4, max_num_seqs=3)
+    reqs = [Request(i, [11 * (i + 1)] * 8, SamplingParams(max_new_tokens=12)) for i in range(3)]
+    for r in reqs:
+        sched.add(r)
+    drive(sched, cache)
+    assert sched.stats["preemptions"] > 0
+    assert reqs[0].preemptions == 0                      # the oldest is never the victim
+    for r in reqs:
+        assert r.finish_reason == "length" and r.output == expected_output(r.prompt, 12)
+    assert all(pool.num_free == pool.num_pages for pool in cache.pools)
+
+
+def test_a_request_that_can_never_fit_fails_alone():
+    sched, cache = make(num_pages=3, page=4)
+    big = Request(0, [9] * 20, SamplingParams(max_new_tokens=2))      # 6 pages > 3
+    small = Request(1, [8] * 5, SamplingParams(max_new_tokens=2))
+    grows = Request(2, [7] * 10, SamplingParams(max_new_tokens=30))   # fits at first, then outgrows the pool
+    for r in (big, small, grows):
+        sched.add(r)
+    drive(sched, cache)
+    assert big.finish_reason == "error" and "cache is too small" in big.error
+    assert small.finish_reason == "length" and small.output == expected_output(small.prompt, 2)
+    assert grows.finish_reason == "error" and grows.output == expected_output(grows.prompt, len(grows.output))
+    assert all(pool.num_free == pool.num_pages for pool in cache.pools)
+
+
+def test_shared_prefix_is_taken_over_at_admission():
+    sched, cache = make(page=4, sharing=True, max_num_seqs=2, budget=64, chunk=64)
+    common = list(range(50, 66))                          # 16 tokens = 4 pages
+    a = Request(0, common + [1, 2, 3], SamplingParams(max_new_tokens=4))
+    b = Request(1, common + [4, 5], SamplingParams(max_new_tokens=4))
+    sched.add(a)
+    log = []
+    planned = sched.plan()
+    for p in planned:
+        cache.reserve(p.request.req_id, p.request.num_computed + len(p.tokens))
+        cache.commit(p.request.req_id, p.tokens)
+    sched.update(planned, [fake_next(a.known)])
+    sched.add(b)
+    drive(sched, cache, log)
+    assert (1, 2, True) in log[0]                         # b computes only its own two tokens
+    assert sched.stats["shared_prefix_tokens"] == 16
+    assert a.output == expected_output(a.prompt, 4) and b.output == expected_output(b.prompt, 4)
+
+
+def test_bad_requests_are_refused():
+    sched, _ = make()
+    r = Request(0, [], SamplingParams())
+    sched.add(r)
+    assert r.finish_reason == "error"
+    with pytest.raises(ValueError):
+        sched.add(Request(1, [1], SamplingParams(max_new_tokens=0)))
+    with pytest.raises(ValueError):
+        sched.add(Request(2, [1], SamplingParams(temperature=-1.0)))
