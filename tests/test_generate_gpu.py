@@ -1,0 +1,167 @@
+"""Generation through the entry points on the GPU: greedy tokens equal the plain
+implementation's, whatever the engine's sizes; long decoding; the first tokens of a
+sequence; temperature sampling does not depend on the batch."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import qwen_engine_amd
+from qwen_engine_amd import EngineConfig, LLMEngine, SamplingParams, generate
+from plain import qwen3_plain as P
+from tiny import TINY, make_folder
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("gen")
+    return {w: make_folder(tmp, w, dtype=torch.bfloat16, std=0.08) for w in "AB"}
+
+
+def prompts_for(cfg, lengths, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lengths]
+
+
+def test_greedy_generation_equals_the_plain_implementation(folders):
+    """BASELINE workload of the first tiny configuration: prompts of 5, 9 and 13 tokens, 8 greedy tokens."""
+    cfg, w = P.read_folder(folders["A"])
+    prompts = prompts_for(cfg, (5, 9, 13), 1)
+    want = [P.greedy_generate(cfg, w, p, 8) for p in prompts]
+    res = generate(folders["A"], prompts, SamplingParams(max_new_tokens=8, ignore_eos=True),
+                   EngineConfig(dtype="float32", block_size=4, max_num_seqs=4, max_model_len=64))
+    assert [r.token_ids for r in res] == want
+    assert all(r.finish_reason == "length" for r in res)
+    assert [r.prompt_token_ids for r in res] == prompts
+
+
+@pytest.mark.parametrize("sizes", [dict(max_num_seqs=1), dict(max_step_tokens=7, prefill_chunk=6),
+                                   dict(num_blocks=9, block_size=8), dict(block_size=1, num_blocks=200),
+                                   dict(enable_prefix_sharing=False)])
+def test_outputs_do_not_depend_on_the_engine_sizes(folders, sizes):
+    """Second tiny configuration: prompts of 1, 7, 16 and 30 tokens, two sharing 16 tokens; portions
+    of 6 mixed with decoding; few pages (preemption); greedy and temperature 0.7 with a fixed seed."""
+    cfg, w = P.read_folder(folders["B"])
+    p = prompts_for(cfg, (1, 7, 16, 30), 2)
+    p[3] = p[2] + p[3][16:]                               # the last two share a prefix of 16 tokens
+    want = [P.greedy_generate(cfg, w, q, 10) for q in p]
+    base = dict(dtype="float32", block_size=8, max_num_seqs=4, max_model_len=48, prefill_chunk=6)
+    base.update(sizes)
+    eng = LLMEngine.from_folder(folders["B"], EngineConfig(**base))
+    eng.submit(p, max_new_tokens=10, ignore_eos=True)
+    res = eng.run()
+    assert [r.token_ids for r in res] == want
+    eng.runner.cache.check_invariants()
+    assert all(pool.num_free == pool.num_pages for pool in eng.runner.cache.pools)
+    # temperature: the same tokens as a run of each request alone with the same seed
+    eng.submit(p, max_new_tokens=10, temperature=0.7, seed=11, ignore_eos=True)
+    together = [r.token_ids for r in eng.run()]
+    ref_engine = LLMEngine.from_folder(folders["B"], EngineConfig(dtype="float32", block_size=8, max_num_seqs=1,
+                                                                  max_model_len=48))
+    alone = []
+    for i, q in enumerate(p):
+        ref_engine._next_id = eng._next_id - len(p) + i    # the draw is keyed by (seed, request id, position)
+        ref_engine.submit([q], max_new_tokens=10, temperature=0.7, seed=11, ignore_eos=True)
+        alone.append(ref_engine.run()[0].token_ids)
+    assert together == alone
+    assert together != want                                # and it is not greedy
+
+
+def test_shared_prefix_pages_are_taken_over(folders):
+    cfg, w = P.read_folder(folders["B"])
+    common = prompts_for(cfg, (32,), 3)[0]
+    a, b = common + [5, 6, 7], common + [9]
+    eng = LLMEngine.from_folder(folders["B"], EngineConfig(dtype="float32", block_size=8, max_num_seqs=2,
+                                                           max_model_len=64))
+    eng.submit([a], max_new_tokens=4, ignore_eos=True)
+    eng.step()                                            # a's prompt is computed, a is still live
+    eng.submit([b], max_new_tokens=4, ignore_eos=True)
+    res = eng.run()
+    assert eng.stats()["shared_prefix_tokens"] == 32
+    assert res[0].token_ids == P.greedy_generate(cfg, w, a, 4)
+    assert res[1].token_ids == P.greedy_generate(cfg, w, b, 4)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """300 tokens decoded one by one after a short prompt: logits at every decoded position equal
+    the plain implementation's on the whole sequence (pages fill and new ones are taken 75 times)."""
+    from qwen_engine_amd.engine import ModelRunner, StepEntry, load_model
+    cfg, w = P.read_folder(folders["A"])
+    toks = prompts_for(cfg, (305,), 4)[0]
+    act = None if dtype == "float32" else torch.bfloat16
+    ref = P.forward_logits(cfg, w, toks, act_dtype=act)
+    runner = ModelRunner(load_model(folders["A"], dtype=dtype), page_size=4, num_pages=80, max_requests=1)
+    runner.add_request("r")
+    rows = [runner.step([StepEntry("r", toks[:5], [4])])]
+    for i in range(5, 305):
+        rows.append(runner.step([StepEntry("r", toks[i:i + 1], [0])]))
+    got = torch.cat(rows).cpu()
+    tol = 1e-4 if dtype == "float32" else 2e-2
+    err = (got - ref[4:]).abs().max(dim=1).values / ref.abs().max()
+    bad = torch.nonzero(err > tol)
+    assert bad.numel() == 0, f"first wrong position {int(bad[0]) + 4}, error {float(err[bad[0]])}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(folders, dtype):
+    """Positions 0, 1 and 2, each asked for alone and together, over a page size of 1 and of 8."""
+    from qwen_engine_amd.engine import ModelRunner, StepEntry, load_model
+    cfg, w = P.read_folder(folders["B"])
+    toks = prompts_for(cfg, (3,), 5)[0]
+    act = None if dtype == "float32" else torch.bfloat16
+    ref = P.forward_logits(cfg, w, toks, act_dtype=act)
+    tol = (1e-4 if dtype == "float32" else 2e-2) * float(ref.abs().max())
+    model = load_model(folders["B"], dtype=dtype)
+    for page in (1, 8):
+        runner = ModelRunner(model, page_size=page, num_pages=8, max_requests=2)
+        runner.add_request("a")
+        runner.add_request("b")
+        one = [runner.step([StepEntry("a", toks[i:i + 1], [0])]).cpu()[0] for i in range(3)]
+        together = runner.step([StepEntry("b", toks, [0, 1, 2])]).cpu()
+        for i in range(3):
+            assert (one[i] - ref[i]).abs().max() <= tol and (together[i] - ref[i]).abs().max() <= tol
+
+
+def test_step_refuses_bad_entries(folders):
+    from qwen_engine_amd.cache import OutOfPages
+    from qwen_engine_amd.engine import ModelRunner, StepEntry, load_model
+    runner = ModelRunner(load_model(folders["A"], dtype="float32"), page_size=4, num_pages=2, max_requests=2)
+    runner.add_request("a")
+    with pytest.raises(ValueError):
+        runner.step([StepEntry("a", [256], [0])])           # outside the vocabulary
+    with pytest.raises(ValueError):
+        runner.step([StepEntry("a", [1, 2], [2])])          # wants a place it does not bring
+    with pytest.raises(ValueError):
+        runner.step([StepEntry("a", [1], []), StepEntry("a", [2], [])])
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("a", list(range(9)), [])])   # 3 pages, the pool has 2
+    assert runner.cache.num_free_pages() == 2                # nothing was taken
+    assert runner.step([StepEntry("a", list(range(8)), [7])]).shape == (1, 256)
+
+
+def test_command_line(folders, tmp_path):
+    """main.py with the reference's option names: random weights from a config file, prompts as ids."""
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(TINY["A"][0]))
+    out = tmp_path / "model"
+    cmd = [sys.executable, os.path.join(ROOT, "main.py"), "--random-weights", str(cfg_path), "--seed", "4",
+           "--model-name-or-path", str(out), "--prompt-ids", "5,6,7,8", "--prompt-ids", "9,10",
+           "--max-new-tokens", "5", "--max-num-seqs", "2", "--max-model-len", "32", "--block-size", "4",
+           "--model-dtype", "float32", "--ignore-eos", "--stats"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr[-2000:]
+    cfg, w = P.read_folder(str(out))
+    want = [P.greedy_generate(cfg, w, p, 5) for p in ([5, 6, 7, 8], [9, 10])]
+    lines = r.stdout.splitlines()
+    assert "Prompt: 5 6 7 8" in lines and "Prompt: 9 10" in lines
+    assert " ".join(map(str, [5, 6, 7, 8] + want[0])) in lines
+    assert " ".join(map(str, [9, 10] + want[1])) in lines
+    stats = json.loads(lines[-1])
+    assert stats["decode_tokens"] == 8 and stats["prefill_tokens"] == 6

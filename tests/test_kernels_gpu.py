@@ -1,0 +1,300 @@
+"""Each HIP kernel alone against a plain 32-bit reference, at other sizes than the
+engine's: widths and vocabularies that are no power of two, head sizes in steps of 16,
+several head groupings and page sizes.  Inputs are made so that faults show: one key
+far away or at a page's or a window's edge carries the whole result."""
+import math
+
+import pytest
+import torch
+
+import qwen_engine_amd  # noqa: F401
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from qwen_engine_amd.kernels import ops
+    ops.load_library()
+    return ops
+
+
+def rand(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def close(got, want, dtype, scale=None):
+    got, want = got.float().cpu(), want.float().cpu()
+    s = float(want.abs().max()) if scale is None else scale
+    tol = 2e-5 if dtype == torch.float32 else 1.2e-2
+    err = float((got - want).abs().max())
+    assert err <= tol * max(s, 1e-6), f"error {err} beside scale {s}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding(ops, dtype):
+    table = rand(331, 80, seed=1, dtype=dtype)
+    ids = torch.tensor([0, 330, 5, 5, 17, 200], dtype=torch.int32)
+    out = ops.embedding(ids.to(DEV), table.to(DEV))
+    assert out.dtype == torch.float32
+    assert torch.equal(out.cpu(), P.embedding(ids, table).float())     # a copy: exact
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H", [80, 1024, 3000])
+def test_rmsnorm_plain_fused_and_gathered(ops, dtype, H):
+    h = rand(7, H, seed=2, scale=3.0)
+    w = 1 + rand(H, seed=3, scale=0.1)
+    delta = rand(7, H, seed=4, dtype=dtype)
+    eps = 1e-5
+    close(ops.rmsnorm(h.to(DEV), w.to(DEV), eps, dtype), P.rms_norm(h, w, eps), dtype)
+    hd = h.to(DEV)
+    out = ops.rmsnorm(hd, w.to(DEV), eps, dtype, delta=delta.to(DEV))
+    total = h + delta.float()
+    close(out, P.rms_norm(total, w, eps), dtype)
+    assert torch.equal(hd.cpu(), total)                                # the residual sum, in 32-bit
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32)
+    hd = h.to(DEV)
+    out = ops.rmsnorm(hd, w.to(DEV), eps, dtype, delta=delta.to(DEV), rows=rows.to(DEV))
+    close(out, P.rms_norm(total[rows.long()], w, eps), dtype)
+    assert torch.equal(hd.cpu(), h)                                    # gathered: h is left alone
+
+
+def test_rmsnorm_eps_is_inside_the_root(ops):
+    h = torch.full((1, 64), 2.0)
+    out = ops.rmsnorm(h.to(DEV), torch.ones(64, device=DEV), 5.0, torch.float32)
+    torch.testing.assert_close(out.cpu(), torch.full((1, 64), 2.0 / 3.0))
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 500, 96), (5, 331, 80), (64, 64, 64), (130, 77, 200), (3, 2048, 1024)])
+@pytest.mark.parametrize("dt_x,dt_w,dt_o", [(torch.float32, torch.float32, torch.float32),
+                                            (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+                                            (torch.bfloat16, torch.bfloat16, torch.float32),
+                                            (torch.bfloat16, torch.float32, torch.bfloat16)])
+def test_gemm_generic(ops, M, N, K, dt_x, dt_w, dt_o):
+    x, w = rand(M, K, seed=5, dtype=dt_x), rand(N, K, seed=6, dtype=dt_w, scale=0.1)
+    bias = rand(N, seed=7)
+    want = P.linear(x.double(), w.double())
+    got = ops.gemm(x.to(DEV), w.to(DEV), out_dtype=dt_o, algo=ops.ALGO_GENERIC)
+    assert got.dtype == dt_o
+    close(got, want, dt_o)
+    got = ops.gemm(x.to(DEV), w.to(DEV), bias.to(DEV), out_dtype=dt_o, algo=ops.ALGO_GENERIC)
+    close(got, want + bias.double(), dt_o)
+
+
+def test_float32_gemm_keeps_what_reduced_precision_loses(ops):
+    # 1 + 2^-12 is exact in float32, lost in bfloat16 or tf32-like modes
+    x = torch.full((2, 64), 1.0 + 2.0 ** -12)
+    w = torch.ones(3, 64)
+    got = ops.gemm(x.to(DEV), w.to(DEV)).cpu()
+    assert torch.equal(got, torch.full((2, 3), 64.0 * (1.0 + 2.0 ** -12)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(ops, dtype):
+    gu = rand(9, 2 * 112, seed=8, dtype=dtype, scale=2.0)
+    got = ops.silu_mul(gu.to(DEV))
+    g, u = gu[:, :112].float(), gu[:, 112:].float()
+    close(got, P.silu_mul(g, u), dtype)
+    ones = torch.cat([g, torch.ones_like(g)], dim=1).to(dtype)
+    close(ops.silu_mul(ones.to(DEV)), torch.nn.functional.silu(ones[:, :112].float()), dtype)
+
+
+def paged_cache(k, v, page, perm_seed, dtype, extra_pages=3):
+    """k, v [L, Hkv, D] -> (cache [pages, 2, Hkv, P, D], block table row) with shuffled pages."""
+    L, hkv, d = k.shape
+    n = (L + page - 1) // page
+    g = torch.Generator().manual_seed(perm_seed)
+    ids = torch.randperm(n + extra_pages, generator=g)[:n]
+    cache = torch.full((n + extra_pages, 2, hkv, page, d), float("nan")).to(dtype)
+    for pos in range(L):
+        cache[ids[pos // page], 0, :, pos % page] = k[pos]
+        cache[ids[pos // page], 1, :, pos % page] = v[pos]
+    return cache, ids.to(torch.int32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,d,page", [(4, 2, 16, 4), (6, 1, 32, 8), (6, 2, 48, 16), (8, 8, 64, 1),
+                                           (3, 3, 80, 5), (16, 8, 128, 16), (2, 1, 256, 64)])
+def test_attention_over_pages(ops, dtype, hq, hkv, d, page):
+    """Two requests in one batch: a portion of 9 tokens after 140 cached ones, and a decoded token
+    at position 70.  Pages are shuffled and unused pages hold NaN."""
+    scale = 1 / math.sqrt(d)
+    lens = [(140, 9), (70, 1)]
+    qs, pos, seq, tables, caches, want = [], [], [], [], [], []
+    base_page = 0
+    for b, (before, n) in enumerate(lens):
+        L = before + n
+        k, v = rand(L, hkv, d, seed=10 + b, dtype=dtype), rand(L, hkv, d, seed=20 + b, dtype=dtype)
+        q = rand(n, hq, d, seed=30 + b, dtype=dtype)
+        cache, ids = paged_cache(k, v, page, 40 + b, dtype)
+        tables.append(ids + base_page)
+        base_page += cache.shape[0]
+        caches.append(cache)
+        qs.append(q)
+        pos += list(range(before, L))
+        seq += [b] * n
+        want.append(P.attention(q.float(), k.float(), v.float(), scale))
+    width = max(len(t) for t in tables)
+    table = torch.full((2, width), -1, dtype=torch.int32)
+    for b, t in enumerate(tables):
+        table[b, :len(t)] = t
+    out = ops.attention(torch.cat(qs).to(DEV), torch.cat(caches).to(DEV),
+                        torch.tensor(pos, dtype=torch.int32, device=DEV),
+                        torch.tensor(seq, dtype=torch.int32, device=DEV), table.to(DEV), scale)
+    assert not torch.isnan(out.float()).any()
+    close(out, torch.cat(want), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page", [4, 16])
+@pytest.mark.parametrize("key_pos", [0, 3, 4, 63, 64, 127, 128, 511, 700])
+def test_one_far_key_among_hundreds_decides(ops, dtype, page, key_pos):
+    """A query at position 700 whose score with one key stands out returns that key's value:
+    a kernel that skips or misplaces a key (a page's edge, a chunk's edge, the first or the
+    last key) returns something else."""
+    hq = hkv = 2
+    d, L = 32, 701
+    k = rand(L, hkv, d, seed=50, dtype=dtype, scale=0.1)
+    v = rand(L, hkv, d, seed=51, dtype=dtype)
+    q = rand(1, hq, d, seed=52, dtype=dtype)
+    k[key_pos] = (q[0].float() * 8).to(dtype)               # score ~ 8 |q|^2 / sqrt(d): far above the rest
+    cache, ids = paged_cache(k, v, page, 53, dtype)
+    out = ops.attention(q.to(DEV), cache.to(DEV), torch.tensor([L - 1], dtype=torch.int32, device=DEV),
+                        torch.zeros(1, dtype=torch.int32, device=DEV), ids[None].to(DEV), 1 / math.sqrt(d))
+    want = P.attention(q.float(), k.float(), v.float(), 1 / math.sqrt(d))
+    close(out, want, dtype)
+    assert float((want[0] - v[key_pos].float()).abs().max()) < 0.05     # the input does what it is meant to
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 5, 64, 65, 100])
+def test_window_edge(ops, dtype, window):
+    """The key just inside the window decides the result when it stands out; the key just
+    outside must not, however large its score."""
+    hq, hkv, d, L, page = 4, 2, 16, 300, 8
+    scale = 1 / math.sqrt(d)
+    q = rand(1, hq, d, seed=60, dtype=dtype)
+    for standout in (L - window, L - window - 1):           # inside, outside
+        k = rand(L, hkv, d, seed=61, dtype=dtype, scale=0.1)
+        v = rand(L, hkv, d, seed=62, dtype=dtype)
+        if standout >= 0:
+            k[standout, 0] = (q[0, 0].float() * 8).to(dtype)
+            k[standout, 1] = (q[0, 2].float() * 8).to(dtype)
+        cache, ids = paged_cache(k, v, page, 63, dtype)
+        # pages that the window has passed are given back: the table holds -1 there
+        first_live = max(0, L - 1 - window + 1) // page
+        ids = ids.clone()
+        ids[:first_live] = -1
+        out = ops.attention(q.to(DEV), cache.to(DEV), torch.tensor([L - 1], dtype=torch.int32, device=DEV),
+                            torch.zeros(1, dtype=torch.int32, device=DEV), ids[None].to(DEV), scale, window=window)
+        want = P.attention(q.float(), k.float(), v.float(), scale, window=window)
+        close(out, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,d,page", [(4, 2, 16, 4), (6, 1, 32, 8), (6, 2, 48, 16), (16, 8, 128, 16), (2, 2, 80, 3)])
+def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, page):
+    T, pages, eps = 11, 9, 1e-5
+    width = (hq + 2 * hkv) * d
+    qkv = rand(T, width, seed=70, dtype=dtype)
+    qw, kw = 1 + rand(d, seed=71, scale=0.1), 1 + rand(d, seed=72, scale=0.1)
+    table = P.rope_table(10000.0, d, 64)
+    pos = torch.tensor([0, 1, 2, 3, 40, 41, 63, 7, 8, 9, 10], dtype=torch.int32)
+    slots = torch.tensor([5 * page + 0, 5 * page + 1, 2 * page + page - 1, 0, 1, 8 * page + page - 1,
+                          3 * page, 4 * page, -1, 6 * page, 7 * page], dtype=torch.int32)
+    if page == 1:
+        slots = torch.arange(T, dtype=torch.int32)
+    slots = torch.where(slots >= pages * page, torch.tensor(-1, dtype=torch.int32), slots)
+    cache = torch.zeros(pages, 2, hkv, page, d, dtype=dtype, device=DEV)
+    q_out = ops.qk_rope_store(qkv.to(DEV), hq, hkv, d, pos.to(DEV), qw.to(DEV), kw.to(DEV), eps,
+                              table.to(DEV), slots.to(DEV), cache, page)
+    x = qkv.float()
+    q = x[:, :hq * d].view(T, hq, d)
+    k = x[:, hq * d:(hq + hkv) * d].view(T, hkv, d)
+    v = x[:, (hq + hkv) * d:].view(T, hkv, d)
+    q_ref = P.apply_rope(table, pos, P.rms_norm(q, qw, eps))
+    k_ref = P.apply_rope(table, pos, P.rms_norm(k, kw, eps))
+    close(q_out, q_ref, dtype)
+    want = torch.zeros(pages, 2, hkv, page, d)
+    for t in range(T):
+        s = int(slots[t])
+        if s >= 0:
+            want[s // page, 0, :, s % page] = k_ref[t]
+            want[s // page, 1, :, s % page] = v[t]
+    close(cache, want, dtype)
+    assert torch.equal(cache[:, 1].float().cpu(), want[:, 1].to(dtype).float())      # values are copied exactly
+    # the steps apart: norm only into the packed form, then rotation and store from it
+    packed = ops.qk_rope_store(qkv.to(DEV), hq, hkv, d, None, qw.to(DEV), kw.to(DEV), eps, None, None, None,
+                               page, packed=True)
+    close(packed[:, :hq], P.rms_norm(q, qw, eps), dtype)
+    close(packed[:, hq:hq + hkv], P.rms_norm(k, kw, eps), dtype)
+    assert torch.equal(packed[:, hq + hkv:].cpu().float(), v.to(dtype).float())
+    no_norm = ops.qk_rope_store(qkv.to(DEV), hq, hkv, d, pos.to(DEV), None, None, 0.0, table.to(DEV), None, None, page)
+    close(no_norm, P.apply_rope(table, pos, q), dtype)
+
+
+def test_argmax_takes_the_lowest_index_on_ties(ops):
+    logits = rand(5, 50000, seed=80)
+    logits[0, 49999] = 9.0
+    logits[1, 0] = 9.0
+    logits[2, 777] = logits[2, 40001] = 9.0                  # a tie: the lower index wins
+    logits[3] = -3.0                                         # all equal
+    logits[4, 255] = logits[4, 256] = 9.0                    # a tie across two threads' strides
+    got = ops.argmax(logits.to(DEV)).cpu().tolist()
+    assert got == [49999, 0, 777, 0, 255]
+    assert got == P.greedy(logits)
+    odd = rand(3, 331, seed=81)
+    assert ops.argmax(odd.to(DEV)).cpu().tolist() == P.greedy(odd)
+
+
+def test_temperature_sampling_is_the_inverse_cdf(ops):
+    V = 331
+    logits = rand(64, V, seed=82, scale=2.0)
+    temps = torch.tensor([0.7, 1.0, 1.5, 0.2] * 16)
+    us = torch.rand(64, generator=torch.Generator().manual_seed(83))
+    us[0], us[1] = 0.0, 1.0 - 2.0 ** -24
+    got = ops.sample(logits.to(DEV), temps.to(DEV), us.to(DEV)).cpu().tolist()
+    cdf = torch.softmax(logits.double() / temps.double()[:, None], dim=-1).cumsum(-1)
+    for r, tok in enumerate(got):
+        lo = float(cdf[r, tok - 1]) if tok > 0 else 0.0
+        hi = float(cdf[r, tok])
+        assert lo - 1e-5 <= float(us[r]) <= hi + 1e-5, (r, tok, lo, float(us[r]), hi)
+    # a low temperature approaches greedy
+    cold = ops.sample(logits.to(DEV), torch.full((64,), 1e-3, device=DEV), us.to(DEV)).cpu().tolist()
+    assert cold == P.greedy(logits)
+    # frequencies follow the distribution
+    row = torch.tensor([[2.0, 1.0, 0.0, -1.0, 0.5]]).repeat(4000, 1)
+    u = torch.rand(4000, generator=torch.Generator().manual_seed(84))
+    draws = ops.sample(row.to(DEV), torch.ones(4000, device=DEV), u.to(DEV)).cpu()
+    freq = torch.bincount(draws, minlength=5).double() / 4000
+    assert (freq - torch.softmax(row[0].double(), -1)).abs().max() < 0.03
+
+
+def test_kernels_refuse_what_they_do_not_take(ops):
+    x = torch.zeros(4, 8, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.gemm(x, torch.zeros(3, 9, device=DEV))                       # inner sizes differ
+    with pytest.raises(ops.KernelError):
+        ops.gemm(x, torch.zeros(3, 8, device=DEV, dtype=torch.bfloat16))  # 32-bit activations, 16-bit weights
+    with pytest.raises(ops.KernelError):
+        ops.gemm(x.t(), torch.zeros(3, 4, device=DEV))                   # not contiguous
+    with pytest.raises(ops.KernelError):
+        ops.rmsnorm(x, torch.ones(7, device=DEV), 1e-6, torch.float32)
+    with pytest.raises(ops.KernelError):
+        ops.embedding(torch.zeros(3, dtype=torch.int64, device=DEV), x)  # ids must be int32
+    q = torch.zeros(1, 3, 16, device=DEV)
+    cache = torch.zeros(2, 2, 2, 4, 16, device=DEV)
+    i32 = lambda *v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.attention(q, cache, i32(0), i32(0), i32(0)[None], 1.0)       # 3 heads on 2 kv heads
+    big = torch.zeros(1, 2, 272, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.attention(big, torch.zeros(2, 2, 2, 4, 272, device=DEV), i32(0), i32(0), i32(0)[None], 1.0)
+    with pytest.raises(ops.KernelError):
+        ops.silu_mul(torch.zeros(2, 7, device=DEV))
