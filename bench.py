@@ -1,0 +1,188 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16] [--layers L]
+
+The default run has the layer sizes of Qwen3-0.6B (BASELINE.json configs[2]) with
+random weights, a batch of 8 requests and a context of 4096 tokens: every request is
+first prefilled with random tokens through the engine's own step function, so that
+the K timed decode steps end at that context.  A "step" is one decode step (one new
+token per request, through the cache, sampled greedily on the device).  One JSON
+line is printed:
+
+  value      decoded tokens a second at batch 8
+  prefill    one 2048-token prompt in one step: tokens a second, and flops / time / peak
+  roofline   the decode step's bytes (every weight once + the live requests' cache) / time / 8 TB/s
+  points     decoded tokens a second at batch 1 and at batch 64
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN3_0_6B = dict(
+    architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_size=1024, intermediate_size=3072,
+    num_hidden_layers=28, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
+    max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True)
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
+    ap.add_argument("--seed", type=int, default=0)
+    return ap.parse_args()
+
+
+def main() -> int:
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported (the engine has no multi-GPU path)")
+        return 2
+    import torch
+    import qwen_engine_amd  # noqa: F401
+    from qwen_engine_amd.config import Qwen3Config
+    from qwen_engine_amd.engine import ModelRunner, StepEntry
+    from qwen_engine_amd.kernels import ops
+    from qwen_engine_amd.parts import DecoderModel, Runtime
+    from qwen_engine_amd.weights import random_tensors
+
+    full_layers = QWEN3_0_6B["num_hidden_layers"]
+    layers = args.layers or full_layers
+    cfg = Qwen3Config.from_dict(dict(QWEN3_0_6B, num_hidden_layers=layers))
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    ops.load_library()
+
+    t0 = time.time()
+    model = DecoderModel(cfg.to_model_spec())
+    model.load(random_tensors(cfg, args.seed, dtype=torch.bfloat16), Runtime(dev, dtype))
+    print(f"[bench] random weights for {layers} layers in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+
+    P = args.block_size
+    itemsize = 2 if args.dtype == "bf16" else 4
+    H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    Hq, Hkv, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    layer_params = (Hq + 2 * Hkv) * D * H + Hq * D * H + 3 * H * I
+    weight_bytes = (layers * layer_params + V * H) * itemsize + (layers * (2 * H + 2 * D) + H) * 4
+    kv_bytes_per_token = layers * 2 * Hkv * D * itemsize
+    g = torch.Generator().manual_seed(args.seed + 1)
+
+    def decode_run(batch, context, steps, warmup):
+        """Prefill `batch` requests so that `warmup + steps` decode steps end at `context` tokens."""
+        pages = batch * ((context + P - 1) // P + 1)
+        runner = ModelRunner(model, page_size=P, num_pages=pages, max_requests=batch)
+        start = context - (warmup + steps)
+        ids = list(range(batch))
+        for r in ids:
+            runner.add_request(r)
+        last = None
+        chunk = 2048
+        for r in ids:
+            toks = torch.randint(0, V, (start,), generator=g).tolist()
+            for a in range(0, start, chunk):
+                part = toks[a:a + chunk]
+                want = [len(part) - 1] if a + chunk >= start else []
+                out = runner.step([StepEntry(r, part, want)])
+            last = out
+        tokens = torch.randint(0, V, (batch,), generator=g).tolist()
+
+        def one_step(tokens):
+            logits = runner.step([StepEntry(r, [tokens[i]], [0]) for i, r in enumerate(ids)])
+            return ops.argmax(logits).tolist()          # the host needs the tokens to go on: a sync per step
+
+        for _ in range(warmup):
+            tokens = one_step(tokens)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            tokens = one_step(tokens)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        for r in ids:
+            runner.free_request(r)
+        del runner
+        torch.cuda.empty_cache()
+        mean_ctx = context - steps / 2.0
+        step_bytes = weight_bytes + batch * mean_ctx * kv_bytes_per_token
+        return dict(tok_s=batch * steps / dt, ms=dt / steps * 1e3, gbs=step_bytes / (dt / steps) / 1e9)
+
+    def prefill_run(T, reps=3):
+        runner = ModelRunner(model, page_size=P, num_pages=(T + P - 1) // P + 1, max_requests=1)
+        toks = torch.randint(0, V, (T,), generator=g).tolist()
+        best = None
+        for _ in range(reps + 1):
+            runner.add_request("p")
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            logits = runner.step([StepEntry("p", toks, [T - 1])])
+            ops.argmax(logits).tolist()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            runner.free_request("p")
+            best = dt if best is None else min(best, dt)     # the first repetition warms up
+        flops = 2.0 * T * layers * layer_params + 2.0 * V * H \
+            + layers * 4.0 * Hq * D * T * (T + 1) / 2.0
+        del runner
+        torch.cuda.empty_cache()
+        return dict(value=T / best, tokens=T, ms=best * 1e3, frac=flops / best / PEAK_FLOPS[args.dtype])
+
+    main_run = decode_run(args.batch, args.context, args.steps, args.warmup)
+    print(f"[bench] decode batch {args.batch}: {main_run}", file=sys.stderr, flush=True)
+    prefill = prefill_run(args.prefill_tokens)
+    print(f"[bench] prefill: {prefill}", file=sys.stderr, flush=True)
+    points = {}
+    if not args.skip_points:
+        for b in (1, 64):
+            r = decode_run(b, args.context, max(8, args.steps // 2), max(2, args.warmup // 2))
+            points[f"decode_b{b}"] = round(r["tok_s"], 1)
+            print(f"[bench] decode batch {b}: {r}", file=sys.stderr, flush=True)
+
+    line = {
+        "metric": "decode tok/s @ batch 8 (Qwen3-0.6B sizes, context 4096)",
+        "value": round(main_run["tok_s"], 1),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_run["ms"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": args.dtype,
+        "data": "synthetic: random weights N(0, 0.02), uniform-random token ids",
+        "config": {
+            "model": "Qwen3-0.6B sizes (random weights)", "layers": layers, "layers_of_model": full_layers,
+            "hidden_size": H, "num_attention_heads": Hq, "num_key_value_heads": Hkv, "head_dim": D,
+            "intermediate_size": I, "vocab_size": V, "tie_word_embeddings": True,
+            "global_batch": args.batch, "seq_len": args.context, "page_size": P,
+            "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU",
+        },
+        "prefill": {"value": round(prefill["value"], 1), "tokens": prefill["tokens"],
+                    "ms": round(prefill["ms"], 3), "frac": round(prefill["frac"], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(main_run["gbs"], 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(main_run["gbs"] / HBM_PEAK_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
