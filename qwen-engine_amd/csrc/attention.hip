@@ -1,20 +1,50 @@
-// Entry point of attention over the paged cache: picks a kernel for the shape.
+// Entry points of attention over the paged cache.
+//
+// qe_attention          any sizes, float32 or bfloat16, one wave per (token, head); for all
+//                       tokens of the batch or for a list of them
+// qe_attention_decode_* bfloat16 MFMA kernel for tokens that are the single new token of their
+//                       request (see attention_decode.hip)
 #include "common.h"
 
 int qe_attention_generic(const void* q, void* out, const void* cache, const int* positions,
-                         const int* tok_seq, const int* block_table, int max_blocks, int T, int Hq,
-                         int Hkv, int D, int P, float scale, int window, int dt_a, hipStream_t stream);
+                         const int* tok_seq, const int* block_table, int max_blocks, const int* tokens,
+                         int T, int Hq, int Hkv, int D, int P, float scale, int window, int dt_a,
+                         hipStream_t stream);
+bool qe_attention_decode_ok(int Hq, int Hkv, int D, int P, int dt_a);
+size_t qe_attention_decode_workspace(int n_dec, int Hq, int D, int num_splits);
+int qe_attention_decode(const void* q, void* out, const void* cache, const int* dec_tokens, int n_dec,
+                        const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
+                        int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
+                        int split_keys, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
-// algo: 0 = choose, 1 = generic 32-bit kernel.
+// tokens: null for all T rows of q, else n_tokens row indices.
 extern "C" int qe_attention(const void* q, void* out, const void* cache, const int* positions,
-                            const int* tok_seq, const int* block_table, int max_blocks, int T,
-                            int Hq, int Hkv, int D, int P, float scale, int window, int dt_a, int algo,
+                            const int* tok_seq, const int* block_table, int max_blocks, const int* tokens,
+                            int n_tokens, int Hq, int Hkv, int D, int P, float scale, int window, int dt_a,
                             hipStream_t stream) {
-    QE_REQUIRE(T >= 0 && Hq > 0 && Hkv > 0 && D > 0 && P > 0 && max_blocks > 0, "attention: bad sizes");
+    QE_REQUIRE(n_tokens >= 0 && Hq > 0 && Hkv > 0 && D > 0 && P > 0 && max_blocks > 0, "attention: bad sizes");
     QE_REQUIRE(Hq % Hkv == 0, "attention: %d query heads are no multiple of %d key/value heads", Hq, Hkv);
     QE_REQUIRE(window >= 0, "attention: negative window");
-    QE_REQUIRE(algo == 0 || algo == 1, "attention: unknown algo %d", algo);
-    if (T == 0) return 0;
-    return qe_attention_generic(q, out, cache, positions, tok_seq, block_table, max_blocks, T, Hq, Hkv,
-                                D, P, scale, window, dt_a, stream);
+    if (n_tokens == 0) return 0;
+    return qe_attention_generic(q, out, cache, positions, tok_seq, block_table, max_blocks, tokens, n_tokens,
+                                Hq, Hkv, D, P, scale, window, dt_a, stream);
+}
+
+extern "C" int qe_attention_decode_supported(int Hq, int Hkv, int D, int P, int dt_a) {
+    return qe_attention_decode_ok(Hq, Hkv, D, P, dt_a) ? 1 : 0;
+}
+
+extern "C" long qe_attention_decode_workspace_bytes(int n_dec, int Hq, int D, int max_position, int split_keys) {
+    return (long)qe_attention_decode_workspace(n_dec, Hq, D, max_position / split_keys + 1);
+}
+
+extern "C" int qe_attention_decode_run(const void* q, void* out, const void* cache, const int* dec_tokens,
+                                       int n_dec, const int* positions, const int* tok_seq,
+                                       const int* block_table, int max_blocks, int Hq, int Hkv, int D, int P,
+                                       float scale, int window, int max_position, int split_keys,
+                                       void* workspace, long workspace_bytes, hipStream_t stream) {
+    QE_REQUIRE(Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && max_position >= 0, "decode attention: bad sizes");
+    return qe_attention_decode(q, out, cache, dec_tokens, n_dec, positions, tok_seq, block_table, max_blocks,
+                               Hq, Hkv, D, P, scale, window, max_position, split_keys, workspace,
+                               (size_t)workspace_bytes, stream);
 }

@@ -8,7 +8,8 @@
 // sums depends on p and the window only: not on how the request's tokens were cut
 // into steps, nor on what else is in the batch.
 //
-// cache of one layer: [page][2 (k, v)][Hkv][P][D].
+// cache of one layer: [page][2 (k, v)][Hkv][P * D]; a key tile is [P][D], a value tile is
+// stored transposed, [D][P] (the layout the MFMA kernels read without a shuffle).
 #include "common.h"
 
 #define ATTN_MAX_D 256
@@ -17,13 +18,13 @@ template <typename TA>
 __global__ __launch_bounds__(64) void attention_generic_kernel(
     const TA* __restrict__ q, TA* __restrict__ out, const TA* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ tok_seq,
-    const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tokens,
     int Hq, int Hkv, int D, int P, float scale, int window) {
     extern __shared__ float smem[];
     float* qs = smem;            // D
     float* ps = smem + D;        // 64 probabilities of the current chunk
     long* voff = (long*)(smem + ((D + 64 + 1) & ~1));  // 64 offsets of the chunk's value rows
-    const long t = blockIdx.x;
+    const long t = tokens ? tokens[blockIdx.x] : blockIdx.x;   // a subset of the batch, or all of it
     const int h = blockIdx.y;
     const int lane = threadIdx.x;
     const int kvh = h / (Hq / Hkv);
@@ -49,7 +50,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
             const long page = bt[j / P];
             const int off = j % P;
             const long kbase = page * page_stride + ((long)kvh * P + off) * D;
-            vo = kbase + (long)Hkv * P * D;
+            vo = page * page_stride + ((long)(Hkv + kvh) * P) * D + off;   // + d * P
             const TA* krow = cache + kbase;
             float dot = 0.f;
             for (int d = 0; d < D; ++d) dot = fmaf(qs[d], Elem<TA>::load(krow + d), dot);
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
             if (d < D) {
                 float a = acc[i] * alpha;
                 for (int jj = 0; jj < cnt; ++jj)
-                    a = fmaf(ps[jj], Elem<TA>::load(cache + voff[jj] + d), a);
+                    a = fmaf(ps[jj], Elem<TA>::load(cache + voff[jj] + (long)d * P), a);
                 acc[i] = a;
             }
         }
@@ -86,8 +87,9 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
 }
 
 int qe_attention_generic(const void* q, void* out, const void* cache, const int* positions,
-                         const int* tok_seq, const int* block_table, int max_blocks, int T, int Hq,
-                         int Hkv, int D, int P, float scale, int window, int dt_a, hipStream_t stream) {
+                         const int* tok_seq, const int* block_table, int max_blocks, const int* tokens,
+                         int T, int Hq, int Hkv, int D, int P, float scale, int window, int dt_a,
+                         hipStream_t stream) {
     QE_REQUIRE(D <= ATTN_MAX_D, "attention: head_dim=%d exceeds %d", D, ATTN_MAX_D);
     QE_REQUIRE(Hq <= 65535, "attention: too many heads");
     dim3 grid(T, Hq);
@@ -95,11 +97,11 @@ int qe_attention_generic(const void* q, void* out, const void* cache, const int*
     if (dt_a == QE_F32)
         attention_generic_kernel<float><<<grid, 64, shmem, stream>>>(
             (const float*)q, (float*)out, (const float*)cache, positions, tok_seq, block_table,
-            max_blocks, Hq, Hkv, D, P, scale, window);
+            max_blocks, tokens, Hq, Hkv, D, P, scale, window);
     else if (dt_a == QE_BF16)
         attention_generic_kernel<bf16_t><<<grid, 64, shmem, stream>>>(
             (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions, tok_seq, block_table,
-            max_blocks, Hq, Hkv, D, P, scale, window);
+            max_blocks, tokens, Hq, Hkv, D, P, scale, window);
     else
         QE_REQUIRE(false, "attention: unknown dtype %d", dt_a);
     QE_LAUNCH_CHECK();

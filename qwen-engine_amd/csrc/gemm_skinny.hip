@@ -1,0 +1,139 @@
+// Matrix product for few rows of activations (decode): out[M, N] = x[M, K] . W[N, K]^T, M <= 64,
+// bfloat16 in, 32-bit accumulation on the MFMA units.  The weights are streamed from HBM
+// exactly once; this kernel is bound by that stream.
+//
+// A block of 4 waves owns 16 rows of W.  The rows are the M side of v_mfma_f32_16x16x32_bf16
+// (lane (g, r), g = lane / 16, r = lane % 16, holds W[n0 + r][c * 32 + g * 8 .. + 8]: one 16-byte
+// load), the tokens are the N side (lane (g, r) holds x[j * 16 + r][the same k]).  Wave w takes
+// the 32-wide chunks c = w, w + 4, ... of K, so the four waves read neighbouring 64-byte pieces
+// of the same rows at the same time; their partial tiles are summed through shared memory.
+// The result tile has, per lane, 4 consecutive n for one token: one 8- or 16-byte store.
+//
+// Epilogues: store (+ bias); add into a 32-bit residual stream; silu(gate) * up, where W holds
+// the gate rows followed by the up rows and a block owns 16 of each.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2 };
+
+template <int MT, int EPI, typename TO>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
+    TO* __restrict__ out, int M, int N, int K) {
+    constexpr int NW = (EPI == EPI_SILU_MUL) ? 2 : 1;   // weight tiles per block
+    __shared__ float red[4][NW][MT][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 4, r = lane & 15;
+    const int n0 = blockIdx.x * 16;
+    const int nchunks = K / 32;
+
+    floatx4 acc[NW][MT];
+#pragma unroll
+    for (int a = 0; a < NW; ++a)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) acc[a][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const bool row_ok = n0 + r < N;
+    const bf16_t* wrow0 = w + (long)(row_ok ? n0 + r : 0) * K + g * 8;
+    const bf16_t* wrow1 = (EPI == EPI_SILU_MUL) ? wrow0 + (long)N * K : wrow0;
+    const bf16_t* xrow[MT];
+    bool tok_ok[MT];
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+        tok_ok[j] = j * 16 + r < M;
+        xrow[j] = x + (long)(tok_ok[j] ? j * 16 + r : 0) * K + g * 8;
+    }
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    for (int c = wave; c < nchunks; c += 4) {
+        bf16x8 a0 = row_ok ? *(const bf16x8*)(wrow0 + c * 32) : zero;
+        bf16x8 a1 = zero;
+        if (EPI == EPI_SILU_MUL) a1 = row_ok ? *(const bf16x8*)(wrow1 + c * 32) : zero;
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            const bf16x8 b = tok_ok[j] ? *(const bf16x8*)(xrow[j] + c * 32) : zero;
+            acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b, acc[0][j], 0, 0, 0);
+            if (EPI == EPI_SILU_MUL)
+                acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b, acc[1][j], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < NW; ++a)
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave][a][j][lane][i] = acc[a][j][i];
+    __syncthreads();
+    // wave w finishes the token tiles j = w, w + 4, ...
+    for (int j = wave; j < MT; j += 4) {
+        float v[NW][4];
+#pragma unroll
+        for (int a = 0; a < NW; ++a)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                v[a][i] = red[0][a][j][lane][i] + red[1][a][j][lane][i] + red[2][a][j][lane][i] + red[3][a][j][lane][i];
+        const int t = j * 16 + r;          // lane (g, r): token t, rows n0 + g * 4 + i
+        if (t >= M) continue;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + g * 4 + i;
+            if (n >= N) continue;
+            float y = v[0][i];
+            if (EPI == EPI_SILU_MUL) {
+                y = y / (1.f + __expf(-y)) * v[1][i];
+            } else if (bias) {
+                y += bias[n];
+            }
+            TO* o = out + (long)t * N + n;
+            if (EPI == EPI_RESIDUAL) {
+                *(float*)o = *(const float*)o + y;
+            } else {
+                Elem<TO>::store(o, y);
+            }
+        }
+    }
+}
+
+template <int EPI, typename TO>
+static int launch_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
+                         hipStream_t stream) {
+    const int blocks = qe_cdiv(N, 16);
+    const int mt = qe_cdiv(M, 16);
+#define QE_SKINNY(MT_)                                                                            \
+    gemm_skinny_kernel<MT_, EPI, TO><<<blocks, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, \
+                                                                 (TO*)out, M, N, K)
+    switch (mt) {
+        case 1: QE_SKINNY(1); break;
+        case 2: QE_SKINNY(2); break;
+        case 3: QE_SKINNY(3); break;
+        default: QE_SKINNY(4); break;
+    }
+#undef QE_SKINNY
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+bool qe_gemm_skinny_ok(int M, int N, int K, int dt_a, int dt_w) {
+    return dt_a == QE_BF16 && dt_w == QE_BF16 && M >= 1 && M <= 64 && K % 32 == 0 && K >= 32;
+}
+
+// epilogue EPI_STORE: out [M, N] in dt_o.  EPI_RESIDUAL: out is the 32-bit stream [M, N], added to.
+// EPI_SILU_MUL: w is [2 N, K] (gate rows, then up rows), out [M, N] in dt_o.
+int qe_gemm_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
+                   int dt_o, int epilogue, hipStream_t stream) {
+    QE_REQUIRE(M >= 1 && M <= 64 && K % 32 == 0, "skinny gemm: M=%d K=%d not taken", M, K);
+    if (epilogue == EPI_RESIDUAL) {
+        QE_REQUIRE(dt_o == QE_F32, "skinny gemm: the residual stream is 32-bit");
+        return launch_skinny<EPI_RESIDUAL, float>(x, w, bias, out, M, N, K, stream);
+    }
+    if (epilogue == EPI_SILU_MUL) {
+        QE_REQUIRE(!bias, "skinny gemm: silu-mul takes no bias");
+        if (dt_o == QE_BF16) return launch_skinny<EPI_SILU_MUL, bf16_t>(x, w, bias, out, M, N, K, stream);
+        return launch_skinny<EPI_SILU_MUL, float>(x, w, bias, out, M, N, K, stream);
+    }
+    QE_REQUIRE(epilogue == EPI_STORE, "skinny gemm: unknown epilogue %d", epilogue);
+    if (dt_o == QE_BF16) return launch_skinny<EPI_STORE, bf16_t>(x, w, bias, out, M, N, K, stream);
+    return launch_skinny<EPI_STORE, float>(x, w, bias, out, M, N, K, stream);
+}

@@ -3,7 +3,8 @@
 //
 //   qkv   [T, (Hq + 2 Hkv) D]   row = q heads, k heads, v heads
 //   q_out [T, Hq, D]            normalised and rotated queries
-//   cache of one layer: [page][2 (k, v)][Hkv][P][D];  slot[t] = page * P + offset, < 0: no write
+//   cache of one layer: [page][2 (k, v)][Hkv][P * D]: key tiles [P][D], value tiles transposed [D][P];
+//   slot[t] = page * P + offset, < 0: no write
 //
 // With packed_out [T, Hq + 2 Hkv, D] every head is written there instead (q and k
 // after norm and rotation, v as it is) and neither q_out nor the cache is touched.
@@ -41,9 +42,15 @@ __global__ __launch_bounds__(64) void qk_rope_store_kernel(
         if (s < 0) return;
         const int kh = is_k ? head - Hq : head - Hq - Hkv;
         const long page = s / P, off = s % P;
-        dst = cache + page * (2L * Hkv * P * D) + (((is_k ? 0L : 1L) * Hkv + kh) * P + off) * D;
+        if (is_k) {
+            dst = cache + page * (2L * Hkv * P * D) + ((long)kh * P + off) * D;
+        } else {   // value tile is [D][P]
+            TA* vt = cache + page * (2L * Hkv * P * D) + ((long)(Hkv + kh) * P) * D + off;
+            for (int d = lane; d < D; d += 64) vt[(long)d * P] = src[d];
+            return;
+        }
     }
-    if (is_v) {
+    if (is_v) {   // packed form
         for (int d = lane; d < D; d += 64) dst[d] = src[d];
         return;
     }

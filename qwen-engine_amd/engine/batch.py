@@ -35,3 +35,7 @@ class StepContext:
     logit_rows: torch.Tensor           # int32 [R] rows whose logits are wanted
     state_slots: torch.Tensor          # int32 [B]
     max_position: int = 0              # largest position in the batch (host)
+    # rows that are the single new token of their request, and all other rows (None: not split)
+    dec_tokens: Optional[torch.Tensor] = None
+    other_tokens: Optional[torch.Tensor] = None
+    max_dec_position: int = 0

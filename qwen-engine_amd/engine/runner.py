@@ -163,7 +163,10 @@ class ModelRunner:
             tables.append([row + [-1] * (width - len(row)) for row in tab])
 
         # one host buffer, one copy to the device
-        parts = [token_ids, positions, tok_seq, rows, [s.state_slot for s in seqs]]
+        dec_rows = [s.q_start for s in seqs if s.q_len == 1]
+        other_rows = [s.q_start + i for s in seqs if s.q_len > 1 for i in range(s.q_len)]
+        max_dec = max([s.kv_before for s in seqs if s.q_len == 1], default=0)
+        parts = [token_ids, positions, tok_seq, rows, [s.state_slot for s in seqs], dec_rows, other_rows]
         for g in range(n_groups):
             parts.append(slots[g])
             parts.append([p for row in tables[g] for p in row])
@@ -180,6 +183,7 @@ class ModelRunner:
 
         d_tok, d_pos, d_seq = take(T), take(T), take(T)
         d_rows, d_state = take(len(rows)), take(B)
+        d_dec, d_other = take(len(dec_rows)), take(len(other_rows))
         d_slots, d_tables = [], []
         for g in range(n_groups):
             d_slots.append(take(T))
@@ -187,7 +191,8 @@ class ModelRunner:
             d_tables.append(take(B * width, (B, width)))
         return StepContext(rt=self.rt, page_size=P, num_tokens=T, seqs=seqs, token_ids=d_tok,
                            positions=d_pos, tok_seq=d_seq, block_tables=d_tables, slots=d_slots,
-                           logit_rows=d_rows, state_slots=d_state, max_position=max(positions))
+                           logit_rows=d_rows, state_slots=d_state, max_position=max(positions),
+                           dec_tokens=d_dec, other_tokens=d_other, max_dec_position=max_dec)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Runs the entries' tokens as one batch; returns float32 logits [wanted, vocab] on the

@@ -17,7 +17,9 @@ from . import build as _build
 F32, BF16 = 0, 1
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
 
-ALGO_AUTO, ALGO_GENERIC = 0, 1
+ALGO_AUTO, ALGO_GENERIC, ALGO_FAST = 0, 1, 2
+EPI_STORE, EPI_RESIDUAL, EPI_SILU_MUL = 0, 1, 2
+DECODE_SPLIT_KEYS = 128   # keys per split of the decode attention kernel
 
 
 class KernelError(RuntimeError):
@@ -43,9 +45,12 @@ def load_library():
         "qe_rmsnorm": [vp, vp, vp, vp, vp, i32, i32, f32, i32, vp],
         "qe_residual_add": [vp, vp, i64, i32, vp],
         "qe_silu_mul": [vp, vp, i32, i32, i32, vp],
-        "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp],
+        "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp],
+        "qe_gemm_fused_supported": [i32, i32, i32, i32, i32],
+        "qe_attention_decode_supported": [i32, i32, i32, i32, i32],
+        "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
         "qe_qk_rope_store": [vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
-        "qe_attention": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp],
+        "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
         "qe_argmax": [vp, vp, i32, i32, vp],
         "qe_sample": [vp, vp, vp, vp, i32, i32, vp],
     }
@@ -53,6 +58,8 @@ def load_library():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = ctypes.c_int
+    lib.qe_attention_decode_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]
+    lib.qe_attention_decode_workspace_bytes.restype = ctypes.c_long
     _lib = lib
     return lib
 
@@ -162,25 +169,43 @@ def silu_mul(gu: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tens
     return out
 
 
+def gemm_fused_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """True if gemm can add into the residual stream or apply silu-mul itself for these operands."""
+    lib = load_library()
+    return bool(lib.qe_gemm_fused_supported(x.shape[0], w.shape[0], x.shape[1], _DT[x.dtype], _DT[w.dtype]))
+
+
 def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
          out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
-         algo: int = ALGO_AUTO) -> torch.Tensor:
-    """x [M, K] . w [N, K]^T (+ bias [N], 32-bit) -> [M, N] in out_dtype (default: x's)."""
+         algo: int = ALGO_AUTO, epilogue: int = EPI_STORE) -> torch.Tensor:
+    """x [M, K] . w [N, K]^T (+ bias [N], 32-bit) -> [M, N] in out_dtype (default: x's).
+
+    epilogue EPI_RESIDUAL: the product is added into ``out``, the 32-bit stream [M, N].
+    epilogue EPI_SILU_MUL: w is [2 N, K] (gate rows, then up rows); the result is
+    silu(x . gate^T) * (x . up^T), [M, N].  Both need gemm_fused_supported(x, w)."""
     lib = load_library()
     _need(x, "x", _ACT, (None, None))
     M, K = x.shape
     _need(w, "w", _ACT, (None, K), x.device)
     N = w.shape[0]
+    if epilogue == EPI_SILU_MUL:
+        if N % 2:
+            raise KernelError("gemm: gate|up weights have an odd number of rows")
+        N //= 2
     if x.dtype == torch.float32 and w.dtype != torch.float32:
         raise KernelError("gemm: 32-bit activations need 32-bit weights")
     if bias is not None:
         _need(bias, "bias", torch.float32, (N,), x.device)
+    if epilogue == EPI_RESIDUAL:
+        if out is None:
+            raise KernelError("gemm: the residual epilogue needs the stream to add into")
+        out_dtype = torch.float32
     out_dtype = out_dtype or x.dtype
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     _need(out, "out", out_dtype, (M, N), x.device)
     _check(lib.qe_gemm(x.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), M, N, K,
-                       _DT[x.dtype], _DT[w.dtype], _DT[out_dtype], algo, _stream()), "gemm")
+                       _DT[x.dtype], _DT[w.dtype], _DT[out_dtype], algo, epilogue, _stream()), "gemm")
     return out
 
 
@@ -232,13 +257,27 @@ def qk_rope_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     return packed_out if packed else q_out
 
 
+def attention_decode_supported(q: torch.Tensor, cache: torch.Tensor) -> bool:
+    """True if the MFMA decode kernel takes these sizes (bfloat16, head size 64 or 128, pages of a
+    multiple of 16 tokens, at most 16 query heads per key/value head)."""
+    lib = load_library()
+    return bool(lib.qe_attention_decode_supported(q.shape[1], cache.shape[2], q.shape[2], cache.shape[3],
+                                                  _DT[q.dtype]))
+
+
 def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
               block_table: torch.Tensor, scale: float, window: int = 0,
-              out: Optional[torch.Tensor] = None, algo: int = ALGO_AUTO) -> torch.Tensor:
-    """q [T, Hq, D]; cache [pages, 2, Hkv, P, D]; positions, tok_seq int32 [T];
-    block_table int32 [B, max_blocks].  Token t sees the keys at positions
-    max(0, p - window + 1) .. p of request tok_seq[t] (window 0: all).  The caller
-    guarantees that those positions have pages in the table."""
+              out: Optional[torch.Tensor] = None, algo: int = ALGO_AUTO,
+              dec_tokens: Optional[torch.Tensor] = None, max_dec_position: int = 0,
+              other_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q [T, Hq, D]; cache [pages, 2, Hkv, P, D] (key tiles [P][D], value tiles transposed [D][P]);
+    positions, tok_seq int32 [T]; block_table int32 [B, max_blocks].  Token t sees the keys at
+    positions max(0, p - window + 1) .. p of request tok_seq[t] (window 0: all).  The caller
+    guarantees that those positions have pages in the table.
+
+    dec_tokens (int32 rows of q that are the single new token of their request, the largest of
+    their positions being max_dec_position) go to the decode kernel where it takes the sizes;
+    other_tokens are the remaining rows.  Without the two lists every row is treated alike."""
     lib = load_library()
     _need(q, "q", _ACT, (None, None, None))
     T, Hq, D = q.shape
@@ -251,10 +290,36 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
     if out is None:
         out = torch.empty_like(q)
     _need(out, "out", q.dtype, (T, Hq, D), dev)
-    _check(lib.qe_attention(q.data_ptr(), out.data_ptr(), cache.data_ptr(), positions.data_ptr(),
-                            tok_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, Hq,
-                            Hkv, D, P, float(scale), int(window), _DT[q.dtype], algo, _stream()),
-           "attention")
+    if Hq % Hkv:
+        raise KernelError(f"attention: {Hq} query heads are no multiple of {Hkv} key/value heads")
+    max_blocks = block_table.shape[1]
+
+    def generic(tokens):
+        n = T if tokens is None else tokens.shape[0]
+        _check(lib.qe_attention(q.data_ptr(), out.data_ptr(), cache.data_ptr(), positions.data_ptr(),
+                                tok_seq.data_ptr(), block_table.data_ptr(), max_blocks, _ptr(tokens), n,
+                                Hq, Hkv, D, P, float(scale), int(window), _DT[q.dtype], _stream()), "attention")
+
+    if dec_tokens is None and other_tokens is None:
+        generic(None)
+        return out
+    if dec_tokens is not None and dec_tokens.shape[0]:
+        _need(dec_tokens, "dec_tokens", torch.int32, (None,), dev)
+        n_dec = dec_tokens.shape[0]
+        if algo != ALGO_GENERIC and attention_decode_supported(q, cache):
+            nbytes = lib.qe_attention_decode_workspace_bytes(n_dec, Hq, D, int(max_dec_position), DECODE_SPLIT_KEYS)
+            ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+            _check(lib.qe_attention_decode_run(q.data_ptr(), out.data_ptr(), cache.data_ptr(),
+                                               dec_tokens.data_ptr(), n_dec, positions.data_ptr(),
+                                               tok_seq.data_ptr(), block_table.data_ptr(), max_blocks, Hq, Hkv,
+                                               D, P, float(scale), int(window), int(max_dec_position),
+                                               DECODE_SPLIT_KEYS, ws.data_ptr(), nbytes, _stream()),
+                   "attention (decode)")
+        else:
+            generic(dec_tokens)
+    if other_tokens is not None and other_tokens.shape[0]:
+        _need(other_tokens, "other_tokens", torch.int32, (None,), dev)
+        generic(other_tokens)
     return out
 
 

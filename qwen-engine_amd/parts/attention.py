@@ -75,7 +75,10 @@ class PagedAttention:
             self.position.load({}, rt)
 
     # ---- one step -------------------------------------------------------------------
-    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding) -> torch.Tensor:
+    fuses_residual = True   # forward may add its output into the 32-bit stream itself
+
+    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding, residual: Optional[torch.Tensor] = None):
+        """Returns the mixer's output, or None after adding it into ``residual``."""
         if binding.kv is None:
             raise RuntimeError("attention was given no cache")
         T = x.shape[0]
@@ -100,8 +103,14 @@ class PagedAttention:
             pos.apply(packed, ctx.positions, self.hq, self.hkv)
             q = ops.qk_rope_store(packed.view(T, -1), self.hq, self.hkv, self.d, None, None, None, 0.0,
                                   None, slots, cache, ctx.page_size)
-        o = ops.attention(q, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g], self.scale, self.window)
-        return ops.gemm(o.view(T, self.hq * self.d), self.w_o)
+        o = ops.attention(q, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g], self.scale, self.window,
+                          dec_tokens=ctx.dec_tokens, max_dec_position=ctx.max_dec_position,
+                          other_tokens=ctx.other_tokens)
+        o = o.view(T, self.hq * self.d)
+        if residual is not None and ops.gemm_fused_supported(o, self.w_o):
+            ops.gemm(o, self.w_o, out=residual, epilogue=ops.EPI_RESIDUAL)
+            return None
+        return ops.gemm(o, self.w_o)
 
 
 register_part("paged_attention", PagedAttention)

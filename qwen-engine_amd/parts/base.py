@@ -7,6 +7,8 @@ Norm          forward(h, rt, delta=None, rows=None) -> x
 Mixer         forward(x, ctx, binding) -> y      x, y [T, H] in the activation type
               cache_need(spec) -> KVNeed | None, state_need(spec, hidden) -> StateNeed | None
 FeedForward   forward(x, ctx) -> y
+              A mixer or feed-forward with the class attribute ``fuses_residual = True`` is also
+              given ``residual=h`` and may add its output into h itself and return None.
 Position      table() for the fused kernel, or apply(packed, positions, num_q, num_k) in place
               on a [T, Hq + 2 Hkv, D] tensor of q | k | v heads.
 """

@@ -4,7 +4,7 @@ with the product formed in 32-bit before the one rounding).  gate and up are one
 product with the two weights stacked."""
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 
@@ -35,9 +35,17 @@ class SwiGLU:
         self.w_gu = rt.place_matrix(torch.cat([g, u], dim=0))
         self.w_down = rt.place_matrix(tensors["down_proj.weight"])
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        gu = ops.gemm(x, self.w_gu)
-        a = ops.silu_mul(gu)
+    fuses_residual = True   # forward may add its output into the 32-bit stream itself
+
+    def forward(self, x: torch.Tensor, ctx, residual: Optional[torch.Tensor] = None):
+        """Returns the feed-forward output, or None after adding it into ``residual``."""
+        if ops.gemm_fused_supported(x, self.w_gu):
+            a = ops.gemm(x, self.w_gu, epilogue=ops.EPI_SILU_MUL)   # silu.mul in the product's epilogue
+        else:
+            a = ops.silu_mul(ops.gemm(x, self.w_gu))
+        if residual is not None and ops.gemm_fused_supported(a, self.w_down):
+            ops.gemm(a, self.w_down, out=residual, epilogue=ops.EPI_RESIDUAL)
+            return None
         return ops.gemm(a, self.w_down)
 
 

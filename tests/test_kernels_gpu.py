@@ -106,15 +106,17 @@ def test_silu_mul(ops, dtype):
 
 
 def paged_cache(k, v, page, perm_seed, dtype, extra_pages=3):
-    """k, v [L, Hkv, D] -> (cache [pages, 2, Hkv, P, D], block table row) with shuffled pages."""
+    """k, v [L, Hkv, D] -> (cache [pages, 2, Hkv, P, D], block table row) with shuffled pages.
+    A key tile is [P][D]; a value tile is stored transposed, [D][P]."""
     L, hkv, d = k.shape
     n = (L + page - 1) // page
     g = torch.Generator().manual_seed(perm_seed)
     ids = torch.randperm(n + extra_pages, generator=g)[:n]
     cache = torch.full((n + extra_pages, 2, hkv, page, d), float("nan")).to(dtype)
+    vt = cache[:, 1].view(-1, hkv, d, page)               # the same memory, seen as [D][P] tiles
     for pos in range(L):
         cache[ids[pos // page], 0, :, pos % page] = k[pos]
-        cache[ids[pos // page], 1, :, pos % page] = v[pos]
+        vt[ids[pos // page], :, :, pos % page] = v[pos]
     return cache, ids.to(torch.int32)
 
 
@@ -222,11 +224,12 @@ def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, page):
     k_ref = P.apply_rope(table, pos, P.rms_norm(k, kw, eps))
     close(q_out, q_ref, dtype)
     want = torch.zeros(pages, 2, hkv, page, d)
+    want_vt = want[:, 1].view(pages, hkv, d, page)         # value tiles are [D][P]
     for t in range(T):
         s = int(slots[t])
         if s >= 0:
             want[s // page, 0, :, s % page] = k_ref[t]
-            want[s // page, 1, :, s % page] = v[t]
+            want_vt[s // page, :, :, s % page] = v[t]
     close(cache, want, dtype)
     assert torch.equal(cache[:, 1].float().cpu(), want[:, 1].to(dtype).float())      # values are copied exactly
     # the steps apart: norm only into the packed form, then rotation and store from it
@@ -298,3 +301,103 @@ def test_kernels_refuse_what_they_do_not_take(ops):
         ops.attention(big, torch.zeros(2, 2, 2, 4, 272, device=DEV), i32(0), i32(0), i32(0)[None], 1.0)
     with pytest.raises(ops.KernelError):
         ops.silu_mul(torch.zeros(2, 7, device=DEV))
+
+
+# ---- the MFMA kernels of the bfloat16 mode -------------------------------------------------------
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(64, 64), (500, 96), (331, 160), (4096, 1024), (1024, 3072)])
+def test_gemm_for_few_rows(ops, M, N, K):
+    bf = torch.bfloat16
+    x, w = rand(M, K, seed=90, dtype=bf), rand(N, K, seed=91, dtype=bf, scale=0.1)
+    bias = rand(N, seed=92)
+    assert ops.gemm_fused_supported(x.to(DEV), w.to(DEV))
+    want = P.linear(x.double(), w.double())
+    for dt_o in (bf, torch.float32):
+        got = ops.gemm(x.to(DEV), w.to(DEV), out_dtype=dt_o, algo=ops.ALGO_FAST)
+        close(got, want, dt_o if dt_o == bf else torch.float32, scale=float(want.abs().max()))
+    close(ops.gemm(x.to(DEV), w.to(DEV), bias.to(DEV), algo=ops.ALGO_FAST), want + bias.double(), bf)
+    # added into the 32-bit stream
+    h = rand(M, N, seed=93)
+    hd = h.to(DEV)
+    ops.gemm(x.to(DEV), w.to(DEV), out=hd, epilogue=ops.EPI_RESIDUAL)
+    close(hd, h.double() + want, torch.float32, scale=float(want.abs().max()))
+
+
+@pytest.mark.parametrize("M", [1, 8, 40, 64])
+@pytest.mark.parametrize("I,K", [(160, 96), (112, 64), (3072, 1024)])
+def test_gemm_with_silu_mul(ops, M, I, K):
+    bf = torch.bfloat16
+    x, w = rand(M, K, seed=94, dtype=bf), rand(2 * I, K, seed=95, dtype=bf, scale=0.2)
+    got = ops.gemm(x.to(DEV), w.to(DEV), epilogue=ops.EPI_SILU_MUL)
+    gu = P.linear(x.double(), w.double())
+    close(got, P.silu_mul(gu[:, :I], gu[:, I:]), bf)
+
+
+def test_gemm_for_few_rows_refuses_other_shapes(ops):
+    bf = torch.bfloat16
+    x = torch.zeros(4, 80, dtype=bf, device=DEV)             # K = 80 is no multiple of 32
+    w = torch.zeros(16, 80, dtype=bf, device=DEV)
+    assert not ops.gemm_fused_supported(x, w)
+    with pytest.raises(ops.KernelError):
+        ops.gemm(x, w, algo=ops.ALGO_FAST)
+    ops.gemm(x, w)                                           # the generic kernel takes it
+    big = torch.zeros(65, 64, dtype=bf, device=DEV)
+    assert not ops.gemm_fused_supported(big, torch.zeros(16, 64, dtype=bf, device=DEV))
+    f = torch.zeros(4, 64, device=DEV)
+    assert not ops.gemm_fused_supported(f, torch.zeros(16, 64, device=DEV))
+
+
+@pytest.mark.parametrize("hq,hkv,d,page", [(16, 8, 128, 16), (8, 8, 64, 16), (32, 4, 128, 32), (16, 1, 64, 64), (6, 2, 128, 16)])
+@pytest.mark.parametrize("window", [0, 200])
+def test_decode_attention_kernel(ops, hq, hkv, d, page, window):
+    """Five requests with one new token each, at positions that end inside a tile, at a tile's and at
+    a split's edge; pages shuffled, unwritten parts of pages hold NaN."""
+    bf = torch.bfloat16
+    scale = 1 / math.sqrt(d)
+    positions = [0, 15, 16, 127, 128, 700]
+    qs, tables, caches, want = [], [], [], []
+    base = 0
+    for b, p in enumerate(positions):
+        L = p + 1
+        k, v = rand(L, hkv, d, seed=100 + b, dtype=bf), rand(L, hkv, d, seed=200 + b, dtype=bf)
+        q = rand(1, hq, d, seed=300 + b, dtype=bf)
+        cache, ids = paged_cache(k, v, page, 400 + b, bf)
+        tables.append(ids + base)
+        base += cache.shape[0]
+        caches.append(cache)
+        qs.append(q)
+        want.append(P.attention(q.float(), k.float(), v.float(), scale, window=window or None))
+    width = max(len(t) for t in tables)
+    table = torch.full((len(positions), width), -1, dtype=torch.int32)
+    for b, t in enumerate(tables):
+        table[b, :len(t)] = t
+    B = len(positions)
+    qd, cd = torch.cat(qs).to(DEV), torch.cat(caches).to(DEV)
+    assert ops.attention_decode_supported(qd, cd)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    out = ops.attention(qd, cd, i32(positions), i32(list(range(B))), table.to(DEV), scale, window=window,
+                        dec_tokens=i32(list(range(B))), max_dec_position=max(positions))
+    assert not torch.isnan(out.float()).any()
+    close(out, torch.cat(want), bf)
+    # a subset through the decode kernel, the rest through the generic one: every row is written once
+    out2 = ops.attention(qd, cd, i32(positions), i32(list(range(B))), table.to(DEV), scale, window=window,
+                         dec_tokens=i32([5, 1, 3]), max_dec_position=700, other_tokens=i32([0, 2, 4]))
+    close(out2, torch.cat(want), bf)
+
+
+@pytest.mark.parametrize("key_pos", [0, 15, 16, 127, 128, 255, 256, 1000, 1023])
+def test_decode_kernel_one_far_key_decides(ops, key_pos):
+    bf = torch.bfloat16
+    hq, hkv, d, L, page = 4, 2, 128, 1024, 16
+    k = rand(L, hkv, d, seed=500, dtype=bf, scale=0.1)
+    v = rand(L, hkv, d, seed=501, dtype=bf)
+    q = rand(1, hq, d, seed=502, dtype=bf)
+    k[key_pos, 0] = (q[0, 1].float() * 4).to(bf)            # head 1 of group 0, head 3 of group 1
+    k[key_pos, 1] = (q[0, 3].float() * 4).to(bf)
+    cache, ids = paged_cache(k, v, page, 503, bf)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    out = ops.attention(q.to(DEV), cache.to(DEV), i32([L - 1]), i32([0]), ids[None].to(DEV), 1 / math.sqrt(d),
+                        dec_tokens=i32([0]), max_dec_position=L - 1)
+    want = P.attention(q.float(), k.float(), v.float(), 1 / math.sqrt(d))
+    close(out, want, bf)
+    assert float((want[0, 1] - v[key_pos, 0].float()).abs().max()) < 0.05
