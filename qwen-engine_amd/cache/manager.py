@@ -132,6 +132,7 @@ class RequestCache:
     hashes: List[int] = field(default_factory=list)   # chain hashes of the full pages so far
     shared_len: int = 0                # tokens taken over from other requests at admission
     new_request: bool = True           # no step has run yet: fixed-size state must be cleared
+    dirty: List[List[int]] = field(default_factory=list)   # per group: table indices changed since taken
 
 
 @dataclass
@@ -169,7 +170,8 @@ class CacheManager:
         if req_id in self.requests:
             raise CacheError(f"request {req_id!r} is live already")
         slot = self.slots.take(req_id)
-        rc = RequestCache(req_id=req_id, state_slot=slot, tables=[[] for _ in self.groups])
+        rc = RequestCache(req_id=req_id, state_slot=slot, tables=[[] for _ in self.groups],
+                          dirty=[[] for _ in self.groups])
         self.requests[req_id] = rc
         return rc
 
@@ -240,6 +242,7 @@ class CacheManager:
             for i in range(lo, hi):
                 if table[i] < 0:
                     table[i] = self.pools[g].allocate()
+                    rc.dirty[g].append(i)
                     self.stats["pages_allocated"] += 1
 
     def commit(self, req_id: Hashable, tokens: Sequence[int]) -> None:
@@ -263,6 +266,7 @@ class CacheManager:
                 if table[i] >= 0:
                     self._release(g, table[i])
                     table[i] = -1
+                    rc.dirty[g].append(i)
 
     def _release(self, g: int, page: int) -> None:
         if self.pools[g].release(page):
@@ -275,6 +279,15 @@ class CacheManager:
     # ---- tables and slots for a step ------------------------------------------------
     def block_table(self, req_id: Hashable, group: int) -> List[int]:
         return self.get(req_id).tables[group]
+
+    def take_dirty(self, req_id: Hashable, group: int) -> List[Tuple[int, int]]:
+        """(table index, page id) of every entry of the request's table that changed since the
+        last call; for keeping a copy of the tables elsewhere (on the device) up to date."""
+        rc = self.get(req_id)
+        table = rc.tables[group]
+        out = [(i, table[i]) for i in dict.fromkeys(rc.dirty[group])]
+        rc.dirty[group] = []
+        return out
 
     def token_slots(self, req_id: Hashable, group: int, start: int, count: int) -> List[int]:
         """page * page_size + offset for positions start .. start + count - 1."""
@@ -315,6 +328,7 @@ class CacheManager:
         for entry in taken:
             for g, page in enumerate(entry.pages):
                 self.pools[g].retain(page)
+                rc.dirty[g].append(len(rc.tables[g]))
                 rc.tables[g].append(page)
         n = len(taken) * P
         rc.num_tokens = n

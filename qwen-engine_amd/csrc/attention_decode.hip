@@ -24,24 +24,44 @@ typedef __attribute__((ext_vector_type(4))) float floatx4;
 
 __device__ __forceinline__ short bf16_bits(float f) { return (short)float_to_bf16(f).bits; }
 
+// One tile of 16 keys in registers: the K rows as MFMA A operands, the V^T rows likewise.
 template <int D>
+struct KVTile {
+    bf16x8 k[D / 32];
+    short4_t v[D / 16];
+};
+
+template <int D>
+__device__ __forceinline__ void load_tile(KVTile<D>& tile, const bf16_t* __restrict__ cache, long page,
+                                          long page_stride, int kvh, int Hkv, int P, int o, int g, int n) {
+    const bf16_t* kbase = cache + page * page_stride + ((long)kvh * P + o) * D + (long)n * D + g * 8;
+    const bf16_t* vbase = cache + page * page_stride + ((long)(Hkv + kvh) * P) * D + o + (long)n * P + g * 4;
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) tile.k[c] = *(const bf16x8*)(kbase + c * 32);
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) tile.v[db] = *(const short4_t*)(vbase + (long)db * 16 * P);
+}
+
+// SPLIT: keys per split (a multiple of 16).  The next tile is loaded while the current one is
+// computed, and the split's page ids are read before the loop.
+template <int D, int SPLIT>
 __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
     const int* __restrict__ dec_tokens, const int* __restrict__ positions, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int max_blocks,
     float* __restrict__ part_acc, float* __restrict__ part_ml,
-    int Hq, int Hkv, int P, float scale, int window, int split_keys, int num_splits) {
+    int Hq, int Hkv, int P, float scale, int window, int num_splits) {
+    constexpr int TILES = SPLIT / 16;
     const int lane = threadIdx.x, g = lane >> 4, n = lane & 15;
     const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
     const int G = Hq / Hkv;
     const int t = dec_tokens[di];
     const int p = positions[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    const int k_begin = max(split * split_keys, lo);
-    const int k_end = min((split + 1) * split_keys, p + 1);
+    const int k_begin = max(split * SPLIT, lo);
+    const int k_end = min((split + 1) * SPLIT, p + 1);
     const int head = kvh * G + n;
     const bool head_ok = n < G;
-    // partial results of this (token, head, split)
     float* pacc = part_acc + (((long)di * Hq + head) * num_splits + split) * D;
     float* pml = part_ml + (((long)di * Hq + head) * num_splits + split) * 2;
     if (k_begin >= k_end) {   // nothing of this split is seen by the token
@@ -50,6 +70,14 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     }
     const int* bt = block_table + (long)tok_seq[t] * max_blocks;
     const long page_stride = 2L * Hkv * P * D;
+    const int tile0 = (k_begin - split * SPLIT) / 16;                 // first and one-past-last tile of the split
+    const int tile1 = (k_end - split * SPLIT + 15) / 16;
+    int pages[TILES];
+#pragma unroll
+    for (int i = 0; i < TILES; ++i) {
+        const int kk = split * SPLIT + i * 16;
+        pages[i] = (i >= tile0 && i < tile1) ? bt[kk / P] : 0;
+    }
 
     bf16x8 qreg[D / 32];
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -62,29 +90,26 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
 #pragma unroll
     for (int db = 0; db < D / 16; ++db) acc[db] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    for (int kk = (k_begin / 16) * 16; kk < k_end; kk += 16) {
-        const long page = bt[kk / P];
-        const int o = kk % P;
-        const bf16_t* kbase = cache + page * page_stride + ((long)kvh * P + o) * D;
-        const bf16_t* vbase = cache + page * page_stride + ((long)(Hkv + kvh) * P) * D + o;
-        bf16x8 kreg[D / 32];
+    KVTile<D> cur, nxt;
+    load_tile<D>(cur, cache, pages[tile0], page_stride, kvh, Hkv, P, (split * SPLIT + tile0 * 16) % P, g, n);
 #pragma unroll
-        for (int c = 0; c < D / 32; ++c) kreg[c] = *(const bf16x8*)(kbase + (long)n * D + c * 32 + g * 8);
-        short4_t vreg[D / 16];
-#pragma unroll
-        for (int db = 0; db < D / 16; ++db) vreg[db] = *(const short4_t*)(vbase + (long)(db * 16 + n) * P + g * 4);
+    for (int i = 0; i < TILES; ++i) {
+        if (i < tile0 || i >= tile1) continue;
+        const int kk = split * SPLIT + i * 16;
+        if (i + 1 < tile1)
+            load_tile<D>(nxt, cache, pages[(i + 1 < TILES) ? i + 1 : i], page_stride, kvh, Hkv, P, (kk + 16) % P, g, n);
 
         floatx4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int c = 0; c < D / 32; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[c], qreg[c], s, 0, 0, 0);
+        for (int c = 0; c < D / 32; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[c], qreg[c], s, 0, 0, 0);
         float tmax = -INFINITY;
         bool ok[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int key = kk + g * 4 + i;
-            ok[i] = key >= k_begin && key < k_end;
-            s[i] = ok[i] ? s[i] * scale : -INFINITY;
-            tmax = fmaxf(tmax, s[i]);
+        for (int j = 0; j < 4; ++j) {
+            const int key = kk + g * 4 + j;
+            ok[j] = key >= k_begin && key < k_end;
+            s[j] = ok[j] ? s[j] * scale : -INFINITY;
+            tmax = fmaxf(tmax, s[j]);
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
@@ -93,10 +118,10 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
         short4_t pb;
         float psum = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float pi = __expf(s[i] - mn);  // 0 for keys that are not seen
-            psum += pi;
-            pb[i] = bf16_bits(pi);
+        for (int j = 0; j < 4; ++j) {
+            const float pj = __expf(s[j] - mn);  // 0 for keys that are not seen
+            psum += pj;
+            pb[j] = bf16_bits(pj);
         }
         l = l * alpha + psum;
         m = mn;
@@ -105,50 +130,67 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
 #pragma unroll
         for (int db = 0; db < D / 16; ++db) {
             acc[db] *= alpha;
-            acc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg[db] & vmask, pb, acc[db], 0, 0, 0);
+            acc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(cur.v[db] & vmask, pb, acc[db], 0, 0, 0);
         }
+        cur = nxt;
     }
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (head_ok) {
 #pragma unroll
         for (int db = 0; db < D / 16; ++db)
-            *(floatx4*)(pacc + db * 16 + g * 4) = acc[db];    // O^T rows d = db * 16 + g * 4 + i of column head n
+            *(floatx4*)(pacc + db * 16 + g * 4) = acc[db];    // O^T rows d = db * 16 + g * 4 + j of column head n
         if (g == 0) { pml[0] = m; pml[1] = l; }
     }
 }
 
-// out[t, head, :] = sum_s e^{m_s - M} acc_s / sum_s e^{m_s - M} l_s,  M = max_s m_s
+// out[t, head, :] = sum_s e^{m_s - M} acc_s / sum_s e^{m_s - M} l_s,  M = max_s m_s.
+// One block of 256 threads per (token, head): wave w sums the splits w, w + 4, ... in ascending
+// order, the four sums are added in the order of the waves.
 template <int D>
-__global__ __launch_bounds__(64) void attention_decode_merge_kernel(
+__global__ __launch_bounds__(256) void attention_decode_merge_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, const int* __restrict__ dec_tokens,
     bf16_t* __restrict__ out, int Hq, int num_splits) {
-    const int di = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    constexpr int PER = (D + 63) / 64;
+    __shared__ float red_o[4][D];
+    __shared__ float red_l[4];
+    __shared__ float red_m[4];
+    const int di = blockIdx.x, head = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* pml = part_ml + ((long)di * Hq + head) * num_splits * 2;
     const float* pacc = part_acc + ((long)di * Hq + head) * num_splits * D;
     float M = -INFINITY;
-    for (int s = 0; s < num_splits; ++s) M = fmaxf(M, pml[2 * s]);
+    for (int s = lane; s < num_splits; s += 64) M = fmaxf(M, pml[2 * s]);
+    M = wave_max(M);
     float denom = 0.f;
-    float o[(D + 63) / 64];
+    float o[PER];
 #pragma unroll
-    for (int i = 0; i < (D + 63) / 64; ++i) o[i] = 0.f;
-    for (int s = 0; s < num_splits; ++s) {
+    for (int i = 0; i < PER; ++i) o[i] = 0.f;
+    for (int s = wave; s < num_splits; s += 4) {
         const float ms = pml[2 * s];
         if (ms == -INFINITY) continue;          // an empty split: its accumulator was never written
         const float wgt = __expf(ms - M);
         denom += wgt * pml[2 * s + 1];
 #pragma unroll
-        for (int i = 0; i < (D + 63) / 64; ++i) {
+        for (int i = 0; i < PER; ++i) {
             const int d = lane + i * 64;
             if (d < D) o[i] += wgt * pacc[(long)s * D + d];
         }
     }
-    bf16_t* orow = out + ((long)dec_tokens[di] * Hq + head) * D;
-    const float inv = 1.f / denom;
 #pragma unroll
-    for (int i = 0; i < (D + 63) / 64; ++i) {
+    for (int i = 0; i < PER; ++i) {
         const int d = lane + i * 64;
-        if (d < D) orow[d] = float_to_bf16(o[i] * inv);
+        if (d < D) red_o[wave][d] = o[i];
+    }
+    if (lane == 0) red_l[wave] = denom;
+    __syncthreads();
+    if (wave == 0) {
+        const float inv = 1.f / (red_l[0] + red_l[1] + red_l[2] + red_l[3]);
+        bf16_t* orow = out + ((long)dec_tokens[di] * Hq + head) * D;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int d = lane + i * 64;
+            if (d < D) orow[d] = float_to_bf16((red_o[0][d] + red_o[1][d] + red_o[2][d] + red_o[3][d]) * inv);
+        }
     }
 }
 
@@ -168,7 +210,7 @@ int qe_attention_decode(const void* q, void* out, const void* cache, const int* 
                         int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
                         int split_keys, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     QE_REQUIRE(qe_attention_decode_ok(Hq, Hkv, D, P, QE_BF16), "decode attention: sizes not taken");
-    QE_REQUIRE(split_keys >= 16 && split_keys % 16 == 0, "decode attention: split of %d keys", split_keys);
+    QE_REQUIRE(split_keys == 128 || split_keys == 256, "decode attention: splits of 128 or 256 keys, not %d", split_keys);
     if (n_dec == 0) return 0;
     const int num_splits = max_position / split_keys + 1;
     QE_REQUIRE(num_splits <= 65535 && n_dec <= 65535, "decode attention: too many splits or tokens");
@@ -176,19 +218,22 @@ int qe_attention_decode(const void* q, void* out, const void* cache, const int* 
                "decode attention: workspace of %zu bytes is too small", workspace_bytes);
     float* part_acc = (float*)workspace;
     float* part_ml = part_acc + (size_t)n_dec * Hq * num_splits * D;
+    (void)qe_cdiv;
     dim3 grid(num_splits, Hkv, n_dec);
     dim3 mgrid(n_dec, Hq);
-    if (D == 128) {
-        attention_decode_split_kernel<128><<<grid, 64, 0, stream>>>(
-            (const bf16_t*)q, (const bf16_t*)cache, dec_tokens, positions, tok_seq, block_table, max_blocks,
-            part_acc, part_ml, Hq, Hkv, P, scale, window, split_keys, num_splits);
-        attention_decode_merge_kernel<128><<<mgrid, 64, 0, stream>>>(part_acc, part_ml, dec_tokens, (bf16_t*)out, Hq, num_splits);
-    } else {
-        attention_decode_split_kernel<64><<<grid, 64, 0, stream>>>(
-            (const bf16_t*)q, (const bf16_t*)cache, dec_tokens, positions, tok_seq, block_table, max_blocks,
-            part_acc, part_ml, Hq, Hkv, P, scale, window, split_keys, num_splits);
-        attention_decode_merge_kernel<64><<<mgrid, 64, 0, stream>>>(part_acc, part_ml, dec_tokens, (bf16_t*)out, Hq, num_splits);
-    }
+#define QE_DECODE(D_, S_)                                                                               \
+    do {                                                                                                \
+        attention_decode_split_kernel<D_, S_><<<grid, 64, 0, stream>>>(                                 \
+            (const bf16_t*)q, (const bf16_t*)cache, dec_tokens, positions, tok_seq, block_table,        \
+            max_blocks, part_acc, part_ml, Hq, Hkv, P, scale, window, num_splits);                      \
+        attention_decode_merge_kernel<D_><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, dec_tokens,     \
+                                                                     (bf16_t*)out, Hq, num_splits);     \
+    } while (0)
+    if (D == 128 && split_keys == 128) QE_DECODE(128, 128);
+    else if (D == 128) QE_DECODE(128, 256);
+    else if (split_keys == 128) QE_DECODE(64, 128);
+    else QE_DECODE(64, 256);
+#undef QE_DECODE
     QE_LAUNCH_CHECK();
     return 0;
 }

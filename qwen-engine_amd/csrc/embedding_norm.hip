@@ -28,23 +28,26 @@ extern "C" int qe_embedding(const int* ids, const void* table, float* out, int T
 }
 
 // One block per output row r.  src row = rows ? rows[r] : r.
-//   v = h[src] (+ delta[src]);  if delta and !rows: h[src] = v  (the residual sum, in 32-bit)
+//   v = h[src] (+ delta_0[src] + delta_1[src] + ...);  if delta and !rows: h[src] = v  (the residual sum, 32-bit)
 //   out[r] = v * rsqrt(mean(v^2) + eps) * w        (all in 32-bit, one rounding at the store)
-// Two passes over the row; the second re-reads h (and delta) instead of keeping
-// the row in registers, so any H is taken.
-template <typename TA>
-__global__ void rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__ delta,
+// delta holds n_delta tensors [T, H] one after the other (partial products of a matrix product cut
+// along K, or one branch output); they are added in ascending order.
+// Two passes over the row; the second re-reads h (and delta) instead of keeping the row in
+// registers, so any H is taken.
+template <typename TA, typename TD>
+__global__ void rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_delta, long delta_stride,
                                const int* __restrict__ rows, const float* __restrict__ w,
                                TA* __restrict__ out, int H, float eps) {
     __shared__ float red[16];
     const long r = blockIdx.x;
     const long src = rows ? (long)rows[r] : r;
     float* hr = h + src * H;
-    const TA* dr = delta ? delta + src * H : nullptr;
+    const TD* dr = delta ? delta + src * H : nullptr;
     float ss = 0.f;
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float v = hr[c];
-        if (dr) v += Elem<TA>::load(dr + c);
+        if (dr)
+            for (int s = 0; s < n_delta; ++s) v += Elem<TD>::load(dr + s * delta_stride + c);
         ss += v * v;
     }
     ss = block_sum(ss, red);
@@ -53,23 +56,30 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__ del
     const bool write_back = dr && !rows;
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float v = hr[c];
-        if (dr) v += Elem<TA>::load(dr + c);
+        if (dr)
+            for (int s = 0; s < n_delta; ++s) v += Elem<TD>::load(dr + s * delta_stride + c);
         if (write_back) hr[c] = v;
         Elem<TA>::store(o + c, v * rstd * w[c]);
     }
 }
 
-extern "C" int qe_rmsnorm(float* h, const void* delta, const int* rows, const float* w, void* out,
-                          int n_out_rows, int H, float eps, int dt_a, hipStream_t stream) {
+// dt_d: element type of delta (that of the output, or float for partial products)
+extern "C" int qe_rmsnorm(float* h, const void* delta, int n_delta, int dt_d, long n_rows_h, const int* rows,
+                          const float* w, void* out, int n_out_rows, int H, float eps, int dt_a,
+                          hipStream_t stream) {
     QE_REQUIRE(n_out_rows >= 0 && H > 0, "rmsnorm: bad sizes rows=%d H=%d", n_out_rows, H);
+    QE_REQUIRE(!delta || n_delta >= 1, "rmsnorm: %d delta tensors", n_delta);
     if (n_out_rows == 0) return 0;
     const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
-    if (dt_a == QE_F32)
-        rmsnorm_kernel<float><<<n_out_rows, threads, 0, stream>>>(h, (const float*)delta, rows, w, (float*)out, H, eps);
-    else if (dt_a == QE_BF16)
-        rmsnorm_kernel<bf16_t><<<n_out_rows, threads, 0, stream>>>(h, (const bf16_t*)delta, rows, w, (bf16_t*)out, H, eps);
+    const long stride = n_rows_h * H;
+    if (dt_a == QE_F32 && (!delta || dt_d == QE_F32))
+        rmsnorm_kernel<float, float><<<n_out_rows, threads, 0, stream>>>(h, (const float*)delta, n_delta, stride, rows, w, (float*)out, H, eps);
+    else if (dt_a == QE_BF16 && (!delta || dt_d == QE_BF16))
+        rmsnorm_kernel<bf16_t, bf16_t><<<n_out_rows, threads, 0, stream>>>(h, (const bf16_t*)delta, n_delta, stride, rows, w, (bf16_t*)out, H, eps);
+    else if (dt_a == QE_BF16 && dt_d == QE_F32)
+        rmsnorm_kernel<bf16_t, float><<<n_out_rows, threads, 0, stream>>>(h, (const float*)delta, n_delta, stride, rows, w, (bf16_t*)out, H, eps);
     else
-        QE_REQUIRE(false, "rmsnorm: unknown dtype %d", dt_a);
+        QE_REQUIRE(false, "rmsnorm: no kernel for output type %d with delta type %d", dt_a, dt_d);
     QE_LAUNCH_CHECK();
     return 0;
 }
@@ -118,6 +128,22 @@ extern "C" int qe_silu_mul(const void* gu, void* out, int T, int I, int dt_a, hi
         silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, T, I);
     else
         QE_REQUIRE(false, "silu_mul: unknown dtype %d", dt_a);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// table[idx[i]] = val[i] for idx[i] >= 0: keeps the device's copy of the block tables up to date.
+__global__ void scatter_int_kernel(int* __restrict__ table, const int* __restrict__ idx,
+                                   const int* __restrict__ val, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n && idx[i] >= 0) table[idx[i]] = val[i];
+}
+
+extern "C" int qe_scatter_int(int* table, const int* idx, const int* val, int n, long table_size,
+                              hipStream_t stream) {
+    QE_REQUIRE(n >= 0 && table_size >= 0, "scatter: bad sizes");
+    if (n == 0) return 0;
+    scatter_int_kernel<<<qe_cdiv(n, 256), 256, 0, stream>>>(table, idx, val, n);
     QE_LAUNCH_CHECK();
     return 0;
 }

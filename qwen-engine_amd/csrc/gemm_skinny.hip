@@ -10,24 +10,31 @@
 // The result tile has, per lane, 4 consecutive n for one token: one 8- or 16-byte store.
 //
 // Epilogues: store (+ bias); add into a 32-bit residual stream; silu(gate) * up, where W holds
-// the gate rows followed by the up rows and a block owns 16 of each.
+// the gate rows followed by the up rows and a block owns 16 of each; 32-bit partial products
+// of a product cut along K over several blocks (for matrices with few rows, to fill the chip).
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 
-enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2 };
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3 };
 
+// grid (N / 16, S): block (bx, s) sums the chunks [s * cps, (s + 1) * cps) of K.  With S > 1 the
+// epilogue is EPI_PARTIAL: 32-bit partial products out[s][M][N] that the consumer adds up in the
+// order of s (the fused residual-add + norm kernel does), so the sum has one fixed order.
 template <int MT, int EPI, typename TO>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    TO* __restrict__ out, int M, int N, int K) {
+    TO* __restrict__ out, int M, int N, int K, int cps) {
     constexpr int NW = (EPI == EPI_SILU_MUL) ? 2 : 1;   // weight tiles per block
+    constexpr int U = (MT <= 2) ? 4 : 2;                // chunks whose loads are issued together
     __shared__ float red[4][NW][MT][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r = lane & 15;
     const int n0 = blockIdx.x * 16;
     const int nchunks = K / 32;
+    const int c_begin = blockIdx.y * cps;
+    const int c_end = min(nchunks, c_begin + cps);
 
     floatx4 acc[NW][MT];
 #pragma unroll
@@ -47,17 +54,25 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
     }
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-    for (int c = wave; c < nchunks; c += 4) {
-        bf16x8 a0 = row_ok ? *(const bf16x8*)(wrow0 + c * 32) : zero;
-        bf16x8 a1 = zero;
-        if (EPI == EPI_SILU_MUL) a1 = row_ok ? *(const bf16x8*)(wrow1 + c * 32) : zero;
+    for (int c = c_begin + wave; c < c_end; c += 4 * U) {
+        bf16x8 a0[U], a1[U], b[U][MT];
 #pragma unroll
-        for (int j = 0; j < MT; ++j) {
-            const bf16x8 b = tok_ok[j] ? *(const bf16x8*)(xrow[j] + c * 32) : zero;
-            acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b, acc[0][j], 0, 0, 0);
-            if (EPI == EPI_SILU_MUL)
-                acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b, acc[1][j], 0, 0, 0);
+        for (int u = 0; u < U; ++u) {
+            const int cc = c + 4 * u;
+            const bool ok = cc < c_end;
+            a0[u] = (ok && row_ok) ? *(const bf16x8*)(wrow0 + cc * 32) : zero;
+            if (EPI == EPI_SILU_MUL) a1[u] = (ok && row_ok) ? *(const bf16x8*)(wrow1 + cc * 32) : zero;
+#pragma unroll
+            for (int j = 0; j < MT; ++j) b[u][j] = (ok && tok_ok[j]) ? *(const bf16x8*)(xrow[j] + cc * 32) : zero;
         }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < MT; ++j) {
+                acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[u], b[u][j], acc[0][j], 0, 0, 0);
+                if (EPI == EPI_SILU_MUL)
+                    acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[u], b[u][j], acc[1][j], 0, 0, 0);
+            }
     }
 #pragma unroll
     for (int a = 0; a < NW; ++a)
@@ -83,14 +98,16 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
             float y = v[0][i];
             if (EPI == EPI_SILU_MUL) {
                 y = y / (1.f + __expf(-y)) * v[1][i];
-            } else if (bias) {
+            } else if (bias && blockIdx.y == 0) {
                 y += bias[n];
             }
-            TO* o = out + (long)t * N + n;
-            if (EPI == EPI_RESIDUAL) {
-                *(float*)o = *(const float*)o + y;
+            if (EPI == EPI_PARTIAL) {
+                ((float*)out)[((long)blockIdx.y * M + t) * N + n] = y;
+            } else if (EPI == EPI_RESIDUAL) {
+                float* o = (float*)out + (long)t * N + n;
+                *o = *o + y;
             } else {
-                Elem<TO>::store(o, y);
+                Elem<TO>::store(out + (long)t * N + n, y);
             }
         }
     }
@@ -98,12 +115,13 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
 
 template <int EPI, typename TO>
 static int launch_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                         hipStream_t stream) {
-    const int blocks = qe_cdiv(N, 16);
+                         int splits, hipStream_t stream) {
+    const dim3 grid(qe_cdiv(N, 16), splits);
+    const int cps = qe_cdiv(K / 32, splits);
     const int mt = qe_cdiv(M, 16);
 #define QE_SKINNY(MT_)                                                                            \
-    gemm_skinny_kernel<MT_, EPI, TO><<<blocks, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, \
-                                                                 (TO*)out, M, N, K)
+    gemm_skinny_kernel<MT_, EPI, TO><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, \
+                                                               (TO*)out, M, N, K, cps)
     switch (mt) {
         case 1: QE_SKINNY(1); break;
         case 2: QE_SKINNY(2); break;
@@ -119,21 +137,39 @@ bool qe_gemm_skinny_ok(int M, int N, int K, int dt_a, int dt_w) {
     return dt_a == QE_BF16 && dt_w == QE_BF16 && M >= 1 && M <= 64 && K % 32 == 0 && K >= 32;
 }
 
+// How many partial products a [M, N] = [M, K] . [N, K]^T product is best cut into along K so that
+// the launch has some 512 blocks, each wave still summing at least two chunks.
+int qe_gemm_skinny_splits(int N, int K) {
+    const int blocks = qe_cdiv(N, 16);
+    int s = 512 / (blocks > 0 ? blocks : 1);
+    const int most = (K / 32) / 8;
+    if (s > most) s = most;
+    if (s > 16) s = 16;
+    return s < 1 ? 1 : s;
+}
+
 // epilogue EPI_STORE: out [M, N] in dt_o.  EPI_RESIDUAL: out is the 32-bit stream [M, N], added to.
 // EPI_SILU_MUL: w is [2 N, K] (gate rows, then up rows), out [M, N] in dt_o.
+// EPI_PARTIAL: out is float [splits, M, N]; the product is the sum over the first index.
 int qe_gemm_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                   int dt_o, int epilogue, hipStream_t stream) {
+                   int dt_o, int epilogue, int splits, hipStream_t stream) {
     QE_REQUIRE(M >= 1 && M <= 64 && K % 32 == 0, "skinny gemm: M=%d K=%d not taken", M, K);
+    QE_REQUIRE(splits >= 1 && splits <= 64 && (epilogue == EPI_PARTIAL || splits == 1),
+               "skinny gemm: %d splits with epilogue %d", splits, epilogue);
+    if (epilogue == EPI_PARTIAL) {
+        QE_REQUIRE(dt_o == QE_F32, "skinny gemm: partial products are 32-bit");
+        return launch_skinny<EPI_PARTIAL, float>(x, w, bias, out, M, N, K, splits, stream);
+    }
     if (epilogue == EPI_RESIDUAL) {
         QE_REQUIRE(dt_o == QE_F32, "skinny gemm: the residual stream is 32-bit");
-        return launch_skinny<EPI_RESIDUAL, float>(x, w, bias, out, M, N, K, stream);
+        return launch_skinny<EPI_RESIDUAL, float>(x, w, bias, out, M, N, K, 1, stream);
     }
     if (epilogue == EPI_SILU_MUL) {
         QE_REQUIRE(!bias, "skinny gemm: silu-mul takes no bias");
-        if (dt_o == QE_BF16) return launch_skinny<EPI_SILU_MUL, bf16_t>(x, w, bias, out, M, N, K, stream);
-        return launch_skinny<EPI_SILU_MUL, float>(x, w, bias, out, M, N, K, stream);
+        if (dt_o == QE_BF16) return launch_skinny<EPI_SILU_MUL, bf16_t>(x, w, bias, out, M, N, K, 1, stream);
+        return launch_skinny<EPI_SILU_MUL, float>(x, w, bias, out, M, N, K, 1, stream);
     }
     QE_REQUIRE(epilogue == EPI_STORE, "skinny gemm: unknown epilogue %d", epilogue);
-    if (dt_o == QE_BF16) return launch_skinny<EPI_STORE, bf16_t>(x, w, bias, out, M, N, K, stream);
-    return launch_skinny<EPI_STORE, float>(x, w, bias, out, M, N, K, stream);
+    if (dt_o == QE_BF16) return launch_skinny<EPI_STORE, bf16_t>(x, w, bias, out, M, N, K, 1, stream);
+    return launch_skinny<EPI_STORE, float>(x, w, bias, out, M, N, K, 1, stream);
 }

@@ -32,10 +32,78 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
     if (threadIdx.x == 0) out[blockIdx.x] = si[0];
 }
 
-extern "C" int qe_argmax(const float* logits, int* out, int R, int V, hipStream_t stream) {
+// Two stages for wide vocabularies: each block of the first takes a contiguous span of a row
+// and leaves its best (value, index); the second picks among the spans, lowest index on ties.
+__global__ __launch_bounds__(256) void argmax_span_kernel(const float* __restrict__ logits, float* __restrict__ pv,
+                                                          int* __restrict__ pi, int V, int span) {
+    __shared__ float sv[256];
+    __shared__ int si[256];
+    const float* row = logits + (long)blockIdx.x * V;
+    const int c0 = blockIdx.y * span;
+    const int c1 = min(V, c0 + span);
+    float best = -INFINITY;
+    int bi = -1;
+    for (int c = c0 + threadIdx.x; c < c1; c += 256) {
+        const float v = row[c];
+        if (bi < 0 || v > best) { best = v; bi = c; }
+    }
+    sv[threadIdx.x] = best;
+    si[threadIdx.x] = bi;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) {
+            const float ov = sv[threadIdx.x + s], mv = sv[threadIdx.x];
+            const int oi = si[threadIdx.x + s], mi = si[threadIdx.x];
+            if (oi >= 0 && (mi < 0 || ov > mv || (ov == mv && oi < mi))) { sv[threadIdx.x] = ov; si[threadIdx.x] = oi; }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        pv[blockIdx.x * gridDim.y + blockIdx.y] = sv[0];
+        pi[blockIdx.x * gridDim.y + blockIdx.y] = si[0];
+    }
+}
+
+__global__ __launch_bounds__(64) void argmax_pick_kernel(const float* __restrict__ pv, const int* __restrict__ pi,
+                                                         int* __restrict__ out, int spans) {
+    float best = -INFINITY;
+    int bi = -1;
+    for (int s = threadIdx.x; s < spans; s += 64) {
+        const float v = pv[blockIdx.x * spans + s];
+        const int i = pi[blockIdx.x * spans + s];
+        if (i >= 0 && (bi < 0 || v > best || (v == best && i < bi))) { best = v; bi = i; }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (oi >= 0 && (bi < 0 || ov > best || (ov == best && oi < bi))) { best = ov; bi = oi; }
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = bi;
+}
+
+#define ARGMAX_SPAN 2048
+
+// bytes of workspace that qe_argmax needs for these sizes (0: none)
+extern "C" long qe_argmax_workspace_bytes(int R, int V) {
+    if (V <= 2 * ARGMAX_SPAN) return 0;
+    return (long)R * qe_cdiv(V, ARGMAX_SPAN) * 8;
+}
+
+extern "C" int qe_argmax(const float* logits, int* out, int R, int V, void* workspace, long workspace_bytes,
+                         hipStream_t stream) {
     QE_REQUIRE(R >= 0 && V > 0, "argmax: bad sizes R=%d V=%d", R, V);
     if (R == 0) return 0;
-    argmax_kernel<<<R, 256, 0, stream>>>(logits, out, V);
+    if (V <= 2 * ARGMAX_SPAN) {
+        argmax_kernel<<<R, 256, 0, stream>>>(logits, out, V);
+    } else {
+        const int spans = qe_cdiv(V, ARGMAX_SPAN);
+        QE_REQUIRE(workspace && workspace_bytes >= (long)R * spans * 8, "argmax: workspace too small");
+        QE_REQUIRE(spans <= 65535, "argmax: vocabulary too wide");
+        float* pv = (float*)workspace;
+        int* pi = (int*)(pv + (long)R * spans);
+        argmax_span_kernel<<<dim3(R, spans), 256, 0, stream>>>(logits, pv, pi, V, ARGMAX_SPAN);
+        argmax_pick_kernel<<<R, 64, 0, stream>>>(pv, pi, out, spans);
+    }
     QE_LAUNCH_CHECK();
     return 0;
 }

@@ -17,6 +17,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.plan import CachePlan
 from ..config.registry import config_from_folder
+from ..kernels import ops
 from ..parts.base import CacheBinding, Runtime
 from ..parts.model import DecoderModel, cache_plan, expected_tensors
 from ..weights.loader import read_checked
@@ -57,15 +58,25 @@ def load_model(folder: str, dtype="bfloat16", device="cuda:0") -> DecoderModel:
 
 
 class ModelRunner:
-    """Owns the cache storage on the device and runs steps of one model."""
+    """Owns the cache storage on the device and runs steps of one model.
+
+    The block tables live on the device, one row per state slot; a step uploads only the
+    entries that changed (new pages, pages a window has passed) together with the batch's
+    tokens, positions and cache slots in one copy.  Steps in which every request brings one
+    token and wants its logits (decoding) are recorded once per batch size as a HIP graph
+    and replayed, so that their launch cost does not grow with the number of kernels.
+    """
+
+    SPLIT_BUCKET = 8      # decode graphs are recorded per this many splits of the keys
 
     def __init__(self, model: DecoderModel, page_size: int, num_pages, max_requests: int,
-                 prefix_sharing: bool = False):
+                 prefix_sharing: bool = False, use_graphs: Optional[bool] = None):
         if model.rt is None:
             raise RuntimeError("the model has no weights yet")
         self.model = model
         self.rt = model.rt
         self.page_size = int(page_size)
+        self.max_requests = int(max_requests)
         self.plan: CachePlan = cache_plan(model.spec)
         has_state = any(s is not None for s in self.plan.entry_state)
         self.cache = CacheManager(self.plan.groups or [], num_pages, page_size, max_requests,
@@ -94,7 +105,18 @@ class ModelRunner:
                 group=self.plan.entry_group[i],
                 write=(src == i),
                 state=self.state[i]))
+        # device copies of the block tables: [state slots, pages a request can hold]
+        per_request = (model.spec.max_positions + page_size - 1) // page_size
+        # (a table is indexed by position // page size: with a window the indices go on growing
+        # while the entries behind the window are -1, so only a group that keeps all keys is
+        # bounded by its pool)
+        self.table_width = [max(1, per_request if grp.window is not None else min(pool.num_pages, per_request))
+                            for grp, pool in zip(self.cache.groups, self.cache.pools)]
+        self.tables = [torch.full((max_requests, w), -1, dtype=torch.int32, device=dev) for w in self.table_width]
+        self.use_graphs = (dt == torch.bfloat16 and not has_state) if use_graphs is None else bool(use_graphs)
+        self._graphs = {}
         self.steps_run = 0
+        self.graph_steps = 0
 
     # ---- requests ------------------------------------------------------------------
     def add_request(self, req_id: Hashable):
@@ -107,9 +129,8 @@ class ModelRunner:
         return sum(t.numel() * t.element_size() for t in self.kv if t is not None)
 
     # ---- one step ----------------------------------------------------------------------
-    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
-        """Reserves pages for the entries' tokens and lays the batch out flat."""
-        cache, P = self.cache, self.page_size
+    def _check_and_reserve(self, entries: Sequence[StepEntry]) -> None:
+        cache = self.cache
         vocab = self.model.spec.vocab_size
         max_pos = self.model.spec.max_positions
         if not entries:
@@ -136,6 +157,9 @@ class ModelRunner:
         for e in entries:
             cache.reserve(e.req_id, cache.get(e.req_id).num_tokens + len(e.tokens))
 
+    def _layout(self, entries: Sequence[StepEntry]):
+        """The batch as flat host lists: (seqs, named lists of ints, per-group lists)."""
+        cache = self.cache
         seqs: List[SeqInfo] = []
         token_ids: List[int] = []
         positions: List[int] = []
@@ -143,68 +167,174 @@ class ModelRunner:
         rows: List[int] = []
         n_groups = len(cache.groups)
         slots: List[List[int]] = [[] for _ in range(n_groups)]
+        upd_idx: List[List[int]] = [[] for _ in range(n_groups)]
+        upd_val: List[List[int]] = [[] for _ in range(n_groups)]
         q_start = 0
-        for b, e in enumerate(entries):
+        for e in entries:
             rc = cache.get(e.req_id)
             n = len(e.tokens)
             seqs.append(SeqInfo(e.req_id, q_start, n, rc.num_tokens, rc.state_slot, rc.new_request))
             token_ids.extend(int(t) for t in e.tokens)
             positions.extend(range(rc.num_tokens, rc.num_tokens + n))
-            tok_seq.extend([b] * n)
+            tok_seq.extend([rc.state_slot] * n)          # the request's row in the device tables
             rows.extend(q_start + int(w) for w in e.want)
             for g in range(n_groups):
                 slots[g].extend(cache.token_slots(e.req_id, g, rc.num_tokens, n))
+                width = self.table_width[g]
+                for i, page in cache.take_dirty(e.req_id, g):
+                    if i >= width:
+                        raise RuntimeError("a request holds more pages than its table row has entries")
+                    upd_idx[g].append(rc.state_slot * width + i)
+                    upd_val[g].append(page)
             q_start += n
-        T, B = q_start, len(entries)
-        tables = []
-        for g in range(n_groups):
-            width = max(1, max(len(cache.block_table(e.req_id, g)) for e in entries))
-            tab = [list(cache.block_table(e.req_id, g)) for e in entries]
-            tables.append([row + [-1] * (width - len(row)) for row in tab])
+        return seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val
 
-        # one host buffer, one copy to the device
+    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Reserves pages for the entries' tokens, lays the batch out flat, and brings the
+        device's block tables up to date (one copy to the device, one small kernel per group)."""
+        self._check_and_reserve(entries)
+        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(entries)
+        T, B, n_groups = len(token_ids), len(seqs), len(self.cache.groups)
         dec_rows = [s.q_start for s in seqs if s.q_len == 1]
         other_rows = [s.q_start + i for s in seqs if s.q_len > 1 for i in range(s.q_len)]
         max_dec = max([s.kv_before for s in seqs if s.q_len == 1], default=0)
         parts = [token_ids, positions, tok_seq, rows, [s.state_slot for s in seqs], dec_rows, other_rows]
         for g in range(n_groups):
-            parts.append(slots[g])
-            parts.append([p for row in tables[g] for p in row])
+            parts += [slots[g], upd_idx[g], upd_val[g]]
         flat = [v for part in parts for v in part]
-        host = torch.tensor(flat, dtype=torch.int32).pin_memory() if flat else torch.zeros(0, dtype=torch.int32)
+        host = torch.tensor(flat, dtype=torch.int32).pin_memory()
         dev = host.to(self.rt.device, non_blocking=True)
         off = 0
 
-        def take(n, shape=None):
+        def take(n):
             nonlocal off
             t = dev[off:off + n]
             off += n
-            return t.view(shape) if shape is not None else t
+            return t
 
         d_tok, d_pos, d_seq = take(T), take(T), take(T)
         d_rows, d_state = take(len(rows)), take(B)
         d_dec, d_other = take(len(dec_rows)), take(len(other_rows))
-        d_slots, d_tables = [], []
+        d_slots = []
         for g in range(n_groups):
             d_slots.append(take(T))
-            width = len(tables[g][0])
-            d_tables.append(take(B * width, (B, width)))
-        return StepContext(rt=self.rt, page_size=P, num_tokens=T, seqs=seqs, token_ids=d_tok,
-                           positions=d_pos, tok_seq=d_seq, block_tables=d_tables, slots=d_slots,
+            n_upd = len(upd_idx[g])
+            d_idx, d_val = take(n_upd), take(n_upd)
+            if n_upd:
+                ops.scatter_int(self.tables[g], d_idx, d_val)
+        return StepContext(rt=self.rt, page_size=self.page_size, num_tokens=T, seqs=seqs, token_ids=d_tok,
+                           positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
                            logit_rows=d_rows, state_slots=d_state, max_position=max(positions),
                            dec_tokens=d_dec, other_tokens=d_other, max_dec_position=max_dec)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Runs the entries' tokens as one batch; returns float32 logits [wanted, vocab] on the
         device, in the order of the entries and of their ``want``."""
-        ctx = self.build_context(entries)
-        for s in ctx.seqs:          # fixed-size state of a starting request begins at zero
-            if s.new_request:
-                for st in self.state:
-                    if st is not None:
-                        st[s.state_slot].zero_()
-        logits = self.model.forward(ctx, self.bindings)
+        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries) and entries:
+            logits = self._decode_step_with_graph(entries)
+        else:
+            ctx = self.build_context(entries)
+            for s in ctx.seqs:          # fixed-size state of a starting request begins at zero
+                if s.new_request:
+                    for st in self.state:
+                        if st is not None:
+                            st[s.state_slot].zero_()
+            logits = self.model.forward(ctx, self.bindings)
         for e in entries:
             self.cache.commit(e.req_id, e.tokens)
         self.steps_run += 1
         return logits
+
+    # ---- decoding through a recorded graph ------------------------------------------------
+    def _decode_step_with_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        self._check_and_reserve(entries)
+        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(entries)
+        B, n_groups = len(seqs), len(self.cache.groups)
+        cap = 2 * B                                    # table updates a decode step can bring per group
+        splits = max(positions) // ops.DECODE_SPLIT_KEYS + 1
+        bucket = (splits + self.SPLIT_BUCKET - 1) // self.SPLIT_BUCKET * self.SPLIT_BUCKET
+        if any(len(u) > cap for u in upd_idx):
+            # more table changes than the recorded step takes (the first decode step after a
+            # preemption, say): bring the tables up to date apart, then go on with none
+            for g in range(n_groups):
+                if upd_idx[g]:
+                    ops.scatter_int(self.tables[g],
+                                    torch.tensor(upd_idx[g], dtype=torch.int32).to(self.rt.device),
+                                    torch.tensor(upd_val[g], dtype=torch.int32).to(self.rt.device))
+                upd_idx[g], upd_val[g] = [], []
+        key = (B, bucket)
+        rec = self._graphs.get(key)
+        if rec is None:
+            rec = self._record_decode_graph(B, bucket, cap)
+            self._graphs[key] = rec
+        parts = [token_ids, positions, tok_seq, list(range(B)), [s.state_slot for s in seqs], list(range(B))]
+        for g in range(n_groups):
+            pad = cap - len(upd_idx[g])
+            parts += [slots[g], upd_idx[g] + [-1] * pad, upd_val[g] + [0] * pad]
+        flat = [v for part in parts for v in part]
+        rec["event"].synchronize()                     # the last copy out of the host buffer is done
+        rec["host"].copy_(torch.tensor(flat, dtype=torch.int32))
+        rec["meta"].copy_(rec["host"], non_blocking=True)
+        rec["event"].record()
+        rec["graph"].replay()
+        self.graph_steps += 1
+        return rec["logits"].clone()                   # the graph's own output is overwritten by the next replay
+
+    def _record_decode_graph(self, B: int, bucket: int, cap: int):
+        """Static buffers for a decode step of B requests whose keys fit ``bucket`` splits, one
+        run outside the graph (so that nothing is set up for the first time while recording),
+        then the recording."""
+        dev, n_groups = self.rt.device, len(self.cache.groups)
+        n = 6 * B + n_groups * (B + 2 * cap)
+        host = torch.zeros(n, dtype=torch.int32).pin_memory()
+        meta = torch.zeros(n, dtype=torch.int32, device=dev)
+        # a harmless stand-in batch for the runs that only record: every token at position 0 of
+        # slot 0, writing nowhere (cache slot -1), no table updates
+        stand_in = [0] * (3 * B) + list(range(B)) + [0] * B + list(range(B))
+        for g in range(n_groups):
+            stand_in += [-1] * B + [-1] * cap + [0] * cap
+        meta.copy_(torch.tensor(stand_in, dtype=torch.int32))
+        off = 0
+
+        def take(k):
+            nonlocal off
+            t = meta[off:off + k]
+            off += k
+            return t
+
+        d_tok, d_pos, d_seq, d_rows, d_state, d_dec = (take(B) for _ in range(6))
+        d_slots, d_upd = [], []
+        for g in range(n_groups):
+            d_slots.append(take(B))
+            d_upd.append((take(cap), take(cap)))
+        seqs = [SeqInfo(None, i, 1, 0, 0, False) for i in range(B)]
+        ctx = StepContext(rt=self.rt, page_size=self.page_size, num_tokens=B, seqs=seqs, token_ids=d_tok,
+                          positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
+                          logit_rows=d_rows, state_slots=d_state,
+                          max_position=0, dec_tokens=d_dec, other_tokens=None,
+                          max_dec_position=bucket * ops.DECODE_SPLIT_KEYS - 1)
+
+        def run():
+            for g in range(n_groups):
+                ops.scatter_int(self.tables[g], d_upd[g][0], d_upd[g][1])
+            return self.model.forward(ctx, self.bindings)
+
+        # slot 0's first table entry must name a real page while the stand-in batch runs
+        saved = [t[0, 0].item() for t in self.tables]
+        for t in self.tables:
+            t[0, 0] = 0
+        torch.cuda.synchronize()
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            run()
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            logits = run()
+        torch.cuda.synchronize()
+        for t, v in zip(self.tables, saved):
+            t[0, 0] = v
+        event = torch.cuda.Event()
+        event.record()
+        return {"graph": graph, "host": host, "meta": meta, "logits": logits, "event": event}

@@ -18,7 +18,7 @@ F32, BF16 = 0, 1
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
 
 ALGO_AUTO, ALGO_GENERIC, ALGO_FAST = 0, 1, 2
-EPI_STORE, EPI_RESIDUAL, EPI_SILU_MUL = 0, 1, 2
+EPI_STORE, EPI_RESIDUAL, EPI_SILU_MUL, EPI_PARTIAL = 0, 1, 2, 3
 DECODE_SPLIT_KEYS = 128   # keys per split of the decode attention kernel
 
 
@@ -42,22 +42,26 @@ def load_library():
     vp, i32, f32, i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_long
     sigs = {
         "qe_embedding": [vp, vp, vp, i32, i32, i32, i32, vp],
-        "qe_rmsnorm": [vp, vp, vp, vp, vp, i32, i32, f32, i32, vp],
+        "qe_rmsnorm": [vp, vp, i32, i32, i64, vp, vp, vp, i32, i32, f32, i32, vp],
         "qe_residual_add": [vp, vp, i64, i32, vp],
+        "qe_scatter_int": [vp, vp, vp, i32, i64, vp],
         "qe_silu_mul": [vp, vp, i32, i32, i32, vp],
-        "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp],
+        "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
+        "qe_gemm_partial_splits": [i32, i32],
         "qe_gemm_fused_supported": [i32, i32, i32, i32, i32],
         "qe_attention_decode_supported": [i32, i32, i32, i32, i32],
         "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
         "qe_qk_rope_store": [vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
-        "qe_argmax": [vp, vp, i32, i32, vp],
+        "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
         "qe_sample": [vp, vp, vp, vp, i32, i32, vp],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = ctypes.c_int
+    lib.qe_argmax_workspace_bytes.argtypes = [i32, i32]
+    lib.qe_argmax_workspace_bytes.restype = ctypes.c_long
     lib.qe_attention_decode_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]
     lib.qe_attention_decode_workspace_bytes.restype = ctypes.c_long
     _lib = lib
@@ -124,15 +128,22 @@ def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
     """RMSNorm of the 32-bit stream h [T, H] into out_dtype.
 
     With ``delta`` the residual sum h + delta is normed; it is written back to h
-    unless ``rows`` is given.  With ``rows`` (int32 [R]) only those rows are normed
-    and the result is [R, H].
+    unless ``rows`` is given.  delta is [T, H] in out_dtype, or float32 [S, T, H]:
+    partial products that are added in the order of S.  With ``rows`` (int32 [R])
+    only those rows are normed and the result is [R, H].
     """
     lib = load_library()
     _need(h, "h", torch.float32, (None, None))
     T, H = h.shape
     _need(weight, "weight", torch.float32, (H,), h.device)
+    n_delta, dt_d = 0, _DT[out_dtype]
     if delta is not None:
-        _need(delta, "delta", out_dtype, (T, H), h.device)
+        if delta.dim() == 3:
+            _need(delta, "delta", torch.float32, (None, T, H), h.device)
+            n_delta, dt_d = delta.shape[0], F32
+        else:
+            _need(delta, "delta", out_dtype, (T, H), h.device)
+            n_delta = 1
     n = T
     if rows is not None:
         _need(rows, "rows", torch.int32, (None,), h.device)
@@ -140,18 +151,30 @@ def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
     if out is None:
         out = torch.empty((n, H), dtype=out_dtype, device=h.device)
     _need(out, "out", out_dtype, (n, H), h.device)
-    _check(lib.qe_rmsnorm(h.data_ptr(), _ptr(delta), _ptr(rows), weight.data_ptr(), out.data_ptr(),
-                          n, H, float(eps), _DT[out_dtype], _stream()), "rmsnorm")
+    _check(lib.qe_rmsnorm(h.data_ptr(), _ptr(delta), n_delta, dt_d, T, _ptr(rows), weight.data_ptr(),
+                          out.data_ptr(), n, H, float(eps), _DT[out_dtype], _stream()), "rmsnorm")
     return out
 
 
 def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
-    """h += delta, h in 32-bit."""
+    """h += delta, h in 32-bit; delta [T, H], or float32 [S, T, H] partial products added in order."""
     lib = load_library()
     _need(h, "h", torch.float32)
-    _need(delta, "delta", _ACT, tuple(h.shape), h.device)
-    _check(lib.qe_residual_add(h.data_ptr(), delta.data_ptr(), h.numel(), _DT[delta.dtype], _stream()),
-           "residual_add")
+    parts = [delta] if delta.dim() == h.dim() else list(delta.unbind(0))
+    for d in parts:
+        _need(d, "delta", _ACT, tuple(h.shape), h.device)
+        _check(lib.qe_residual_add(h.data_ptr(), d.data_ptr(), h.numel(), _DT[d.dtype], _stream()),
+               "residual_add")
+
+
+def scatter_int(table: torch.Tensor, idx: torch.Tensor, val: torch.Tensor) -> None:
+    """table.flatten()[idx[i]] = val[i] wherever idx[i] >= 0 (int32).  The caller guarantees idx < table.numel()."""
+    lib = load_library()
+    _need(table, "table", torch.int32)
+    _need(idx, "idx", torch.int32, (None,), table.device)
+    _need(val, "val", torch.int32, (idx.shape[0],), table.device)
+    _check(lib.qe_scatter_int(table.data_ptr(), idx.data_ptr(), val.data_ptr(), idx.shape[0], table.numel(),
+                              _stream()), "scatter_int")
 
 
 def silu_mul(gu: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -177,12 +200,15 @@ def gemm_fused_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
 
 def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
          out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
-         algo: int = ALGO_AUTO, epilogue: int = EPI_STORE) -> torch.Tensor:
+         algo: int = ALGO_AUTO, epilogue: int = EPI_STORE, splits: int = 0) -> torch.Tensor:
     """x [M, K] . w [N, K]^T (+ bias [N], 32-bit) -> [M, N] in out_dtype (default: x's).
 
     epilogue EPI_RESIDUAL: the product is added into ``out``, the 32-bit stream [M, N].
     epilogue EPI_SILU_MUL: w is [2 N, K] (gate rows, then up rows); the result is
-    silu(x . gate^T) * (x . up^T), [M, N].  Both need gemm_fused_supported(x, w)."""
+    silu(x . gate^T) * (x . up^T), [M, N].
+    epilogue EPI_PARTIAL: the product is cut along K into ``splits`` (0: chosen for the shape)
+    partial products, returned as float32 [splits, M, N]; their sum over the first index, taken
+    in order, is the product.  All three need gemm_fused_supported(x, w)."""
     lib = load_library()
     _need(x, "x", _ACT, (None, None))
     M, K = x.shape
@@ -201,11 +227,17 @@ def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
             raise KernelError("gemm: the residual epilogue needs the stream to add into")
         out_dtype = torch.float32
     out_dtype = out_dtype or x.dtype
+    shape = (M, N)
+    if epilogue == EPI_PARTIAL:
+        splits = splits or lib.qe_gemm_partial_splits(N, K)
+        out_dtype, shape = torch.float32, (splits, M, N)
+    else:
+        splits = 1
     if out is None:
-        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
-    _need(out, "out", out_dtype, (M, N), x.device)
+        out = torch.empty(shape, dtype=out_dtype, device=x.device)
+    _need(out, "out", out_dtype, shape, x.device)
     _check(lib.qe_gemm(x.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), M, N, K,
-                       _DT[x.dtype], _DT[w.dtype], _DT[out_dtype], algo, epilogue, _stream()), "gemm")
+                       _DT[x.dtype], _DT[w.dtype], _DT[out_dtype], algo, epilogue, splits, _stream()), "gemm")
     return out
 
 
@@ -331,7 +363,9 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     if out is None:
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     _need(out, "out", torch.int32, (R,), logits.device)
-    _check(lib.qe_argmax(logits.data_ptr(), out.data_ptr(), R, V, _stream()), "argmax")
+    nbytes = lib.qe_argmax_workspace_bytes(R, V)
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=logits.device) if nbytes else None
+    _check(lib.qe_argmax(logits.data_ptr(), out.data_ptr(), R, V, _ptr(ws), nbytes, _stream()), "argmax")
     return out
 
 

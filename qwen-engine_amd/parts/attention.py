@@ -75,10 +75,8 @@ class PagedAttention:
             self.position.load({}, rt)
 
     # ---- one step -------------------------------------------------------------------
-    fuses_residual = True   # forward may add its output into the 32-bit stream itself
-
-    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding, residual: Optional[torch.Tensor] = None):
-        """Returns the mixer's output, or None after adding it into ``residual``."""
+    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding) -> torch.Tensor:
+        """Returns the mixer's output [T, H], or float32 partial products [S, T, H] of it."""
         if binding.kv is None:
             raise RuntimeError("attention was given no cache")
         T = x.shape[0]
@@ -107,9 +105,9 @@ class PagedAttention:
                           dec_tokens=ctx.dec_tokens, max_dec_position=ctx.max_dec_position,
                           other_tokens=ctx.other_tokens)
         o = o.view(T, self.hq * self.d)
-        if residual is not None and ops.gemm_fused_supported(o, self.w_o):
-            ops.gemm(o, self.w_o, out=residual, epilogue=ops.EPI_RESIDUAL)
-            return None
+        if ops.gemm_fused_supported(o, self.w_o):
+            # few rows: the product is cut along K to fill the chip; the norm that follows adds the parts
+            return ops.gemm(o, self.w_o, epilogue=ops.EPI_PARTIAL)
         return ops.gemm(o, self.w_o)
 
 

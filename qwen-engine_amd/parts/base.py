@@ -2,13 +2,14 @@
 model it is in: each gets its sizes and constants from its spec.
 
 Norm          forward(h, rt, delta=None, rows=None) -> x
-              h is the 32-bit residual stream [T, H]; with ``delta`` the sum h + delta
-              is normed and written back to h; with ``rows`` only those rows are normed.
+              h is the 32-bit residual stream [T, H]; with ``delta`` (a branch output, see
+              below) the sum h + delta is normed and written back to h; with ``rows`` only
+              those rows are normed.
 Mixer         forward(x, ctx, binding) -> y      x, y [T, H] in the activation type
               cache_need(spec) -> KVNeed | None, state_need(spec, hidden) -> StateNeed | None
 FeedForward   forward(x, ctx) -> y
-              A mixer or feed-forward with the class attribute ``fuses_residual = True`` is also
-              given ``residual=h`` and may add its output into h itself and return None.
+              A mixer's or feed-forward's y is [T, H] in the activation type, or float32 [S, T, H]:
+              partial products whose sum over S, taken in order, is the output (the norm adds them).
 Position      table() for the fused kernel, or apply(packed, positions, num_q, num_k) in place
               on a [T, Hq + 2 Hkv, D] tensor of q | k | v heads.
 """

@@ -43,16 +43,12 @@ class PreNormBlock:
 
     def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], ctx, binding: CacheBinding) -> torch.Tensor:
         """h: 32-bit residual stream (updated in place).  pending: branch output not yet
-        added to h, or None.  Returns the feed-forward output, to be added by whoever norms next,
-        or None when the feed-forward has added it itself."""
+        added to h, or None.  Returns the feed-forward output, to be added by whoever norms next.
+        A branch output is [T, H] in the activation type, or float32 [S, T, H]: partial products
+        that the norm adds in the order of S."""
         x = self.mixer_norm.forward(h, ctx.rt, delta=pending)
-        if getattr(self.mixer, "fuses_residual", False):
-            a = self.mixer.forward(x, ctx, binding, residual=h)    # None: already added into h
-        else:
-            a = self.mixer.forward(x, ctx, binding)
+        a = self.mixer.forward(x, ctx, binding)
         x = self.ffn_norm.forward(h, ctx.rt, delta=a)
-        if getattr(self.ffn, "fuses_residual", False):
-            return self.ffn.forward(x, ctx, residual=h)
         return self.ffn.forward(x, ctx)
 
 

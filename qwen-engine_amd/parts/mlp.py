@@ -35,17 +35,14 @@ class SwiGLU:
         self.w_gu = rt.place_matrix(torch.cat([g, u], dim=0))
         self.w_down = rt.place_matrix(tensors["down_proj.weight"])
 
-    fuses_residual = True   # forward may add its output into the 32-bit stream itself
-
-    def forward(self, x: torch.Tensor, ctx, residual: Optional[torch.Tensor] = None):
-        """Returns the feed-forward output, or None after adding it into ``residual``."""
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        """Returns the feed-forward output [T, H], or float32 partial products [S, T, H] of it."""
         if ops.gemm_fused_supported(x, self.w_gu):
             a = ops.gemm(x, self.w_gu, epilogue=ops.EPI_SILU_MUL)   # silu.mul in the product's epilogue
         else:
             a = ops.silu_mul(ops.gemm(x, self.w_gu))
-        if residual is not None and ops.gemm_fused_supported(a, self.w_down):
-            ops.gemm(a, self.w_down, out=residual, epilogue=ops.EPI_RESIDUAL)
-            return None
+        if ops.gemm_fused_supported(a, self.w_down):
+            return ops.gemm(a, self.w_down, epilogue=ops.EPI_PARTIAL)
         return ops.gemm(a, self.w_down)
 
 

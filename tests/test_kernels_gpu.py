@@ -254,6 +254,12 @@ def test_argmax_takes_the_lowest_index_on_ties(ops):
     assert got == P.greedy(logits)
     odd = rand(3, 331, seed=81)
     assert ops.argmax(odd.to(DEV)).cpu().tolist() == P.greedy(odd)
+    wide = rand(7, 151936, seed=85)                          # the two-stage form for wide vocabularies
+    wide[1, 2047] = wide[1, 2048] = wide[1, 151935] = 9.0    # ties across spans
+    wide[2, 151935] = 9.0
+    wide[3] = 1.5
+    got = ops.argmax(wide.to(DEV)).cpu().tolist()
+    assert got == P.greedy(wide) and got[1] == 2047 and got[2] == 151935 and got[3] == 0
 
 
 def test_temperature_sampling_is_the_inverse_cdf(ops):
@@ -321,6 +327,17 @@ def test_gemm_for_few_rows(ops, M, N, K):
     hd = h.to(DEV)
     ops.gemm(x.to(DEV), w.to(DEV), out=hd, epilogue=ops.EPI_RESIDUAL)
     close(hd, h.double() + want, torch.float32, scale=float(want.abs().max()))
+    # cut along K into partial products, which the norm adds up
+    for splits in (0, 1, 3):
+        parts = ops.gemm(x.to(DEV), w.to(DEV), epilogue=ops.EPI_PARTIAL, splits=splits)
+        assert parts.dtype == torch.float32 and parts.dim() == 3 and (splits == 0 or parts.shape[0] == splits)
+        close(parts.sum(0), want, torch.float32, scale=float(want.abs().max()))
+    hd = h.to(DEV)
+    nw = 1 + rand(N, seed=96, scale=0.1)
+    normed = ops.rmsnorm(hd, nw.to(DEV), 1e-6, bf, delta=parts)
+    total = h.double() + parts.double().cpu().sum(0)
+    close(hd, total, torch.float32)
+    close(normed, P.rms_norm(total.float(), nw, 1e-6), bf)
 
 
 @pytest.mark.parametrize("M", [1, 8, 40, 64])

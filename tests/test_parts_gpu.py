@@ -24,8 +24,9 @@ def close(got, want, dtype):
     assert err <= tol * s, f"error {err} beside scale {s}"
 
 
-def r16(x, dtype):
-    return x.to(dtype).float()
+def branch(y):
+    """A mixer's or feed-forward's output: [T, H], or float32 partial products [S, T, H]."""
+    return y.float().sum(0) if y.dim() == 3 else y.float()
 
 
 def one_request_context(rt, positions, page, num_pages, want_rows=()):
@@ -81,7 +82,7 @@ def test_swiglu_part(dtype):
          "down_proj.weight": rand(H, I, seed=5, scale=0.2, dtype=torch.bfloat16)}
     part.load(w, rt)
     x = rand(6, H, seed=6, dtype=dtype)
-    got = part.forward(x.to(DEV), None)
+    got = branch(part.forward(x.to(DEV), None))
     act = None if dtype == torch.float32 else dtype
     want = P.mlp_block(x.float(), {f"p.mlp.{k}": v for k, v in w.items()}, "p", act_dtype=act)
     close(got, want, dtype)
@@ -122,7 +123,7 @@ def test_attention_part_in_two_portions(dtype, bias, window):
         full = one_request_context(rt, list(range(0, T)), page, 12)
         ctx.block_tables = full.block_tables
         ctx.slots = [full.slots[0][a:b].contiguous()]
-        outs.append(part.forward(x[a:b].to(DEV), ctx, binding))
+        outs.append(branch(part.forward(x[a:b].to(DEV), ctx, binding)))
     cfg = dict(num_attention_heads=hq, num_key_value_heads=hkv, head_dim=d, rms_norm_eps=1e-5, attention_bias=bias)
     act = None if dtype == torch.float32 else dtype
     want = P.attention_block(x.float(), torch.arange(T), {f"p.self_attn.{k}": v for k, v in w.items()}, "p",
@@ -154,4 +155,4 @@ def test_block_part_defers_its_last_residual_sum(dtype):
     table = P.rope_table(cfg.rope_theta, cfg.head_dim, cfg.max_position_embeddings)
     h_in = h + pending.float()
     h_ref = P.decoder_layer(h_in, torch.arange(T), w, "model.layers.1", TINY_C, table, act_dtype=act)
-    close(hd.cpu() + out.float().cpu(), h_ref, dtype)       # stream + pending branch = the layer's output
+    close(hd.cpu() + branch(out).cpu(), h_ref, dtype)       # stream + pending branch = the layer's output
