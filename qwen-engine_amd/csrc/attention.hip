@@ -4,6 +4,7 @@
 //                       tokens of the batch or for a list of them
 // qe_attention_decode_* bfloat16 MFMA kernel for tokens that are the single new token of their
 //                       request (see attention_decode.hip)
+// qe_attention_prefill_run  bfloat16 MFMA kernel for portions of prompts (see attention_prefill.hip)
 #include "common.h"
 
 int qe_attention_generic(const void* q, void* out, const void* cache, const int* positions,
@@ -16,6 +17,21 @@ int qe_attention_decode(const void* q, void* out, const void* cache, const int* 
                         const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
                         int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
                         int split_keys, void* workspace, size_t workspace_bytes, hipStream_t stream);
+
+int qe_attention_prefill(const void* q, void* out, const void* cache, const int* tiles, int num_tiles,
+                         const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
+                         int Hq, int Hkv, int D, int P, float scale, int window, hipStream_t stream);
+
+// tiles: num_tiles pairs (first row of q, rows <= 16) of consecutive new tokens of one request.
+// Takes what qe_attention_decode_supported takes.
+extern "C" int qe_attention_prefill_run(const void* q, void* out, const void* cache, const int* tiles,
+                                        int num_tiles, const int* positions, const int* tok_seq,
+                                        const int* block_table, int max_blocks, int Hq, int Hkv, int D, int P,
+                                        float scale, int window, hipStream_t stream) {
+    QE_REQUIRE(num_tiles >= 0 && Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0, "prefill attention: bad sizes");
+    return qe_attention_prefill(q, out, cache, tiles, num_tiles, positions, tok_seq, block_table, max_blocks,
+                                Hq, Hkv, D, P, scale, window, stream);
+}
 
 // tokens: null for all T rows of q, else n_tokens row indices.
 extern "C" int qe_attention(const void* q, void* out, const void* cache, const int* positions,

@@ -1,46 +1,12 @@
 // Attention of single new tokens over the paged cache (decode), bfloat16, split over the keys
-// ("flash decoding"), on the MFMA units.  All query heads of a key/value group are computed by
-// one wave, so the cache is read from HBM once; this kernel is bound by that read.
+// ("flash decoding"), on the MFMA units.  All query heads of a key/value group are the columns
+// of one wave (see attention_tile.h), so the cache is read from HBM once; this kernel is bound
+// by that read.  Heads beyond the group size (lanes n >= G) compute on zeros and are not stored.
 //
-// One wave per (split of the keys, key/value head, token).  For each tile of 16 keys (a page
-// or a part of one; the page size is a multiple of 16):
-//   S^T[key, head] = K[key, :] . Q[head, :]          v_mfma_f32_16x16x32_bf16, D / 32 of them;
-//       lane (g, n), g = lane / 16, n = lane % 16, loads K[key n][c * 32 + g * 8 .. + 8] (16 bytes)
-//       and ends up with the scores of keys g * 4 .. g * 4 + 3 for head n
-//   online softmax per head n in 32-bit (max over the lane's 4 keys and the 4 lanes of the head)
-//   O^T[d, head] += V^T[d, key] . P^T[key, head]     v_mfma_f32_16x16x16_bf16, D / 16 of them;
-//       the probabilities a lane holds are exactly its B operand, and because value tiles are
-//       stored transposed ([D][P]) the A operand is one 8-byte load: V^T[d = db * 16 + n][keys g * 4 .. + 3]
-// No shared memory and no shuffles apart from the two of the max.  Heads beyond the group size
-// (lanes n >= G) compute on zeros and are not stored.
-//
-// The splits are cut at absolute key positions (multiples of split_keys), so a token's result
-// does not depend on what else is in the batch.  A second kernel merges the splits.
-#include "common.h"
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) short short4_t;
-typedef __attribute__((ext_vector_type(4))) float floatx4;
-
-__device__ __forceinline__ short bf16_bits(float f) { return (short)float_to_bf16(f).bits; }
-
-// One tile of 16 keys in registers: the K rows as MFMA A operands, the V^T rows likewise.
-template <int D>
-struct KVTile {
-    bf16x8 k[D / 32];
-    short4_t v[D / 16];
-};
-
-template <int D>
-__device__ __forceinline__ void load_tile(KVTile<D>& tile, const bf16_t* __restrict__ cache, long page,
-                                          long page_stride, int kvh, int Hkv, int P, int o, int g, int n) {
-    const bf16_t* kbase = cache + page * page_stride + ((long)kvh * P + o) * D + (long)n * D + g * 8;
-    const bf16_t* vbase = cache + page * page_stride + ((long)(Hkv + kvh) * P) * D + o + (long)n * P + g * 4;
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c) tile.k[c] = *(const bf16x8*)(kbase + c * 32);
-#pragma unroll
-    for (int db = 0; db < D / 16; ++db) tile.v[db] = *(const short4_t*)(vbase + (long)db * 16 * P);
-}
+// One wave per (split of the keys, key/value head, token).  The splits are cut at absolute key
+// positions (multiples of SPLIT), so a token's result does not depend on what else is in the
+// batch.  A second kernel merges the splits.
+#include "attention_tile.h"
 
 // SPLIT: keys per split (a multiple of 16).  The next tile is loaded while the current one is
 // computed, and the split's page ids are read before the loop.
@@ -85,10 +51,8 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     for (int c = 0; c < D / 32; ++c)
         qreg[c] = head_ok ? *(const bf16x8*)(q + ((long)t * Hq + head) * D + c * 32 + g * 8) : zero8;
 
-    float m = -INFINITY, l = 0.f;
-    floatx4 acc[D / 16];
-#pragma unroll
-    for (int db = 0; db < D / 16; ++db) acc[db] = floatx4{0.f, 0.f, 0.f, 0.f};
+    AttnState<D> st;
+    st.init();
 
     KVTile<D> cur, nxt;
     load_tile<D>(cur, cache, pages[tile0], page_stride, kvh, Hkv, P, (split * SPLIT + tile0 * 16) % P, g, n);
@@ -98,48 +62,17 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
         const int kk = split * SPLIT + i * 16;
         if (i + 1 < tile1)
             load_tile<D>(nxt, cache, pages[(i + 1 < TILES) ? i + 1 : i], page_stride, kvh, Hkv, P, (kk + 16) % P, g, n);
-
-        floatx4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int c = 0; c < D / 32; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[c], qreg[c], s, 0, 0, 0);
-        float tmax = -INFINITY;
-        bool ok[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int key = kk + g * 4 + j;
-            ok[j] = key >= k_begin && key < k_end;
-            s[j] = ok[j] ? s[j] * scale : -INFINITY;
-            tmax = fmaxf(tmax, s[j]);
-        }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float mn = fmaxf(m, tmax);        // finite: the tile holds at least one seen key
-        const float alpha = __expf(m - mn);
-        short4_t pb;
-        float psum = 0.f;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float pj = __expf(s[j] - mn);  // 0 for keys that are not seen
-            psum += pj;
-            pb[j] = bf16_bits(pj);
-        }
-        l = l * alpha + psum;
-        m = mn;
-        // values of unseen keys may be anything (an unwritten part of a page): keep them out
-        const short4_t vmask = {(short)(ok[0] ? -1 : 0), (short)(ok[1] ? -1 : 0), (short)(ok[2] ? -1 : 0), (short)(ok[3] ? -1 : 0)};
-#pragma unroll
-        for (int db = 0; db < D / 16; ++db) {
-            acc[db] *= alpha;
-            acc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(cur.v[db] & vmask, pb, acc[db], 0, 0, 0);
-        }
+        attn_tile_step<D>(st, cur, qreg, scale, kk, g, k_begin, k_end, k_begin, k_end);
         cur = nxt;
     }
+    float l = st.l;
+    const float m = st.m;
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (head_ok) {
 #pragma unroll
         for (int db = 0; db < D / 16; ++db)
-            *(floatx4*)(pacc + db * 16 + g * 4) = acc[db];    // O^T rows d = db * 16 + g * 4 + j of column head n
+            *(floatx4*)(pacc + db * 16 + g * 4) = st.acc[db];    // O^T rows d = db * 16 + g * 4 + j of column head n
         if (g == 0) { pml[0] = m; pml[1] = l; }
     }
 }

@@ -7,8 +7,11 @@ bool qe_gemm_skinny_ok(int M, int N, int K, int dt_a, int dt_w);
 int qe_gemm_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                    int dt_o, int epilogue, int splits, hipStream_t stream);
 int qe_gemm_skinny_splits(int N, int K);
+bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w);
+int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
+                 hipStream_t stream);
 
-enum { ALGO_AUTO = 0, ALGO_GENERIC = 1, ALGO_SKINNY = 2 };
+enum { ALGO_AUTO = 0, ALGO_GENERIC = 1, ALGO_MFMA = 2 };
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3 };
 
 // 1 if the fused epilogues (add into the 32-bit residual stream; silu(gate) * up) can be used
@@ -22,17 +25,23 @@ extern "C" int qe_gemm_partial_splits(int N, int K) { return qe_gemm_skinny_spli
 // out[M, N] = x[M, K] . w[N, K]^T (+ bias).  epilogue 0: store in dt_o.  1: add into out, the
 // 32-bit stream.  2: w is [2 N, K], gate rows then up rows; out = silu(x.gate^T) * (x.up^T).
 // 3: out is float [splits, M, N], partial products along K to be summed over the first index.
-// algo: 0 = choose, 1 = the generic 32-bit kernel, 2 = the MFMA kernel for few rows.
+// algo: 0 = choose, 1 = the generic 32-bit kernel, 2 = an MFMA kernel (the one for few rows up to
+// 64 rows, the tiled one above) or an error if neither takes the operands.
 extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                        int dt_a, int dt_w, int dt_o, int algo, int epilogue, int splits, hipStream_t stream) {
     QE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     if (M == 0) return 0;
     const bool skinny = qe_gemm_skinny_ok(M, N, K, dt_a, dt_w);
-    if (algo == ALGO_SKINNY || epilogue != EPI_STORE) {
+    const bool tiled = qe_gemm_mfma_ok(M, N, K, dt_a, dt_w);
+    if (epilogue != EPI_STORE) {
         QE_REQUIRE(skinny, "gemm: M=%d N=%d K=%d with these element types is not taken by the kernel for few rows", M, N, K);
         return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, epilogue, splits, stream);
     }
-    QE_REQUIRE(algo == ALGO_AUTO || algo == ALGO_GENERIC, "gemm: unknown algo %d", algo);
-    if (algo == ALGO_AUTO && skinny) return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, EPI_STORE, 1, stream);
+    QE_REQUIRE(algo == ALGO_AUTO || algo == ALGO_GENERIC || algo == ALGO_MFMA, "gemm: unknown algo %d", algo);
+    if (algo != ALGO_GENERIC) {
+        if (skinny) return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, EPI_STORE, 1, stream);
+        if (tiled) return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, stream);
+        QE_REQUIRE(algo == ALGO_AUTO, "gemm: M=%d N=%d K=%d with these element types is not taken by an MFMA kernel", M, N, K);
+    }
     return qe_gemm_generic(x, w, bias, out, M, N, K, dt_a, dt_w, dt_o, stream);
 }

@@ -38,4 +38,5 @@ class StepContext:
     # rows that are the single new token of their request, and all other rows (None: not split)
     dec_tokens: Optional[torch.Tensor] = None
     other_tokens: Optional[torch.Tensor] = None
+    other_tiles: Optional[torch.Tensor] = None     # int32 [tiles, 2]: the other rows cut into tiles of <= 16
     max_dec_position: int = 0

@@ -50,6 +50,7 @@ def load_library():
         "qe_gemm_partial_splits": [i32, i32],
         "qe_gemm_fused_supported": [i32, i32, i32, i32, i32],
         "qe_attention_decode_supported": [i32, i32, i32, i32, i32],
+        "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, vp],
         "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
         "qe_qk_rope_store": [vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
@@ -301,7 +302,8 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
               block_table: torch.Tensor, scale: float, window: int = 0,
               out: Optional[torch.Tensor] = None, algo: int = ALGO_AUTO,
               dec_tokens: Optional[torch.Tensor] = None, max_dec_position: int = 0,
-              other_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
+              other_tokens: Optional[torch.Tensor] = None,
+              other_tiles: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [T, Hq, D]; cache [pages, 2, Hkv, P, D] (key tiles [P][D], value tiles transposed [D][P]);
     positions, tok_seq int32 [T]; block_table int32 [B, max_blocks].  Token t sees the keys at
     positions max(0, p - window + 1) .. p of request tok_seq[t] (window 0: all).  The caller
@@ -309,7 +311,9 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
 
     dec_tokens (int32 rows of q that are the single new token of their request, the largest of
     their positions being max_dec_position) go to the decode kernel where it takes the sizes;
-    other_tokens are the remaining rows.  Without the two lists every row is treated alike."""
+    other_tokens are the remaining rows, and other_tiles (int32 [tiles, 2]: first row, number of
+    rows <= 16, consecutive tokens of one request) the same rows cut for the prefill kernel.
+    Without the lists every row is treated alike."""
     lib = load_library()
     _need(q, "q", _ACT, (None, None, None))
     T, Hq, D = q.shape
@@ -351,7 +355,15 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
             generic(dec_tokens)
     if other_tokens is not None and other_tokens.shape[0]:
         _need(other_tokens, "other_tokens", torch.int32, (None,), dev)
-        generic(other_tokens)
+        if other_tiles is not None and algo != ALGO_GENERIC and attention_decode_supported(q, cache):
+            _need(other_tiles, "other_tiles", torch.int32, (None, 2), dev)
+            _check(lib.qe_attention_prefill_run(q.data_ptr(), out.data_ptr(), cache.data_ptr(),
+                                                other_tiles.data_ptr(), other_tiles.shape[0],
+                                                positions.data_ptr(), tok_seq.data_ptr(), block_table.data_ptr(),
+                                                max_blocks, Hq, Hkv, D, P, float(scale), int(window), _stream()),
+                   "attention (prefill)")
+        else:
+            generic(other_tokens)
     return out
 
 

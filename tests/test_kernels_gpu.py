@@ -418,3 +418,85 @@ def test_decode_kernel_one_far_key_decides(ops, key_pos):
     want = P.attention(q.float(), k.float(), v.float(), 1 / math.sqrt(d))
     close(out, want, bf)
     assert float((want[0, 1] - v[key_pos, 0].float()).abs().max()) < 0.05
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 64, 64), (128, 128, 64), (200, 331, 96), (257, 500, 160), (2048, 1024, 1024),
+                                   (300, 3072, 1024), (130, 152, 2048)])
+def test_gemm_tiled_mfma(ops, M, N, K):
+    bf = torch.bfloat16
+    x, w = rand(M, K, seed=110, dtype=bf), rand(N, K, seed=111, dtype=bf, scale=0.1)
+    bias = rand(N, seed=112)
+    want = P.linear(x.double(), w.double())
+    got = ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_FAST)
+    close(got, want, bf)
+    got32 = ops.gemm(x.to(DEV), w.to(DEV), bias.to(DEV), out_dtype=torch.float32, algo=ops.ALGO_FAST)
+    close(got32, want + bias.double(), torch.float32, scale=float(want.abs().max()))
+    # the generic kernel on the same operands agrees to accumulation order
+    close(ops.gemm(x.to(DEV), w.to(DEV), out_dtype=torch.float32, algo=ops.ALGO_GENERIC), want, torch.float32,
+          scale=float(want.abs().max()))
+    with pytest.raises(ops.KernelError):
+        ops.gemm(torch.zeros(100, 76, dtype=bf, device=DEV), torch.zeros(8, 76, dtype=bf, device=DEV), algo=ops.ALGO_FAST)
+
+
+@pytest.mark.parametrize("hq,hkv,d,page", [(16, 8, 128, 16), (4, 4, 64, 16), (8, 1, 128, 32), (6, 2, 64, 64)])
+@pytest.mark.parametrize("window", [0, 40])
+def test_prefill_attention_kernel(ops, hq, hkv, d, page, window):
+    """Three requests in one batch: a whole prompt of 75 tokens, a portion of 37 tokens after 100
+    cached ones, and one of 2 tokens after 15; beside a decoded token.  Pages shuffled, unwritten
+    parts of pages NaN."""
+    bf = torch.bfloat16
+    scale = 1 / math.sqrt(d)
+    lens = [(0, 75), (100, 37), (15, 2), (33, 1)]
+    qs, pos, seq, tables, caches, want, tiles, dec, other = [], [], [], [], [], [], [], [], []
+    base, row = 0, 0
+    for b, (before, n) in enumerate(lens):
+        L = before + n
+        k, v = rand(L, hkv, d, seed=120 + b, dtype=bf), rand(L, hkv, d, seed=130 + b, dtype=bf)
+        q = rand(n, hq, d, seed=140 + b, dtype=bf)
+        cache, ids = paged_cache(k, v, page, 150 + b, bf)
+        tables.append(ids + base)
+        base += cache.shape[0]
+        caches.append(cache)
+        qs.append(q)
+        pos += list(range(before, L))
+        seq += [b] * n
+        want.append(P.attention(q.float(), k.float(), v.float(), scale, window=window or None))
+        if n == 1:
+            dec.append(row)
+        else:
+            other += list(range(row, row + n))
+            tiles += [[row + r, min(16, n - r)] for r in range(0, n, 16)]
+        row += n
+    width = max(len(t) for t in tables)
+    table = torch.full((len(lens), width), -1, dtype=torch.int32)
+    for b, t in enumerate(tables):
+        table[b, :len(t)] = t
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    out = ops.attention(torch.cat(qs).to(DEV), torch.cat(caches).to(DEV), i32(pos), i32(seq), table.to(DEV), scale,
+                        window=window, dec_tokens=i32(dec), max_dec_position=33, other_tokens=i32(other),
+                        other_tiles=i32(tiles))
+    assert not torch.isnan(out.float()).any()
+    close(out, torch.cat(want), bf)
+
+
+@pytest.mark.parametrize("key_pos", [0, 15, 16, 200, 255, 256, 299])
+def test_prefill_kernel_one_far_key_decides(ops, key_pos):
+    """Rows 256..299 of a request; the row at position 299 (and every row at or after the key)
+    returns the value of the one key that stands out."""
+    bf = torch.bfloat16
+    hq, hkv, d, L, page, first = 2, 1, 128, 300, 16, 256
+    k = rand(L, hkv, d, seed=160, dtype=bf, scale=0.1)
+    v = rand(L, hkv, d, seed=161, dtype=bf)
+    direction = rand(d, seed=162)
+    q = (direction[None, None, :] + 0.05 * rand(L - first, hq, d, seed=163)).to(bf)
+    k[key_pos, 0] = (direction * 4).to(bf)
+    cache, ids = paged_cache(k, v, page, 164, bf)
+    n = L - first
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    tiles = [[r, min(16, n - r)] for r in range(0, n, 16)]
+    out = ops.attention(q.to(DEV), cache.to(DEV), i32(list(range(first, L))), i32([0] * n), ids[None].to(DEV),
+                        1 / math.sqrt(d), dec_tokens=i32([]), other_tokens=i32(list(range(n))), other_tiles=i32(tiles))
+    want = P.attention(q.float(), k.float(), v.float(), 1 / math.sqrt(d))
+    close(out, want, bf)
+    last_seen = max(key_pos, first) - first
+    assert float((want[last_seen:, 0] - v[key_pos, 0].float()).abs().max()) < 0.05
