@@ -63,6 +63,99 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ del
     }
 }
 
+// The same for rows of up to NV * 4 * blockDim.x elements with H % 4 == 0: the row is read once
+// (16-byte loads, all in flight together) and kept in registers.  This is the kernel of decode
+// steps, where a launch has few rows and its time is the latency of its memory accesses.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+        const float4 t = *(const float4*)p;
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+        *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+    }
+};
+template <> struct Vec4<bf16_t> {
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+        const uint2 t = *(const uint2*)p;
+        v[0] = bf16_bits_to_float(t.x & 0xffffu); v[1] = bf16_bits_to_float(t.x >> 16);
+        v[2] = bf16_bits_to_float(t.y & 0xffffu); v[3] = bf16_bits_to_float(t.y >> 16);
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+        uint2 t;
+        t.x = (uint32_t)float_to_bf16(v[0]).bits | ((uint32_t)float_to_bf16(v[1]).bits << 16);
+        t.y = (uint32_t)float_to_bf16(v[2]).bits | ((uint32_t)float_to_bf16(v[3]).bits << 16);
+        *(uint2*)p = t;
+    }
+};
+
+template <typename TA, typename TD, int NV>
+__global__ void rmsnorm_regs_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_delta, long delta_stride,
+                                    const int* __restrict__ rows, const float* __restrict__ w,
+                                    TA* __restrict__ out, int H, float eps) {
+    __shared__ float red[16];
+    const long r = blockIdx.x;
+    const long src = rows ? (long)rows[r] : r;
+    float* hr = h + src * H;
+    const TD* dr = delta ? delta + src * H : nullptr;
+    float v[NV][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = (threadIdx.x + i * blockDim.x) * 4;
+        if (c < H) {
+            Vec4<float>::load(hr + c, v[i]);
+            if (dr) {
+#pragma unroll 4
+                for (int s = 0; s < n_delta; ++s) {
+                    float d[4];
+                    Vec4<TD>::load(dr + s * delta_stride + c, d);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[i][e] += d[e];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ss += v[i][e] * v[i][e];
+        }
+    }
+    ss = block_sum(ss, red);
+    const float rstd = rsqrtf(ss / (float)H + eps);
+    const bool write_back = dr && !rows;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = (threadIdx.x + i * blockDim.x) * 4;
+        if (c < H) {
+            if (write_back) Vec4<float>::store(hr + c, v[i]);
+            float wv[4], o[4];
+            Vec4<float>::load(w + c, wv);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = v[i][e] * rstd * wv[e];
+            Vec4<TA>::store(out + r * H + c, o);
+        }
+    }
+}
+
+template <typename TA, typename TD>
+static void launch_rmsnorm(float* h, const void* delta, int n_delta, long stride, const int* rows, const float* w,
+                           void* out, int n_out_rows, int H, float eps, hipStream_t stream) {
+    if (H % 4 == 0 && H <= 8192) {
+        int threads = ((H / 4 + 63) / 64) * 64;
+        if (threads > 256) threads = 256;
+        const int nv = (H / 4 + threads - 1) / threads;
+#define QE_NORM(NV_) rmsnorm_regs_kernel<TA, TD, NV_><<<n_out_rows, threads, 0, stream>>>( \
+        h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps)
+        if (nv <= 1) QE_NORM(1);
+        else if (nv <= 2) QE_NORM(2);
+        else if (nv <= 4) QE_NORM(4);
+        else QE_NORM(8);
+#undef QE_NORM
+        return;
+    }
+    const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
+    rmsnorm_kernel<TA, TD><<<n_out_rows, threads, 0, stream>>>(h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps);
+}
+
 // dt_d: element type of delta (that of the output, or float for partial products)
 extern "C" int qe_rmsnorm(float* h, const void* delta, int n_delta, int dt_d, long n_rows_h, const int* rows,
                           const float* w, void* out, int n_out_rows, int H, float eps, int dt_a,
@@ -70,14 +163,13 @@ extern "C" int qe_rmsnorm(float* h, const void* delta, int n_delta, int dt_d, lo
     QE_REQUIRE(n_out_rows >= 0 && H > 0, "rmsnorm: bad sizes rows=%d H=%d", n_out_rows, H);
     QE_REQUIRE(!delta || n_delta >= 1, "rmsnorm: %d delta tensors", n_delta);
     if (n_out_rows == 0) return 0;
-    const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
     const long stride = n_rows_h * H;
     if (dt_a == QE_F32 && (!delta || dt_d == QE_F32))
-        rmsnorm_kernel<float, float><<<n_out_rows, threads, 0, stream>>>(h, (const float*)delta, n_delta, stride, rows, w, (float*)out, H, eps);
+        launch_rmsnorm<float, float>(h, delta, n_delta, stride, rows, w, out, n_out_rows, H, eps, stream);
     else if (dt_a == QE_BF16 && (!delta || dt_d == QE_BF16))
-        rmsnorm_kernel<bf16_t, bf16_t><<<n_out_rows, threads, 0, stream>>>(h, (const bf16_t*)delta, n_delta, stride, rows, w, (bf16_t*)out, H, eps);
+        launch_rmsnorm<bf16_t, bf16_t>(h, delta, n_delta, stride, rows, w, out, n_out_rows, H, eps, stream);
     else if (dt_a == QE_BF16 && dt_d == QE_F32)
-        rmsnorm_kernel<bf16_t, float><<<n_out_rows, threads, 0, stream>>>(h, (const float*)delta, n_delta, stride, rows, w, (bf16_t*)out, H, eps);
+        launch_rmsnorm<bf16_t, float>(h, delta, n_delta, stride, rows, w, out, n_out_rows, H, eps, stream);
     else
         QE_REQUIRE(false, "rmsnorm: no kernel for output type %d with delta type %d", dt_a, dt_d);
     QE_LAUNCH_CHECK();

@@ -46,7 +46,7 @@ def test_embedding(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H", [80, 1024, 3000])
+@pytest.mark.parametrize("H", [77, 80, 1024, 3000, 9000])
 def test_rmsnorm_plain_fused_and_gathered(ops, dtype, H):
     h = rand(7, H, seed=2, scale=3.0)
     w = 1 + rand(H, seed=3, scale=0.1)
