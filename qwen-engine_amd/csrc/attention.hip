@@ -22,8 +22,16 @@ int qe_attention_prefill(const void* q, void* out, const void* cache, const int*
                          const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
                          int Hq, int Hkv, int D, int P, float scale, int window, hipStream_t stream);
 
-// tiles: num_tiles pairs (first row of q, rows <= 16) of consecutive new tokens of one request.
-// Takes what qe_attention_decode_supported takes.
+int qe_attention_prefill_tile_rows(int Hq, int Hkv);
+
+// rows of a tile for these head counts
+extern "C" int qe_attention_prefill_rows(int Hq, int Hkv) {
+    if (Hq <= 0 || Hkv <= 0 || Hq % Hkv) return 0;
+    return qe_attention_prefill_tile_rows(Hq, Hkv);
+}
+
+// tiles: num_tiles pairs (first row of q, rows <= qe_attention_prefill_rows) of consecutive new
+// tokens of one request.  Takes what qe_attention_decode_supported takes.
 extern "C" int qe_attention_prefill_run(const void* q, void* out, const void* cache, const int* tiles,
                                         int num_tiles, const int* positions, const int* tok_seq,
                                         const int* block_table, int max_blocks, int Hq, int Hkv, int D, int P,

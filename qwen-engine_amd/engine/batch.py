@@ -38,5 +38,18 @@ class StepContext:
     # rows that are the single new token of their request, and all other rows (None: not split)
     dec_tokens: Optional[torch.Tensor] = None
     other_tokens: Optional[torch.Tensor] = None
-    other_tiles: Optional[torch.Tensor] = None     # int32 [tiles, 2]: the other rows cut into tiles of <= 16
+    _tiles: dict = field(default_factory=dict)
     max_dec_position: int = 0
+
+    def other_tiles(self, rows_per_tile: int) -> Optional[torch.Tensor]:
+        """The rows of requests that bring several tokens, cut into tiles of at most
+        ``rows_per_tile`` consecutive rows of one request: int32 [tiles, 2] = (first row, rows).
+        Built and sent to the device once per step and tile size."""
+        if rows_per_tile <= 0:
+            return None
+        if rows_per_tile not in self._tiles:
+            flat = [v for s in self.seqs if s.q_len > 1 for r in range(0, s.q_len, rows_per_tile)
+                    for v in (s.q_start + r, min(rows_per_tile, s.q_len - r))]
+            t = torch.tensor(flat, dtype=torch.int32).view(-1, 2)
+            self._tiles[rows_per_tile] = t.to(self.rt.device) if flat else None
+        return self._tiles[rows_per_tile]

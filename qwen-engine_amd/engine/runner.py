@@ -198,9 +198,7 @@ class ModelRunner:
         dec_rows = [s.q_start for s in seqs if s.q_len == 1]
         other_rows = [s.q_start + i for s in seqs if s.q_len > 1 for i in range(s.q_len)]
         max_dec = max([s.kv_before for s in seqs if s.q_len == 1], default=0)
-        tiles = [v for s in seqs if s.q_len > 1 for r in range(0, s.q_len, 16)
-                 for v in (s.q_start + r, min(16, s.q_len - r))]
-        parts = [token_ids, positions, tok_seq, rows, [s.state_slot for s in seqs], dec_rows, other_rows, tiles]
+        parts = [token_ids, positions, tok_seq, rows, [s.state_slot for s in seqs], dec_rows, other_rows]
         for g in range(n_groups):
             parts += [slots[g], upd_idx[g], upd_val[g]]
         flat = [v for part in parts for v in part]
@@ -217,7 +215,6 @@ class ModelRunner:
         d_tok, d_pos, d_seq = take(T), take(T), take(T)
         d_rows, d_state = take(len(rows)), take(B)
         d_dec, d_other = take(len(dec_rows)), take(len(other_rows))
-        d_tiles = take(len(tiles)).view(-1, 2)
         d_slots = []
         for g in range(n_groups):
             d_slots.append(take(T))
@@ -228,8 +225,7 @@ class ModelRunner:
         return StepContext(rt=self.rt, page_size=self.page_size, num_tokens=T, seqs=seqs, token_ids=d_tok,
                            positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
                            logit_rows=d_rows, state_slots=d_state, max_position=max(positions),
-                           dec_tokens=d_dec, other_tokens=d_other, other_tiles=d_tiles,
-                           max_dec_position=max_dec)
+                           dec_tokens=d_dec, other_tokens=d_other, max_dec_position=max_dec)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Runs the entries' tokens as one batch; returns float32 logits [wanted, vocab] on the

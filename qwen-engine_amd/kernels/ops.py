@@ -50,6 +50,7 @@ def load_library():
         "qe_gemm_partial_splits": [i32, i32],
         "qe_gemm_fused_supported": [i32, i32, i32, i32, i32],
         "qe_attention_decode_supported": [i32, i32, i32, i32, i32],
+        "qe_attention_prefill_rows": [i32, i32],
         "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, vp],
         "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
         "qe_qk_rope_store": [vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
@@ -298,6 +299,11 @@ def attention_decode_supported(q: torch.Tensor, cache: torch.Tensor) -> bool:
                                                   _DT[q.dtype]))
 
 
+def prefill_tile_rows(num_heads: int, num_kv_heads: int) -> int:
+    """Rows of a tile of the prefill attention kernel for these head counts (``other_tiles``)."""
+    return load_library().qe_attention_prefill_rows(num_heads, num_kv_heads)
+
+
 def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
               block_table: torch.Tensor, scale: float, window: int = 0,
               out: Optional[torch.Tensor] = None, algo: int = ALGO_AUTO,
@@ -312,7 +318,8 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
     dec_tokens (int32 rows of q that are the single new token of their request, the largest of
     their positions being max_dec_position) go to the decode kernel where it takes the sizes;
     other_tokens are the remaining rows, and other_tiles (int32 [tiles, 2]: first row, number of
-    rows <= 16, consecutive tokens of one request) the same rows cut for the prefill kernel.
+    rows <= prefill_tile_rows(Hq, Hkv), consecutive tokens of one request) the same rows cut
+    for the prefill kernel.
     Without the lists every row is treated alike."""
     lib = load_library()
     _need(q, "q", _ACT, (None, None, None))

@@ -103,7 +103,8 @@ class PagedAttention:
                                   None, slots, cache, ctx.page_size)
         o = ops.attention(q, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g], self.scale, self.window,
                           dec_tokens=ctx.dec_tokens, max_dec_position=ctx.max_dec_position,
-                          other_tokens=ctx.other_tokens, other_tiles=ctx.other_tiles)
+                          other_tokens=ctx.other_tokens,
+                          other_tiles=ctx.other_tiles(ops.prefill_tile_rows(self.hq, self.hkv)))
         o = o.view(T, self.hq * self.d)
         if ops.gemm_fused_supported(o, self.w_o):
             # few rows: the product is cut along K to fill the chip; the norm that follows adds the parts

@@ -438,8 +438,8 @@ def test_gemm_tiled_mfma(ops, M, N, K):
         ops.gemm(torch.zeros(100, 76, dtype=bf, device=DEV), torch.zeros(8, 76, dtype=bf, device=DEV), algo=ops.ALGO_FAST)
 
 
-@pytest.mark.parametrize("hq,hkv,d,page", [(16, 8, 128, 16), (4, 4, 64, 16), (8, 1, 128, 32), (6, 2, 64, 64)])
-@pytest.mark.parametrize("window", [0, 40])
+@pytest.mark.parametrize("hq,hkv,d,page", [(16, 8, 128, 16), (4, 4, 64, 16), (8, 1, 128, 32), (6, 2, 64, 64), (8, 2, 128, 48)])
+@pytest.mark.parametrize("window", [0, 40, 17])
 def test_prefill_attention_kernel(ops, hq, hkv, d, page, window):
     """Three requests in one batch: a whole prompt of 75 tokens, a portion of 37 tokens after 100
     cached ones, and one of 2 tokens after 15; beside a decoded token.  Pages shuffled, unwritten
@@ -449,6 +449,8 @@ def test_prefill_attention_kernel(ops, hq, hkv, d, page, window):
     lens = [(0, 75), (100, 37), (15, 2), (33, 1)]
     qs, pos, seq, tables, caches, want, tiles, dec, other = [], [], [], [], [], [], [], [], []
     base, row = 0, 0
+    R = ops.prefill_tile_rows(hq, hkv)
+    assert R == 32 // (hq // hkv) if (hq // hkv) in (1, 2, 4, 8, 16, 32) else R == 32
     for b, (before, n) in enumerate(lens):
         L = before + n
         k, v = rand(L, hkv, d, seed=120 + b, dtype=bf), rand(L, hkv, d, seed=130 + b, dtype=bf)
@@ -465,7 +467,7 @@ def test_prefill_attention_kernel(ops, hq, hkv, d, page, window):
             dec.append(row)
         else:
             other += list(range(row, row + n))
-            tiles += [[row + r, min(16, n - r)] for r in range(0, n, 16)]
+            tiles += [[row + r, min(R, n - r)] for r in range(0, n, R)]
         row += n
     width = max(len(t) for t in tables)
     table = torch.full((len(lens), width), -1, dtype=torch.int32)
@@ -493,7 +495,8 @@ def test_prefill_kernel_one_far_key_decides(ops, key_pos):
     cache, ids = paged_cache(k, v, page, 164, bf)
     n = L - first
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
-    tiles = [[r, min(16, n - r)] for r in range(0, n, 16)]
+    R = ops.prefill_tile_rows(hq, hkv)
+    tiles = [[r, min(R, n - r)] for r in range(0, n, R)]
     out = ops.attention(q.to(DEV), cache.to(DEV), i32(list(range(first, L))), i32([0] * n), ids[None].to(DEV),
                         1 / math.sqrt(d), dec_tokens=i32([]), other_tokens=i32(list(range(n))), other_tiles=i32(tiles))
     want = P.attention(q.float(), k.float(), v.float(), 1 / math.sqrt(d))
