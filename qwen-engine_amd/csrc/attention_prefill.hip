@@ -68,51 +68,86 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[db][e] = 0.f;
 
-    for (int kk = (k_start / 32) * 32; kk < k_stop; kk += 32) {
-        // the two halves of 16 keys: their pages and offsets.  A half that no row sees (beyond the
-        // request's keys, or wholly behind the window, where the page may have been given back)
-        // reads the other half's memory again and is masked out.
-        const bool first = kk + 16 > k_start, second = kk + 16 < k_stop;
-        const int ka = first ? kk : kk + 16;
-        const int kb = second ? kk + 16 : kk;
-        const long base_a = (long)bt[ka / P] * page_stride, base_b = (long)bt[kb / P] * page_stride;
-        const int off_a = ka % P, off_b = kb % P;
-        const long kbase = ((r < 16) ? base_a + ((long)kvh * P + off_a + r) * D
-                                     : base_b + ((long)kvh * P + off_b + r - 16) * D) + g * 8;
-        bf16x8 kreg[D / 16];
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) kreg[ks] = *(const bf16x8*)(cache + kbase + ks * 16);
-        PackV vreg[D / 32][2];
-        const long vb_a = base_a + ((long)(Hkv + kvh) * P) * D + off_a + 4 * g;
-        const long vb_b = base_b + ((long)(Hkv + kvh) * P) * D + off_b + 4 * g;
-#pragma unroll
-        for (int db = 0; db < D / 32; ++db) {
-            const long drow = (long)(db * 32 + r) * P;
-            vreg[db][0].u[0] = *(const uint2*)(cache + vb_a + drow);
-            vreg[db][0].u[1] = *(const uint2*)(cache + vb_a + drow + 8);
-            vreg[db][1].u[0] = *(const uint2*)(cache + vb_b + drow);
-            vreg[db][1].u[1] = *(const uint2*)(cache + vb_b + drow + 8);
-        }
+    // what a lane adds to a page's base to reach its piece of a key tile and of a value tile
+    const long k_lane = ((long)kvh * P + (r & 15)) * D + g * 8;
+    const long v_lane = ((long)(Hkv + kvh) * P) * D + (long)r * P + 4 * g;
+    const long v_step = 32L * P;                          // from one block of 32 value rows to the next
+    // keys every column sees without a limit: [all_lo, all_hi); a tile inside needs no masks
+    const int p_last = p_first + cnt - 1;
+    const int all_hi = p_first + 1;
+    const int all_lo = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
 
+    // A 32-key tile has two halves of 16 keys with pages and offsets of their own.  A half that no
+    // row sees (beyond the request's keys, or wholly behind the window, where the page may have
+    // been given back) reads the other half's memory again and is masked out.
+#define TILE_ADDR(kk_)                                                                              \
+    const bool first_ = (kk_) + 16 > k_start, second_ = (kk_) + 16 < k_stop;                        \
+    const int ka_ = first_ ? (kk_) : (kk_) + 16;                                                    \
+    const int kb_ = second_ ? (kk_) + 16 : (kk_);                                                   \
+    const long base_a = (long)bt[ka_ / P] * page_stride + (long)(ka_ % P) * D;                      \
+    const long base_b = (long)bt[kb_ / P] * page_stride + (long)(kb_ % P) * D;                      \
+    const long vbase_a = (long)bt[ka_ / P] * page_stride + (ka_ % P);                               \
+    const long vbase_b = (long)bt[kb_ / P] * page_stride + (kb_ % P);
+#define LOAD_K()                                                                                    \
+    {                                                                                               \
+        const bf16_t* kp = cache + ((r < 16) ? base_a : base_b) + k_lane;                           \
+        _Pragma("unroll") for (int ks = 0; ks < D / 16; ++ks) kreg[ks] = *(const bf16x8*)(kp + ks * 16); \
+    }
+
+    bf16x8 kreg[D / 16];
+    const int kk0 = (k_start / 32) * 32;
+    {
+        TILE_ADDR(kk0)
+        LOAD_K()
+        (void)vbase_a; (void)vbase_b;
+    }
+    for (int kk = kk0; kk < k_stop; kk += 32) {
+        PackV vreg[D / 32][2];
+        {
+            TILE_ADDR(kk)
+            const bf16_t* va = cache + vbase_a + v_lane;
+            const bf16_t* vb = cache + vbase_b + v_lane;
+            (void)base_a; (void)base_b;
+#pragma unroll
+            for (int db = 0; db < D / 32; ++db) {
+                vreg[db][0].u[0] = *(const uint2*)(va + db * v_step);
+                vreg[db][0].u[1] = *(const uint2*)(va + db * v_step + 8);
+                vreg[db][1].u[0] = *(const uint2*)(vb + db * v_step);
+                vreg[db][1].u[1] = *(const uint2*)(vb + db * v_step + 8);
+            }
+        }
         floatx16 s;
 #pragma unroll
         for (int e = 0; e < 16; ++e) s[e] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks)
             s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kreg[ks], qreg[ks], s, 0, 0, 0);
+        if (kk + 32 < k_stop) {   // the next tile's keys travel while this tile's softmax and values are computed
+            TILE_ADDR(kk + 32)
+            LOAD_K()
+            (void)vbase_a; (void)vbase_b;
+        }
 
         float tmax = -INFINITY;
+        if (kk >= all_lo && kk + 32 <= all_hi) {           // every column sees every key of the tile
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int key = kk + 8 * (e >> 2) + 4 * g + (e & 3);
-            s[e] = (key >= lo && key < hi) ? s[e] * scale_log2 : -INFINITY;
-            tmax = fmaxf(tmax, s[e]);
+            for (int e = 0; e < 16; ++e) {
+                s[e] *= scale_log2;
+                tmax = fmaxf(tmax, s[e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int key = kk + 8 * (e >> 2) + 4 * g + (e & 3);
+                s[e] = (key >= lo && key < hi) ? s[e] * scale_log2 : -INFINITY;
+                tmax = fmaxf(tmax, s[e]);
+            }
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
         const float mn = fmaxf(m, tmax);
         const float ref = (mn == -INFINITY) ? 0.f : mn;    // a column that has seen no key yet: all weights 0
         if (__any(mn > m)) {                               // some column's maximum moved: rescale
-            const float alpha = exp2f(m - ref);
+            const float alpha = __builtin_amdgcn_exp2f(m - ref);
             l *= alpha;
 #pragma unroll
             for (int db = 0; db < D / 32; ++db) acc[db] *= alpha;
@@ -122,7 +157,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
         float psum = 0.f;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const float pe = exp2f(s[e] - ref);            // 0 for keys that are not seen
+            const float pe = __builtin_amdgcn_exp2f(s[e] - ref);   // 0 for keys that are not seen
             psum += pe;
             pb[e >> 3].v[e & 7] = (__bf16)pe;
         }
@@ -146,6 +181,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
             for (int h = 0; h < 2; ++h)
                 acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vreg[db][h].v, pb[h].v, acc[db], 0, 0, 0);
     }
+#undef TILE_ADDR
+#undef LOAD_K
     l += __shfl_xor(l, 32, 64);
     if (col_ok) {
         const float inv = 1.f / l;

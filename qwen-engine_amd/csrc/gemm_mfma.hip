@@ -1,8 +1,9 @@
 // Matrix product for many rows of activations (prefill): out[M, N] = x[M, K] . W[N, K]^T (+ bias),
 // bfloat16 in, 32-bit accumulation with v_mfma_f32_32x32x16_bf16, output bfloat16 or float32.
 //
-// A block of 256 threads (4 waves, 2 x 2) computes a 128 x 128 tile of the output; each wave
-// a 64 x 64 quarter as 2 x 2 MFMA tiles.  K is walked in steps of 64 through shared memory with
+// A block of 256 threads (4 waves, 2 x 2) computes a TM x 128 tile of the output, TM = 128 or 64
+// (the smaller one when the larger would leave compute units without a block); each wave
+// a quarter as (TM / 64) x 2 MFMA tiles.  K is walked in steps of 64 through shared memory with
 // two buffers: while the MFMAs of one step run, the 16-byte global loads of the next are in
 // flight.  Both operands are K-contiguous in memory, so they are staged alike: a row of 64
 // bfloat16 (128 bytes) is padded to 144 bytes, which makes the 16-byte fragment reads of the
@@ -18,12 +19,11 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float floatx16;
 typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
 
-#define BM 128
 #define BN 128
 #define BK 64
 #define ROWB 144   // bytes of a staged row: 128 of data + 16 of padding
 
-template <typename TO>
+template <typename TO, int BM>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TO* __restrict__ out, int M, int N, int K, int tiles_m) {
@@ -32,15 +32,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    constexpr int WM = BM / 2;         // rows of a wave's part
+    constexpr int MI = WM / 32;        // MFMA tiles along m per wave
+    constexpr int LD = (BM + BN) / 32; // 16-byte pieces a thread stages per step
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * 64;
 
-    // global -> shared: a step has (BM + BN) rows x 8 pieces of 16 bytes = 2048 pieces, 8 per thread
+    // global -> shared: a step has (BM + BN) rows x 8 pieces of 16 bytes, LD per thread
     // piece q = tid + 256 * i: row = q / 8, piece-in-row = q % 8
     const int nk = (K + BK - 1) / BK;
-    uint4_t stage[8];
+    uint4_t stage[LD];
 
 #define LOAD_GLOBAL(kt_)                                                                 \
-    _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                      \
+    _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                     \
         const int q = tid + 256 * i;                                                     \
         const int row = q >> 3, pc = q & 7;                                              \
         const int k = (kt_) * BK + pc * 8;                                               \
@@ -52,15 +55,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
         stage[i] = ok ? v : uint4_t{0u, 0u, 0u, 0u};                                     \
     }
 #define STORE_SHARED(buf_)                                                               \
-    _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                      \
+    _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                      \
         const int q = tid + 256 * i;                                                     \
         const int row = q >> 3, pc = q & 7;                                              \
         *(uint4_t*)(smem + (buf_) * (BM + BN) * ROWB + row * ROWB + pc * 16) = stage[i]; \
     }
 
-    floatx16 acc[2][2];
+    floatx16 acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -78,13 +81,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
         const unsigned char* b_base = smem + buf * (BM + BN) * ROWB + (BM + wn + fr) * ROWB + fk;
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 a[2], b[2];
+            bf16x8 a[MI], b[2];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) a[i] = *(const bf16x8*)(a_base + i * 32 * ROWB + ks * 32);
+            for (int i = 0; i < MI; ++i) a[i] = *(const bf16x8*)(a_base + i * 32 * ROWB + ks * 32);
 #pragma unroll
             for (int j = 0; j < 2; ++j) b[j] = *(const bf16x8*)(b_base + j * 32 * ROWB + ks * 32);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
@@ -96,7 +99,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
     // C of a 32x32 MFMA: lane holds column (lane % 32), rows 8 * b + 4 * (lane / 32) + r for e = 4 * b + r.
     // With A = x rows and B = W rows that is: token row m, output column n = lane % 32.
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int n = n0 + wn + j * 32 + (lane & 31);
@@ -114,22 +117,31 @@ bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w) {
     return dt_a == QE_BF16 && dt_w == QE_BF16 && M > 64 && K % 8 == 0 && K >= 64;
 }
 
-int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
-                 hipStream_t stream) {
-    QE_REQUIRE(K % 8 == 0, "mfma gemm: K=%d is no multiple of 8", K);
+template <typename TO, int BM>
+static int launch_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
+                       hipStream_t stream) {
     const int tiles_m = qe_cdiv(M, BM), tiles_n = qe_cdiv(N, BN);
     const long blocks = (long)tiles_m * tiles_n;
     QE_REQUIRE(blocks <= 2147483647L, "mfma gemm: too many tiles");
     const size_t shmem = 2 * (BM + BN) * ROWB;
-    if (dt_o == QE_BF16) {
-        static bool set16 = false;
-        if (!set16) { (void)hipFuncSetAttribute((const void*)gemm_mfma_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem); set16 = true; }
-        gemm_mfma_kernel<bf16_t><<<(int)blocks, 256, shmem, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, tiles_m);
-    } else {
-        static bool set32 = false;
-        if (!set32) { (void)hipFuncSetAttribute((const void*)gemm_mfma_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem); set32 = true; }
-        gemm_mfma_kernel<float><<<(int)blocks, 256, shmem, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, tiles_m);
+    static bool attr_set = false;   // one flag per instantiation
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void*)gemm_mfma_kernel<TO, BM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        attr_set = true;
     }
+    gemm_mfma_kernel<TO, BM><<<(int)blocks, 256, shmem, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m);
     QE_LAUNCH_CHECK();
     return 0;
+}
+
+int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
+                 hipStream_t stream) {
+    QE_REQUIRE(K % 8 == 0, "mfma gemm: K=%d is no multiple of 8", K);
+    // 128-row tiles unless they give fewer than two blocks per compute unit (256 of them)
+    const bool small = (long)qe_cdiv(M, 128) * qe_cdiv(N, BN) < 512;
+    if (dt_o == QE_BF16)
+        return small ? launch_mfma<bf16_t, 64>(x, w, bias, out, M, N, K, stream)
+                     : launch_mfma<bf16_t, 128>(x, w, bias, out, M, N, K, stream);
+    return small ? launch_mfma<float, 64>(x, w, bias, out, M, N, K, stream)
+                 : launch_mfma<float, 128>(x, w, bias, out, M, N, K, stream);
 }
