@@ -31,7 +31,7 @@ extern "C" int qe_attention_prefill_rows(int Hq, int Hkv) {
 }
 
 // tiles: num_tiles pairs (first row of q, rows <= qe_attention_prefill_rows) of consecutive new
-// tokens of one request.  Takes what qe_attention_decode_supported takes.
+// tokens of one request.  Takes what qe_attention_prefill_supported takes.
 extern "C" int qe_attention_prefill_run(const void* q, void* out, const void* cache, const int* tiles,
                                         int num_tiles, const int* positions, const int* tok_seq,
                                         const int* block_table, int max_blocks, int Hq, int Hkv, int D, int P,
@@ -56,6 +56,10 @@ extern "C" int qe_attention(const void* q, void* out, const void* cache, const i
 
 extern "C" int qe_attention_decode_supported(int Hq, int Hkv, int D, int P, int dt_a) {
     return qe_attention_decode_ok(Hq, Hkv, D, P, dt_a) ? 1 : 0;
+}
+
+extern "C" int qe_attention_prefill_supported(int Hq, int Hkv, int D, int P, int dt_a) {
+    return (qe_attention_decode_ok(Hq, Hkv, D, P, dt_a) && (P & (P - 1)) == 0) ? 1 : 0;
 }
 
 extern "C" long qe_attention_decode_workspace_bytes(int n_dec, int Hq, int D, int max_position, int split_keys) {

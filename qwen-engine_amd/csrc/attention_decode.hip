@@ -127,6 +127,7 @@ __global__ __launch_bounds__(256) void attention_decode_merge_kernel(
     }
 }
 
+// also what the prefill kernel takes, but for the page size, which it wants to be a power of two
 bool qe_attention_decode_ok(int Hq, int Hkv, int D, int P, int dt_a) {
     return dt_a == QE_BF16 && (D == 64 || D == 128) && P % 16 == 0 && Hq % Hkv == 0 && Hq / Hkv <= 16;
 }

@@ -3,58 +3,90 @@
 //
 // A wave owns 32 columns: R consecutive query rows of a request for each of GH = 32 / R query
 // heads that share one key/value head (GH = the group size when that is a power of two up to 32,
-// else 1), so one pass over the keys serves the whole group.  It walks the keys its rows see,
-// 32 at a time, straight from the cache pages (keys written by this same step included):
+// else 1), so one pass over the keys serves the whole group.  A block is four waves with four
+// neighbouring row tiles of one request.  It walks the keys its rows see, 32 at a time, from the
+// cache pages (keys written by this same step included): the 256 threads bring the next key
+// tile and value tile into shared memory with contiguous 16-byte loads while the waves compute
+// on the current one (two buffers, one barrier per tile); every wave then reads its MFMA
+// operands from shared memory, whose rows are padded so that those reads do not collide.
 //   S^T[key, col] = K[key, :] . Q[col, :]         v_mfma_f32_32x32x16_bf16, D / 16 of them;
-//       lane (g, r), g = lane / 32, r = lane % 32, loads K[key r][ks * 16 + g * 8 .. + 8] (16 bytes)
+//       lane (g, r), g = lane / 32, r = lane % 32, takes K[key r][ks * 16 + g * 8 .. + 8]
 //       and ends up with 16 scores: keys 8 b + 4 g + j (b, j < 4) of column r
 //   online softmax per column in 32-bit, in the base-2 domain (scores are scaled by
 //       scale * log2 e once); the accumulator is rescaled only when a maximum moved
 //   O^T[d, col] += V^T[d, key] . P^T[key, col]    v_mfma_f32_32x32x16_bf16, 2 * D / 32 of them;
 //       the 8 probabilities of a half tile that a lane holds are its B operand as they lie, and
-//       because value tiles are stored transposed ([D][P]) the A operand is two 8-byte loads
-// No shared memory; one shuffle per tile.  The causal and window limits are applied per
-// column, so the order of the sums for a row depends on its position and the window only.
-// A block holds four neighbouring row tiles, so that their key tiles meet in the CU's cache.
+//       because value tiles are stored transposed ([D][P]) the A operand is two 8-byte reads
+// The causal and window limits are applied per column, so the order of the sums for a row
+// depends on its position and the window only.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(16))) float floatx16;
+typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
 
 union PackV {   // two 8-byte pieces of a value row as one MFMA operand
     bf16x8 v;
-    bf16x4 h[2];
     uint2 u[2];
 };
+union Piece {   // a staged 16-byte piece, addressable by element for masking
+    uint4_t q;
+    uint2 u[2];
+    unsigned short e[8];
+};
 
+#define VROW 40   // bytes of a staged value row: 16 keys = 32 bytes of data + 8 of padding
+
+// Two blocks per compute unit (at most 256 registers a lane): while one block waits for its next
+// tile or at its barrier, the other computes.
 template <int D>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(
+__global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
-    const int* __restrict__ tiles, int num_tiles,
-    const int* __restrict__ positions, const int* __restrict__ tok_seq,
+    const int* __restrict__ tiles, const int* __restrict__ positions, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int max_blocks,
-    int Hq, int Hkv, int P, float scale_log2, int window, int R) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int Hq, int Hkv, int P, int log2P, float scale_log2, int window, int R) {
+    constexpr int KROW = D * 2 + 16;                 // bytes of a staged key row
+    constexpr int KBYTES = 32 * KROW, VBYTES = 2 * D * VROW, BUF = KBYTES + VBYTES;
+    constexpr int KP = 32 * (D / 8) / 256;           // 16-byte key pieces per thread (2 for D = 128)
+    constexpr int VP = 2 * D * 2 / 256;              // 16-byte value pieces per thread
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 5, r = lane & 31;
-    const int ti = blockIdx.x * 4 + wave;
-    if (ti >= num_tiles) return;
     const int G = Hq / Hkv;
     const int GH = 32 / R;                                 // heads per wave
     const int kvh = blockIdx.y / (G / GH);
     const int head = kvh * G + (blockIdx.y % (G / GH)) * GH + r / R;   // this lane's column: head and row
-    const int row0 = tiles[2 * ti], cnt = tiles[2 * ti + 1];
+
+    // the block's four tiles belong to one request, in ascending rows; tiles of 0 rows pad the group
+    const int* bt4 = tiles + 8 * blockIdx.x;
+    const int row_first = bt4[0];
+    int last = 0;
+#pragma unroll
+    for (int j = 1; j < 4; ++j) if (bt4[2 * j + 1] > 0) last = j;
+    const int p_block = positions[row_first];
+    const int kmin = (window > 0 && p_block - window + 1 > 0) ? p_block - window + 1 : 0;
+    const int kmax = positions[bt4[2 * last]] + bt4[2 * last + 1];
+    const int* bt = block_table + (long)tok_seq[row_first] * max_blocks;
+    const long page_stride = 2L * Hkv * P * D;
+
+    // this wave's tile
+    const int row0 = bt4[2 * wave], cnt = bt4[2 * wave + 1];
+    const bool wave_on = cnt > 0;
     const int rr = r % R;
-    const bool col_ok = rr < cnt;
-    const int row = row0 + (col_ok ? rr : cnt - 1);        // columns beyond the tile repeat its last row
+    const bool col_ok = wave_on && rr < cnt;
+    const int row = wave_on ? row0 + (rr < cnt ? rr : cnt - 1) : row_first;   // columns beyond the tile repeat its last row
     const int p = positions[row];
     const int hi = p + 1;
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    const int p_first = positions[row0];
+    const int p_first = positions[wave_on ? row0 : row_first];
     const int k_start = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
-    const int k_stop = p_first + cnt;                      // positions of a tile's rows are consecutive
-    const int* bt = block_table + (long)tok_seq[row0] * max_blocks;
-    const long page_stride = 2L * Hkv * P * D;
+    const int k_stop = wave_on ? p_first + cnt : 0;       // positions of a tile's rows are consecutive
+    // keys every column of the wave sees without a limit: [all_lo, all_hi)
+    const int p_last = p_first + cnt - 1;
+    const int all_hi = p_first + 1;
+    const int all_lo = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
 
     bf16x8 qreg[D / 16];
 #pragma unroll
@@ -68,121 +100,140 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[db][e] = 0.f;
 
-    // what a lane adds to a page's base to reach its piece of a key tile and of a value tile
-    const long k_lane = ((long)kvh * P + (r & 15)) * D + g * 8;
-    const long v_lane = ((long)(Hkv + kvh) * P) * D + (long)r * P + 4 * g;
-    const long v_step = 32L * P;                          // from one block of 32 value rows to the next
-    // keys every column sees without a limit: [all_lo, all_hi); a tile inside needs no masks
-    const int p_last = p_first + cnt - 1;
-    const int all_hi = p_first + 1;
-    const int all_lo = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
-
+    // ---- staging: global -> registers -> shared ------------------------------------------------
     // A 32-key tile has two halves of 16 keys with pages and offsets of their own.  A half that no
-    // row sees (beyond the request's keys, or wholly behind the window, where the page may have
-    // been given back) reads the other half's memory again and is masked out.
-#define TILE_ADDR(kk_)                                                                              \
-    const bool first_ = (kk_) + 16 > k_start, second_ = (kk_) + 16 < k_stop;                        \
-    const int ka_ = first_ ? (kk_) : (kk_) + 16;                                                    \
-    const int kb_ = second_ ? (kk_) + 16 : (kk_);                                                   \
-    const long base_a = (long)bt[ka_ / P] * page_stride + (long)(ka_ % P) * D;                      \
-    const long base_b = (long)bt[kb_ / P] * page_stride + (long)(kb_ % P) * D;                      \
-    const long vbase_a = (long)bt[ka_ / P] * page_stride + (ka_ % P);                               \
-    const long vbase_b = (long)bt[kb_ / P] * page_stride + (kb_ % P);
-#define LOAD_K()                                                                                    \
+    // row of the block sees (beyond the request's keys, or wholly behind the window, where the page
+    // may have been given back) reads the other half's memory again; what lies outside
+    // [kmin, kmax) is zeroed in the value tile (it may be unwritten memory, and anything times a
+    // weight of 0 must still be 0) and masked in the scores.
+    Piece kst[KP], vst[VP];
+    // what a thread adds to (page base + offset-in-page scaled) to reach its pieces: constant over the loop
+    long kconst[KP], vconst[VP];
+    bool khalf[KP], vhalf[VP];
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+        const int id = tid + 256 * i;
+        const int krow = id / (D / 8), col = id % (D / 8);
+        khalf[i] = krow >= 16;
+        kconst[i] = ((long)kvh * P + (krow & 15)) * D + col * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < VP; ++i) {
+        const int id = tid + 256 * i;
+        const int rem = id % (2 * D);
+        vhalf[i] = id >= 2 * D;
+        vconst[i] = ((long)(Hkv + kvh) * P) * D + (long)(rem >> 1) * P + (rem & 1) * 8;
+    }
+    const int pmask = P - 1;
+#define STAGE_LOAD(kk_)                                                                             \
     {                                                                                               \
-        const bf16_t* kp = cache + ((r < 16) ? base_a : base_b) + k_lane;                           \
-        _Pragma("unroll") for (int ks = 0; ks < D / 16; ++ks) kreg[ks] = *(const bf16x8*)(kp + ks * 16); \
+        const bool first_ = (kk_) + 16 > kmin, second_ = (kk_) + 16 < kmax;                         \
+        const int ka_ = first_ ? (kk_) : (kk_) + 16;                                                \
+        const int kb_ = second_ ? (kk_) + 16 : (kk_);                                               \
+        const long pa_ = (long)bt[ka_ >> log2P] * page_stride, pb_ = (long)bt[kb_ >> log2P] * page_stride; \
+        const int oa_ = ka_ & pmask, ob_ = kb_ & pmask;                                             \
+        const long ka_base = pa_ + (long)oa_ * D, kb_base = pb_ + (long)ob_ * D;                    \
+        _Pragma("unroll") for (int i = 0; i < KP; ++i)                                              \
+            kst[i].q = *(const uint4_t*)(cache + (khalf[i] ? kb_base : ka_base) + kconst[i]);       \
+        _Pragma("unroll") for (int i = 0; i < VP; ++i)                                              \
+            vst[i].q = *(const uint4_t*)(cache + (vhalf[i] ? pb_ + ob_ : pa_ + oa_) + vconst[i]);   \
+        if ((kk_) + 32 > kmax || (kk_) < kmin) {                                                    \
+            _Pragma("unroll") for (int i = 0; i < VP; ++i) {                                        \
+                const int id = tid + 256 * i;                                                       \
+                const int half = id / (2 * D), part = id & 1;                                       \
+                _Pragma("unroll") for (int e = 0; e < 8; ++e) {                                     \
+                    const int key = (kk_) + 16 * half + 8 * part + e;                               \
+                    if (key < kmin || key >= kmax) vst[i].e[e] = 0;                                 \
+                }                                                                                   \
+            }                                                                                       \
+        }                                                                                           \
+    }
+#define STAGE_STORE(buf_)                                                                           \
+    {                                                                                               \
+        unsigned char* ks_ = smem + (buf_) * BUF;                                                   \
+        unsigned char* vs_ = ks_ + KBYTES;                                                          \
+        _Pragma("unroll") for (int i = 0; i < KP; ++i) {                                            \
+            const int id = tid + 256 * i;                                                           \
+            *(uint4_t*)(ks_ + (id / (D / 8)) * KROW + (id % (D / 8)) * 16) = kst[i].q;              \
+        }                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < VP; ++i) {                                            \
+            const int id = tid + 256 * i;                                                           \
+            unsigned char* dst = vs_ + (id >> 1) * VROW + (id & 1) * 16;                            \
+            *(uint2*)dst = vst[i].u[0];                                                             \
+            *(uint2*)(dst + 8) = vst[i].u[1];                                                       \
+        }                                                                                           \
     }
 
-    bf16x8 kreg[D / 16];
-    const int kk0 = (k_start / 32) * 32;
-    {
-        TILE_ADDR(kk0)
-        LOAD_K()
-        (void)vbase_a; (void)vbase_b;
-    }
-    for (int kk = kk0; kk < k_stop; kk += 32) {
-        PackV vreg[D / 32][2];
-        {
-            TILE_ADDR(kk)
-            const bf16_t* va = cache + vbase_a + v_lane;
-            const bf16_t* vb = cache + vbase_b + v_lane;
-            (void)base_a; (void)base_b;
+    const int kk0 = (kmin / 32) * 32;
+    STAGE_LOAD(kk0)
+    STAGE_STORE(0)
+    __syncthreads();
+    int buf = 0;
+    for (int kk = kk0; kk < kmax; kk += 32, buf ^= 1) {
+        const bool more = kk + 32 < kmax;
+        if (more) STAGE_LOAD(kk + 32)                     // travels while this tile is computed
+        __builtin_amdgcn_sched_barrier(0);                // keep the loads ahead of the computation
+        if (wave_on && kk < k_stop && kk + 32 > k_start) { // some row of the wave sees some key of the tile
+            const unsigned char* ks_ = smem + buf * BUF + r * KROW + g * 16;
+            const unsigned char* vs_ = smem + buf * BUF + KBYTES + r * VROW + g * 8;
+            floatx16 s;
 #pragma unroll
-            for (int db = 0; db < D / 32; ++db) {
-                vreg[db][0].u[0] = *(const uint2*)(va + db * v_step);
-                vreg[db][0].u[1] = *(const uint2*)(va + db * v_step + 8);
-                vreg[db][1].u[0] = *(const uint2*)(vb + db * v_step);
-                vreg[db][1].u[1] = *(const uint2*)(vb + db * v_step + 8);
-            }
-        }
-        floatx16 s;
+            for (int e = 0; e < 16; ++e) s[e] = 0.f;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s[e] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks)
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kreg[ks], qreg[ks], s, 0, 0, 0);
-        if (kk + 32 < k_stop) {   // the next tile's keys travel while this tile's softmax and values are computed
-            TILE_ADDR(kk + 32)
-            LOAD_K()
-            (void)vbase_a; (void)vbase_b;
-        }
+            for (int ks = 0; ks < D / 16; ++ks)
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(ks_ + ks * 32), qreg[ks], s, 0, 0, 0);
 
-        float tmax = -INFINITY;
-        if (kk >= all_lo && kk + 32 <= all_hi) {           // every column sees every key of the tile
+            float tmax = -INFINITY;
+            if (kk >= all_lo && kk + 32 <= all_hi) {       // every column sees every key of the tile
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    s[e] *= scale_log2;
+                    tmax = fmaxf(tmax, s[e]);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int key = kk + 8 * (e >> 2) + 4 * g + (e & 3);
+                    s[e] = (key >= lo && key < hi) ? s[e] * scale_log2 : -INFINITY;
+                    tmax = fmaxf(tmax, s[e]);
+                }
+            }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            const float mn = fmaxf(m, tmax);
+            const float ref = (mn == -INFINITY) ? 0.f : mn;   // a column that has seen no key yet: all weights 0
+            if (__any(mn > m)) {                              // some column's maximum moved: rescale
+                const float alpha = __builtin_amdgcn_exp2f(m - ref);
+                l *= alpha;
+#pragma unroll
+                for (int db = 0; db < D / 32; ++db) acc[db] *= alpha;
+            }
+            m = mn;
+            PackV pb[2];
+            float psum = 0.f;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                s[e] *= scale_log2;
-                tmax = fmaxf(tmax, s[e]);
+                const float pe = __builtin_amdgcn_exp2f(s[e] - ref);   // 0 for keys that are not seen
+                psum += pe;
+                pb[e >> 3].v[e & 7] = (__bf16)pe;
             }
-        } else {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int key = kk + 8 * (e >> 2) + 4 * g + (e & 3);
-                s[e] = (key >= lo && key < hi) ? s[e] * scale_log2 : -INFINITY;
-                tmax = fmaxf(tmax, s[e]);
-            }
-        }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float mn = fmaxf(m, tmax);
-        const float ref = (mn == -INFINITY) ? 0.f : mn;    // a column that has seen no key yet: all weights 0
-        if (__any(mn > m)) {                               // some column's maximum moved: rescale
-            const float alpha = __builtin_amdgcn_exp2f(m - ref);
-            l *= alpha;
-#pragma unroll
-            for (int db = 0; db < D / 32; ++db) acc[db] *= alpha;
-        }
-        m = mn;
-        PackV pb[2];
-        float psum = 0.f;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const float pe = __builtin_amdgcn_exp2f(s[e] - ref);   // 0 for keys that are not seen
-            psum += pe;
-            pb[e >> 3].v[e & 7] = (__bf16)pe;
-        }
-        l += psum;
-        if (kk + 32 > k_stop || kk < k_start) {
-            // the tile reaches beyond what any row sees: such keys may be unwritten memory, and
-            // anything times a weight of 0 must still be 0
+            l += psum;
 #pragma unroll
             for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-                for (int h = 0; h < 2; ++h)
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int key = kk + 16 * h + 8 * (e >> 2) + 4 * g + (e & 3);
-                        if (key < k_start || key >= k_stop) vreg[db][h].v[e] = (__bf16)0.f;
-                    }
+                for (int h = 0; h < 2; ++h) {
+                    PackV vv;
+                    const unsigned char* vp = vs_ + (h * D + db * 32) * VROW;
+                    vv.u[0] = *(const uint2*)vp;
+                    vv.u[1] = *(const uint2*)(vp + 16);
+                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vv.v, pb[h].v, acc[db], 0, 0, 0);
+                }
         }
-#pragma unroll
-        for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vreg[db][h].v, pb[h].v, acc[db], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) STAGE_STORE(buf ^ 1)                    // its readers finished before the last barrier
+        __syncthreads();
     }
-#undef TILE_ADDR
-#undef LOAD_K
+#undef STAGE_LOAD
+#undef STAGE_STORE
     l += __shfl_xor(l, 32, 64);
     if (col_ok) {
         const float inv = 1.f / l;
@@ -206,26 +257,31 @@ int qe_attention_prefill_tile_rows(int Hq, int Hkv) {
     return 32 / (pow2 ? G : 1);
 }
 
-// tiles: num_tiles pairs (first row of q, number of rows <= qe_attention_prefill_tile_rows);
-// a tile's rows belong to one request and have consecutive positions.
+// tiles: num_tiles pairs (first row of q, number of rows <= qe_attention_prefill_tile_rows), in
+// groups of four that belong to one request, in ascending rows, with consecutive positions
+// through the group; a group is filled up with pairs of 0 rows.  num_tiles is a multiple of 4.
 int qe_attention_prefill(const void* q, void* out, const void* cache, const int* tiles, int num_tiles,
                          const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
                          int Hq, int Hkv, int D, int P, float scale, int window, hipStream_t stream) {
-    QE_REQUIRE((D == 64 || D == 128) && P % 16 == 0 && Hq % Hkv == 0, "prefill attention: sizes not taken");
+    QE_REQUIRE((D == 64 || D == 128) && P >= 16 && (P & (P - 1)) == 0 && Hq % Hkv == 0,
+               "prefill attention: sizes not taken");
+    int log2P = 0;
+    while ((1 << log2P) < P) ++log2P;
+    QE_REQUIRE(num_tiles % 4 == 0, "prefill attention: tiles come in groups of four");
     if (num_tiles == 0) return 0;
     const int R = qe_attention_prefill_tile_rows(Hq, Hkv);
     const int waves_per_kv = (Hq / Hkv) / (32 / R);
     QE_REQUIRE(Hkv * waves_per_kv <= 65535, "prefill attention: too many heads");
-    dim3 grid(qe_cdiv(num_tiles, 4), Hkv * waves_per_kv);
+    dim3 grid(num_tiles / 4, Hkv * waves_per_kv);
     const float scale_log2 = scale * 1.4426950408889634f;
     if (D == 128)
         attention_prefill_kernel<128><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache,
-                                                                tiles, num_tiles, positions, tok_seq, block_table,
-                                                                max_blocks, Hq, Hkv, P, scale_log2, window, R);
+                                                                tiles, positions, tok_seq, block_table,
+                                                                max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R);
     else
         attention_prefill_kernel<64><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache,
-                                                               tiles, num_tiles, positions, tok_seq, block_table,
-                                                               max_blocks, Hq, Hkv, P, scale_log2, window, R);
+                                                               tiles, positions, tok_seq, block_table,
+                                                               max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R);
     QE_LAUNCH_CHECK();
     return 0;
 }

@@ -43,13 +43,26 @@ class StepContext:
 
     def other_tiles(self, rows_per_tile: int) -> Optional[torch.Tensor]:
         """The rows of requests that bring several tokens, cut into tiles of at most
-        ``rows_per_tile`` consecutive rows of one request: int32 [tiles, 2] = (first row, rows).
-        Built and sent to the device once per step and tile size."""
+        ``rows_per_tile`` consecutive rows: int32 [tiles, 2] = (first row, rows), in groups of
+        four tiles of one request (a group is filled up with tiles of 0 rows).  Built and sent
+        to the device once per step and tile size."""
         if rows_per_tile <= 0:
             return None
         if rows_per_tile not in self._tiles:
-            flat = [v for s in self.seqs if s.q_len > 1 for r in range(0, s.q_len, rows_per_tile)
-                    for v in (s.q_start + r, min(rows_per_tile, s.q_len - r))]
+            flat = prefill_tiles([(s.q_start, s.q_len) for s in self.seqs if s.q_len > 1], rows_per_tile)
             t = torch.tensor(flat, dtype=torch.int32).view(-1, 2)
             self._tiles[rows_per_tile] = t.to(self.rt.device) if flat else None
         return self._tiles[rows_per_tile]
+
+
+def prefill_tiles(portions, rows_per_tile: int) -> List[int]:
+    """(first row, rows) pairs, flat, for portions given as (first row, number of rows): tiles of
+    at most rows_per_tile rows, in groups of four per portion, padded with (first row, 0)."""
+    flat: List[int] = []
+    for start, n in portions:
+        tiles = [(start + r, min(rows_per_tile, n - r)) for r in range(0, n, rows_per_tile)]
+        while len(tiles) % 4:
+            tiles.append((start, 0))
+        for t in tiles:
+            flat.extend(t)
+    return flat

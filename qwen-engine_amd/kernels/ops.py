@@ -50,6 +50,7 @@ def load_library():
         "qe_gemm_partial_splits": [i32, i32],
         "qe_gemm_fused_supported": [i32, i32, i32, i32, i32],
         "qe_attention_decode_supported": [i32, i32, i32, i32, i32],
+        "qe_attention_prefill_supported": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_rows": [i32, i32],
         "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, vp],
         "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
@@ -299,6 +300,14 @@ def attention_decode_supported(q: torch.Tensor, cache: torch.Tensor) -> bool:
                                                   _DT[q.dtype]))
 
 
+def attention_prefill_supported(q: torch.Tensor, cache: torch.Tensor) -> bool:
+    """True if the MFMA prefill kernel takes these sizes: those of the decode kernel with a page
+    size that is a power of two."""
+    lib = load_library()
+    return bool(lib.qe_attention_prefill_supported(q.shape[1], cache.shape[2], q.shape[2], cache.shape[3],
+                                                   _DT[q.dtype]))
+
+
 def prefill_tile_rows(num_heads: int, num_kv_heads: int) -> int:
     """Rows of a tile of the prefill attention kernel for these head counts (``other_tiles``)."""
     return load_library().qe_attention_prefill_rows(num_heads, num_kv_heads)
@@ -362,7 +371,7 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
             generic(dec_tokens)
     if other_tokens is not None and other_tokens.shape[0]:
         _need(other_tokens, "other_tokens", torch.int32, (None,), dev)
-        if other_tiles is not None and algo != ALGO_GENERIC and attention_decode_supported(q, cache):
+        if other_tiles is not None and algo != ALGO_GENERIC and attention_prefill_supported(q, cache):
             _need(other_tiles, "other_tiles", torch.int32, (None, 2), dev)
             _check(lib.qe_attention_prefill_run(q.data_ptr(), out.data_ptr(), cache.data_ptr(),
                                                 other_tiles.data_ptr(), other_tiles.shape[0],

@@ -447,7 +447,7 @@ def test_prefill_attention_kernel(ops, hq, hkv, d, page, window):
     bf = torch.bfloat16
     scale = 1 / math.sqrt(d)
     lens = [(0, 75), (100, 37), (15, 2), (33, 1)]
-    qs, pos, seq, tables, caches, want, tiles, dec, other = [], [], [], [], [], [], [], [], []
+    qs, pos, seq, tables, caches, want, portions, dec, other = [], [], [], [], [], [], [], [], []
     base, row = 0, 0
     R = ops.prefill_tile_rows(hq, hkv)
     assert R == 32 // (hq // hkv) if (hq // hkv) in (1, 2, 4, 8, 16, 32) else R == 32
@@ -467,8 +467,10 @@ def test_prefill_attention_kernel(ops, hq, hkv, d, page, window):
             dec.append(row)
         else:
             other += list(range(row, row + n))
-            tiles += [[row + r, min(R, n - r)] for r in range(0, n, R)]
+            portions.append((row, n))
         row += n
+    from qwen_engine_amd.engine.batch import prefill_tiles
+    tiles = torch.tensor(prefill_tiles(portions, R), dtype=torch.int32).view(-1, 2).tolist()
     width = max(len(t) for t in tables)
     table = torch.full((len(lens), width), -1, dtype=torch.int32)
     for b, t in enumerate(tables):
@@ -495,8 +497,8 @@ def test_prefill_kernel_one_far_key_decides(ops, key_pos):
     cache, ids = paged_cache(k, v, page, 164, bf)
     n = L - first
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
-    R = ops.prefill_tile_rows(hq, hkv)
-    tiles = [[r, min(R, n - r)] for r in range(0, n, R)]
+    from qwen_engine_amd.engine.batch import prefill_tiles
+    tiles = torch.tensor(prefill_tiles([(0, n)], ops.prefill_tile_rows(hq, hkv)), dtype=torch.int32).view(-1, 2).tolist()
     out = ops.attention(q.to(DEV), cache.to(DEV), i32(list(range(first, L))), i32([0] * n), ids[None].to(DEV),
                         1 / math.sqrt(d), dec_tokens=i32([]), other_tokens=i32(list(range(n))), other_tiles=i32(tiles))
     want = P.attention(q.float(), k.float(), v.float(), 1 / math.sqrt(d))
