@@ -133,6 +133,7 @@ class RequestCache:
     shared_len: int = 0                # tokens taken over from other requests at admission
     new_request: bool = True           # no step has run yet: fixed-size state must be cleared
     dirty: List[List[int]] = field(default_factory=list)   # per group: table indices changed since taken
+    released: List[int] = field(default_factory=list)      # per group: table entries below this were given back
 
 
 @dataclass
@@ -171,7 +172,7 @@ class CacheManager:
             raise CacheError(f"request {req_id!r} is live already")
         slot = self.slots.take(req_id)
         rc = RequestCache(req_id=req_id, state_slot=slot, tables=[[] for _ in self.groups],
-                          dirty=[[] for _ in self.groups])
+                          dirty=[[] for _ in self.groups], released=[0] * len(self.groups))
         self.requests[req_id] = rc
         return rc
 
@@ -206,13 +207,11 @@ class CacheManager:
         rc = self.get(req_id)
         need = []
         for g, table in enumerate(rc.tables):
+            # entries from the first live page up to the table's end hold pages (reserve leaves
+            # no holes there), so what is missing lies beyond the table's end
             lo = self._first_live_page(g, rc.num_tokens)
             hi = (new_len + self.page_size - 1) // self.page_size
-            n = 0
-            for i in range(lo, hi):
-                if i >= len(table) or table[i] < 0:
-                    n += 1
-            need.append(n)
+            need.append(max(0, hi - max(lo, len(table))))
         return need
 
     def can_reserve(self, wants: Sequence[Tuple[Hashable, int]]) -> bool:
@@ -237,13 +236,13 @@ class CacheManager:
         hi = (new_len + self.page_size - 1) // self.page_size
         for g, table in enumerate(rc.tables):
             lo = self._first_live_page(g, rc.num_tokens)
-            while len(table) < hi:
+            start = max(lo, len(table))
+            while len(table) < start:              # behind the window from the start: never held
                 table.append(-1)
-            for i in range(lo, hi):
-                if table[i] < 0:
-                    table[i] = self.pools[g].allocate()
-                    rc.dirty[g].append(i)
-                    self.stats["pages_allocated"] += 1
+            for i in range(start, hi):
+                table.append(self.pools[g].allocate())
+                rc.dirty[g].append(i)
+                self.stats["pages_allocated"] += 1
 
     def commit(self, req_id: Hashable, tokens: Sequence[int]) -> None:
         """The step has written these tokens' keys: lengthen the request, register pages
@@ -261,12 +260,13 @@ class CacheManager:
         for g, table in enumerate(rc.tables):
             if self.groups[g].window is None:
                 continue
-            live_from = self._first_live_page(g, new_len)
-            for i in range(min(live_from, len(table))):
+            live_from = min(self._first_live_page(g, new_len), len(table))
+            for i in range(rc.released[g], live_from):   # pages below rc.released[g] went back earlier
                 if table[i] >= 0:
                     self._release(g, table[i])
                     table[i] = -1
                     rc.dirty[g].append(i)
+            rc.released[g] = max(rc.released[g], live_from)
 
     def _release(self, g: int, page: int) -> None:
         if self.pools[g].release(page):

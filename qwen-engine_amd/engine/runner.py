@@ -68,6 +68,7 @@ class ModelRunner:
     """
 
     SPLIT_BUCKET = 8      # decode graphs are recorded per this many splits of the keys
+    MAX_GRAPHS = 24       # recorded graphs kept (each holds its own activations); the least recently used goes first
 
     def __init__(self, model: DecoderModel, page_size: int, num_pages, max_requests: int,
                  prefix_sharing: bool = False, use_graphs: Optional[bool] = None):
@@ -263,10 +264,12 @@ class ModelRunner:
                                     torch.tensor(upd_val[g], dtype=torch.int32).to(self.rt.device))
                 upd_idx[g], upd_val[g] = [], []
         key = (B, bucket)
-        rec = self._graphs.get(key)
+        rec = self._graphs.pop(key, None)
         if rec is None:
+            while len(self._graphs) >= self.MAX_GRAPHS:
+                self._graphs.pop(next(iter(self._graphs)))     # dicts keep insertion order: the oldest use
             rec = self._record_decode_graph(B, bucket, cap)
-            self._graphs[key] = rec
+        self._graphs[key] = rec                                # (re)inserted last = most recently used
         parts = [token_ids, positions, tok_seq, list(range(B)), [s.state_slot for s in seqs], list(range(B))]
         for g in range(n_groups):
             pad = cap - len(upd_idx[g])
