@@ -9,9 +9,9 @@ int qe_gemm_skinny(const void* x, const void* w, const float* bias, void* out, i
 int qe_gemm_skinny_splits(int N, int K);
 bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w);
 int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
-                 hipStream_t stream);
+                 int tile, hipStream_t stream);
 
-enum { ALGO_AUTO = 0, ALGO_GENERIC = 1, ALGO_MFMA = 2 };
+enum { ALGO_AUTO = 0, ALGO_GENERIC = 1, ALGO_MFMA = 2, ALGO_TILE = 1000 };   // ALGO_TILE + rows: the tiled kernel with that tile
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3 };
 
 // 1 if the fused epilogues (add into the 32-bit residual stream; silu(gate) * up) can be used
@@ -37,10 +37,14 @@ extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* ou
         QE_REQUIRE(skinny, "gemm: M=%d N=%d K=%d with these element types is not taken by the kernel for few rows", M, N, K);
         return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, epilogue, splits, stream);
     }
-    QE_REQUIRE(algo == ALGO_AUTO || algo == ALGO_GENERIC || algo == ALGO_MFMA, "gemm: unknown algo %d", algo);
+    QE_REQUIRE(algo == ALGO_AUTO || algo == ALGO_GENERIC || algo == ALGO_MFMA || algo > ALGO_TILE, "gemm: unknown algo %d", algo);
+    if (algo > ALGO_TILE) {
+        QE_REQUIRE(tiled, "gemm: M=%d N=%d K=%d is not taken by the tiled MFMA kernel", M, N, K);
+        return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, algo - ALGO_TILE, stream);
+    }
     if (algo != ALGO_GENERIC) {
         if (skinny) return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, EPI_STORE, 1, stream);
-        if (tiled) return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, stream);
+        if (tiled) return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, algo >= ALGO_TILE ? algo - ALGO_TILE : 0, stream);
         QE_REQUIRE(algo == ALGO_AUTO, "gemm: M=%d N=%d K=%d with these element types is not taken by an MFMA kernel", M, N, K);
     }
     return qe_gemm_generic(x, w, bias, out, M, N, K, dt_a, dt_w, dt_o, stream);

@@ -429,6 +429,10 @@ def test_gemm_tiled_mfma(ops, M, N, K):
     want = P.linear(x.double(), w.double())
     got = ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_FAST)
     close(got, want, bf)
+    for rows in (64, 128, 256):                              # every tile shape on every size
+        close(ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_TILE + rows), want, bf)
+        close(ops.gemm(x.to(DEV), w.to(DEV), bias.to(DEV), out_dtype=torch.float32, algo=ops.ALGO_TILE + rows),
+              want + bias.double(), torch.float32, scale=float(want.abs().max()))
     got32 = ops.gemm(x.to(DEV), w.to(DEV), bias.to(DEV), out_dtype=torch.float32, algo=ops.ALGO_FAST)
     close(got32, want + bias.double(), torch.float32, scale=float(want.abs().max()))
     # the generic kernel on the same operands agrees to accumulation order
