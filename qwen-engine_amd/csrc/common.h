@@ -39,6 +39,31 @@ template <> struct Elem<bf16_t> {
     static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = float_to_bf16(v); }
 };
 
+// Four consecutive elements as one 16-byte (float) or 8-byte (bfloat16) access.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+        const float4 t = *(const float4*)p;
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+        *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+    }
+};
+template <> struct Vec4<bf16_t> {
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+        const uint2 t = *(const uint2*)p;
+        v[0] = bf16_bits_to_float(t.x & 0xffffu); v[1] = bf16_bits_to_float(t.x >> 16);
+        v[2] = bf16_bits_to_float(t.y & 0xffffu); v[3] = bf16_bits_to_float(t.y >> 16);
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+        uint2 t;
+        t.x = (uint32_t)float_to_bf16(v[0]).bits | ((uint32_t)float_to_bf16(v[1]).bits << 16);
+        t.y = (uint32_t)float_to_bf16(v[2]).bits | ((uint32_t)float_to_bf16(v[3]).bits << 16);
+        *(uint2*)p = t;
+    }
+};
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

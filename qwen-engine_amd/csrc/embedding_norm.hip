@@ -66,30 +66,6 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ del
 // The same for rows of up to NV * 4 * blockDim.x elements with H % 4 == 0: the row is read once
 // (16-byte loads, all in flight together) and kept in registers.  This is the kernel of decode
 // steps, where a launch has few rows and its time is the latency of its memory accesses.
-template <typename T> struct Vec4;
-template <> struct Vec4<float> {
-    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
-        const float4 t = *(const float4*)p;
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-    }
-    static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
-        *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
-    }
-};
-template <> struct Vec4<bf16_t> {
-    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
-        const uint2 t = *(const uint2*)p;
-        v[0] = bf16_bits_to_float(t.x & 0xffffu); v[1] = bf16_bits_to_float(t.x >> 16);
-        v[2] = bf16_bits_to_float(t.y & 0xffffu); v[3] = bf16_bits_to_float(t.y >> 16);
-    }
-    static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
-        uint2 t;
-        t.x = (uint32_t)float_to_bf16(v[0]).bits | ((uint32_t)float_to_bf16(v[1]).bits << 16);
-        t.y = (uint32_t)float_to_bf16(v[2]).bits | ((uint32_t)float_to_bf16(v[3]).bits << 16);
-        *(uint2*)p = t;
-    }
-};
-
 template <typename TA, typename TD, int NV>
 __global__ void rmsnorm_regs_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_delta, long delta_stride,
                                     const int* __restrict__ rows, const float* __restrict__ w,

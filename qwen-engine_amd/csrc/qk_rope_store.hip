@@ -82,6 +82,90 @@ __global__ __launch_bounds__(64) void qk_rope_store_kernel(
     }
 }
 
+// The same work for head sizes D = 8 * 2^k (and a rotation over the whole head): a head is
+// taken by D / 8 lanes, each with 4 features of the first half and the 4 features 64... D / 2
+// further that rotate with them, so a wave works on 512 / D heads at a time with 8-byte
+// accesses and the norm's sum needs log2(D / 8) shuffles.  One block of 256 threads per token.
+template <typename TA>
+__global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
+    const TA* __restrict__ qkv, const int* __restrict__ positions,
+    const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
+    const float* __restrict__ table, const int* __restrict__ slot, TA* __restrict__ cache,
+    TA* __restrict__ q_out, TA* __restrict__ packed_out, int Hq, int Hkv, int D, int P) {
+    const long t = blockIdx.x;
+    const int lph = D / 8;                     // lanes per head
+    const int half = D / 2;
+    const int j = threadIdx.x % lph;           // this lane's place in its head
+    const int heads_per_pass = 256 / lph;
+    const int nheads = Hq + 2 * Hkv;
+    const int width = nheads * D;
+    const int s = slot ? slot[t] : -1;
+    const float* cs = table ? table + (long)positions[t] * D : nullptr;
+    for (int head = threadIdx.x / lph; head < nheads; head += heads_per_pass) {
+        const bool is_q = head < Hq;
+        const bool is_k = !is_q && head < Hq + Hkv;
+        const TA* src = qkv + t * width + (long)head * D;
+        float a[4], b[4];                      // features 4 j .. 4 j + 3 and half + 4 j .. half + 4 j + 3
+        Vec4<TA>::load(src + 4 * j, a);
+        Vec4<TA>::load(src + half + 4 * j, b);
+        TA* dst = nullptr;
+        if (packed_out) {
+            dst = packed_out + t * width + (long)head * D;
+        } else if (is_q) {
+            dst = q_out + (t * Hq + head) * D;
+        } else if (s >= 0) {
+            const long page = s / P, off = s % P;
+            const int kh = is_k ? head - Hq : head - Hq - Hkv;
+            if (is_k) {
+                dst = cache + page * (2L * Hkv * P * D) + ((long)kh * P + off) * D;
+            } else {   // value tile is [D][P]: a column of single elements
+                TA* vt = cache + page * (2L * Hkv * P * D) + ((long)(Hkv + kh) * P) * D + off;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    Elem<TA>::store(vt + (long)(4 * j + e) * P, a[e]);
+                    Elem<TA>::store(vt + (long)(half + 4 * j + e) * P, b[e]);
+                }
+            }
+        }
+        const bool is_v = !is_q && !is_k;
+        if (is_v) {
+            if (packed_out) {
+                Vec4<TA>::store(dst + 4 * j, a);
+                Vec4<TA>::store(dst + half + 4 * j, b);
+            }
+            continue;
+        }
+        const float* w = is_q ? q_w : k_w;
+        if (w) {
+            float ss = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ss += a[e] * a[e] + b[e] * b[e];
+            for (int o = lph >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            const float rstd = rsqrtf(ss / (float)D + eps);
+            float wa[4], wb[4];
+            Vec4<float>::load(w + 4 * j, wa);
+            Vec4<float>::load(w + half + 4 * j, wb);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { a[e] = a[e] * rstd * wa[e]; b[e] = b[e] * rstd * wb[e]; }
+        }
+        if (cs) {
+            float c[4], sn[4];
+            Vec4<float>::load(cs + 4 * j, c);
+            Vec4<float>::load(cs + half + 4 * j, sn);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float x1 = a[e], x2 = b[e];
+                a[e] = c[e] * x1 - sn[e] * x2;
+                b[e] = sn[e] * x1 + c[e] * x2;
+            }
+        }
+        if (dst) {
+            Vec4<TA>::store(dst + 4 * j, a);
+            Vec4<TA>::store(dst + half + 4 * j, b);
+        }
+    }
+}
+
 extern "C" int qe_qk_rope_store(const void* qkv, const int* positions, const float* q_w, const float* k_w,
                                 float eps, const float* table, int rotary_dim, const int* slot,
                                 void* cache, void* q_out, void* packed_out, int T, int Hq, int Hkv,
@@ -94,6 +178,21 @@ extern "C" int qe_qk_rope_store(const void* qkv, const int* positions, const flo
     QE_REQUIRE(Hq + 2 * Hkv <= 65535, "qk_rope_store: too many heads");
     QE_REQUIRE(q_out || packed_out, "qk_rope_store: no output");
     if (T == 0) return 0;
+    const int lph = D / 8;
+    if (D % 8 == 0 && lph >= 1 && lph <= 64 && (lph & (lph - 1)) == 0 && (!table || rotary_dim == D)) {
+        if (dt_a == QE_F32)
+            qk_rope_store_vec_kernel<float><<<T, 256, 0, stream>>>(
+                (const float*)qkv, positions, q_w, k_w, eps, table, slot, (float*)cache, (float*)q_out,
+                (float*)packed_out, Hq, Hkv, D, P);
+        else if (dt_a == QE_BF16)
+            qk_rope_store_vec_kernel<bf16_t><<<T, 256, 0, stream>>>(
+                (const bf16_t*)qkv, positions, q_w, k_w, eps, table, slot, (bf16_t*)cache, (bf16_t*)q_out,
+                (bf16_t*)packed_out, Hq, Hkv, D, P);
+        else
+            QE_REQUIRE(false, "qk_rope_store: unknown dtype %d", dt_a);
+        QE_LAUNCH_CHECK();
+        return 0;
+    }
     dim3 grid(T, Hq + 2 * Hkv);
     const size_t shmem = (size_t)D * sizeof(float);
     if (dt_a == QE_F32)
