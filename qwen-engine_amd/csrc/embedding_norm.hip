@@ -95,6 +95,12 @@ __global__ void rmsnorm_regs_kernel(float* __restrict__ h, const TD* __restrict_
             for (int e = 0; e < 4; ++e) ss += v[i][e] * v[i][e];
         }
     }
+    float wv[NV][4];                       // the weights are asked for before the sum is waited for
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = (threadIdx.x + i * blockDim.x) * 4;
+        if (c < H) Vec4<float>::load(w + c, wv[i]);
+    }
     ss = block_sum(ss, red);
     const float rstd = rsqrtf(ss / (float)H + eps);
     const bool write_back = dr && !rows;
@@ -103,10 +109,9 @@ __global__ void rmsnorm_regs_kernel(float* __restrict__ h, const TD* __restrict_
         const int c = (threadIdx.x + i * blockDim.x) * 4;
         if (c < H) {
             if (write_back) Vec4<float>::store(hr + c, v[i]);
-            float wv[4], o[4];
-            Vec4<float>::load(w + c, wv);
+            float o[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = v[i][e] * rstd * wv[e];
+            for (int e = 0; e < 4; ++e) o[e] = v[i][e] * rstd * wv[i][e];
             Vec4<TA>::store(out + r * H + c, o);
         }
     }

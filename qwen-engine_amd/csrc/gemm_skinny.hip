@@ -27,7 +27,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TO* __restrict__ out, int M, int N, int K, int cps) {
     constexpr int NW = (EPI == EPI_SILU_MUL) ? 2 : 1;   // weight tiles per block
-    constexpr int U = (MT <= 2) ? 4 : 2;                // chunks whose loads are issued together
+    constexpr int U = (MT == 1 && EPI != EPI_SILU_MUL) ? 8 : ((MT <= 2) ? 4 : 2);   // chunks whose loads are issued together
     __shared__ float red[4][NW][MT][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r = lane & 15;

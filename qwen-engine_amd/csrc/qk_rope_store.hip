@@ -179,7 +179,9 @@ extern "C" int qe_qk_rope_store(const void* qkv, const int* positions, const flo
     QE_REQUIRE(q_out || packed_out, "qk_rope_store: no output");
     if (T == 0) return 0;
     const int lph = D / 8;
-    if (D % 8 == 0 && lph >= 1 && lph <= 64 && (lph & (lph - 1)) == 0 && (!table || rotary_dim == D)) {
+    // (with few tokens the kernel with one wave per head has more waves in flight and is quicker)
+    if ((long)T * (Hq + 2 * Hkv) > 2048 && D % 8 == 0 && lph >= 1 && lph <= 64 && (lph & (lph - 1)) == 0 &&
+        (!table || rotary_dim == D)) {
         if (dt_a == QE_F32)
             qk_rope_store_vec_kernel<float><<<T, 256, 0, stream>>>(
                 (const float*)qkv, positions, q_w, k_w, eps, table, slot, (float*)cache, (float*)q_out,
