@@ -8,8 +8,10 @@
 // batch.  A second kernel merges the splits.
 #include "attention_tile.h"
 
-// SPLIT: keys per split (a multiple of 16).  The next tile is loaded while the current one is
-// computed, and the split's page ids are read before the loop.
+// SPLIT: keys per split (a multiple of 16, at most 64 tiles).  The next tile is loaded while the
+// current one is computed, and the split's page ids are read before the loop.
+// (Merging the splits in this same kernel, by the wave that finishes last, was tried: the
+// device-wide fences it needs cost several times what the separate merge kernel costs.)
 template <int D, int SPLIT>
 __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
@@ -38,12 +40,10 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     const long page_stride = 2L * Hkv * P * D;
     const int tile0 = (k_begin - split * SPLIT) / 16;                 // first and one-past-last tile of the split
     const int tile1 = (k_end - split * SPLIT + 15) / 16;
-    int pages[TILES];
-#pragma unroll
-    for (int i = 0; i < TILES; ++i) {
-        const int kk = split * SPLIT + i * 16;
-        pages[i] = (i >= tile0 && i < tile1) ? bt[kk / P] : 0;
-    }
+    // lane i holds the page of tile i (one vector load for the whole split); a tile's page is
+    // then read from that lane
+    int my_page = 0;
+    if (lane >= tile0 && lane < tile1) my_page = bt[(split * SPLIT + lane * 16) / P];
 
     bf16x8 qreg[D / 32];
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -54,17 +54,24 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     AttnState<D> st;
     st.init();
 
-    KVTile<D> cur, nxt;
-    load_tile<D>(cur, cache, pages[tile0], page_stride, kvh, Hkv, P, (split * SPLIT + tile0 * 16) % P, g, n);
-#pragma unroll
-    for (int i = 0; i < TILES; ++i) {
-        if (i < tile0 || i >= tile1) continue;
-        const int kk = split * SPLIT + i * 16;
-        if (i + 1 < tile1)
-            load_tile<D>(nxt, cache, pages[(i + 1 < TILES) ? i + 1 : i], page_stride, kvh, Hkv, P, (kk + 16) % P, g, n);
-        attn_tile_step<D>(st, cur, qreg, scale, kk, g, k_begin, k_end, k_begin, k_end);
-        cur = nxt;
+    // Two tile buffers used in turn: the loads of the next tile are issued before the current
+    // one is computed, and nothing is copied from one buffer to the other.
+#define LOAD(buf_, i_) load_tile<D>(buf_, cache, __builtin_amdgcn_readlane(my_page, (i_)), page_stride, kvh, Hkv, P, \
+                                    (split * SPLIT + (i_) * 16) % P, g, n)
+#define STEP(buf_, i_) attn_tile_step<D>(st, buf_, qreg, scale, split * SPLIT + (i_) * 16, g, k_begin, k_end, k_begin, k_end)
+    KVTile<D> ta, tb;
+    int i = tile0;
+    LOAD(ta, i);
+    while (true) {
+        if (i + 1 < tile1) LOAD(tb, i + 1);
+        STEP(ta, i);
+        if (++i >= tile1) break;
+        if (i + 1 < tile1) LOAD(ta, i + 1);
+        STEP(tb, i);
+        if (++i >= tile1) break;
     }
+#undef LOAD
+#undef STEP
     float l = st.l;
     const float m = st.m;
     l += __shfl_xor(l, 16, 64);
