@@ -27,7 +27,14 @@ TINY_C = dict(
     num_hidden_layers=2, num_attention_heads=6, num_key_value_heads=2, head_dim=48,
     max_position_embeddings=400, rms_norm_eps=1e-6, rope_theta=50000.0, tie_word_embeddings=True)
 
-TINY = {"A": (TINY_A, 0, 4), "B": (TINY_B, 1, 8), "C": (TINY_C, 2, 16)}   # config, seed, page size
+# D: head size 64 and widths in multiples of 32, so that the bfloat16 mode runs on the MFMA kernels
+# (attention for decode and prefill, both matrix products) inside the engine; 4 heads per group.
+TINY_D = dict(
+    architectures=["Qwen3ForCausalLM"], vocab_size=300, hidden_size=128, intermediate_size=192,
+    num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=2, head_dim=64,
+    max_position_embeddings=1024, rms_norm_eps=1e-6, rope_theta=10000.0, tie_word_embeddings=False)
+
+TINY = {"A": (TINY_A, 0, 4), "B": (TINY_B, 1, 8), "C": (TINY_C, 2, 16), "D": (TINY_D, 3, 16)}   # config, seed, page size
 
 
 def make_folder(tmp, which: str, dtype=torch.bfloat16, norm_std=0.01, std=0.02, scale_qk=None):
