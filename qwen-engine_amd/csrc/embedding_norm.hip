@@ -177,28 +177,31 @@ extern "C" int qe_residual_add(float* h, const void* delta, long n, int dt_a, hi
     return 0;
 }
 
-// out[t, i] = silu(gu[t, i]) * gu[t, I + i], the product formed in 32-bit.
+// out[t, i] = silu(gate[t, i]) * up[t, i], the product formed in 32-bit.  gu holds gate | up per
+// row, or (interleave) gate and up in alternating blocks of 32: gate 0..31, up 0..31, gate 32..63, ...
 template <typename TA>
-__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int T, int I) {
+__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int T, int I, int interleave) {
     const long n = (long)T * I;
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (long)gridDim.x * blockDim.x) {
         const long t = idx / I;
         const int i = (int)(idx - t * I);
-        const float g = Elem<TA>::load(gu + t * 2 * I + i);
-        const float u = Elem<TA>::load(gu + t * 2 * I + I + i);
+        const long gi = interleave ? (long)(i >> 5) * 64 + (i & 31) : i;
+        const float g = Elem<TA>::load(gu + t * 2 * I + gi);
+        const float u = Elem<TA>::load(gu + t * 2 * I + gi + (interleave ? 32 : I));
         Elem<TA>::store(out + idx, g / (1.f + expf(-g)) * u);
     }
 }
 
-extern "C" int qe_silu_mul(const void* gu, void* out, int T, int I, int dt_a, hipStream_t stream) {
+extern "C" int qe_silu_mul(const void* gu, void* out, int T, int I, int interleave, int dt_a, hipStream_t stream) {
     QE_REQUIRE(T >= 0 && I > 0, "silu_mul: bad sizes T=%d I=%d", T, I);
+    QE_REQUIRE(!interleave || I % 32 == 0, "silu_mul: interleaved gate|up needs a width in blocks of 32, not %d", I);
     if (T == 0) return 0;
     const long n = (long)T * I;
     const int blocks = (int)((n + 255) / 256 > 8192 ? 8192 : (n + 255) / 256);
     if (dt_a == QE_F32)
-        silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, T, I);
+        silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, T, I, interleave);
     else if (dt_a == QE_BF16)
-        silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, T, I);
+        silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, T, I, interleave);
     else
         QE_REQUIRE(false, "silu_mul: unknown dtype %d", dt_a);
     QE_LAUNCH_CHECK();

@@ -9,14 +9,19 @@ int qe_gemm_skinny(const void* x, const void* w, const float* bias, void* out, i
 int qe_gemm_skinny_splits(int N, int K);
 bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w);
 int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
-                 int tile, hipStream_t stream);
+                 int tile, bool silu, hipStream_t stream);
 
 enum { ALGO_AUTO = 0, ALGO_GENERIC = 1, ALGO_MFMA = 2, ALGO_TILE = 1000 };   // ALGO_TILE + rows: the tiled kernel with that tile
-enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3 };
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3, EPI_SILU_MUL_IL = 4 };
 
 // 1 if the fused epilogues (add into the 32-bit residual stream; silu(gate) * up) can be used
 extern "C" int qe_gemm_fused_supported(int M, int N, int K, int dt_a, int dt_w) {
     return qe_gemm_skinny_ok(M, N, K, dt_a, dt_w) ? 1 : 0;
+}
+
+// 1 if epilogue 4 (silu-mul over interleaved gate|up rows) can be used: N counts the outputs
+extern "C" int qe_gemm_silu_supported(int M, int N, int K, int dt_a, int dt_w) {
+    return (N % 32 == 0 && (qe_gemm_skinny_ok(M, N, K, dt_a, dt_w) || qe_gemm_mfma_ok(M, 2 * N, K, dt_a, dt_w))) ? 1 : 0;
 }
 
 // number of partial products that epilogue 3 should be asked for
@@ -25,6 +30,8 @@ extern "C" int qe_gemm_partial_splits(int N, int K) { return qe_gemm_skinny_spli
 // out[M, N] = x[M, K] . w[N, K]^T (+ bias).  epilogue 0: store in dt_o.  1: add into out, the
 // 32-bit stream.  2: w is [2 N, K], gate rows then up rows; out = silu(x.gate^T) * (x.up^T).
 // 3: out is float [splits, M, N], partial products along K to be summed over the first index.
+// 4: as 2 with the gate and up rows of w interleaved in blocks of 32 (gate 0..31, up 0..31, ...);
+//    taken by the kernel for few rows and by the tiled one.
 // algo: 0 = choose, 1 = the generic 32-bit kernel, 2 = an MFMA kernel (the one for few rows up to
 // 64 rows, the tiled one above) or an error if neither takes the operands.
 extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
@@ -33,6 +40,11 @@ extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* ou
     if (M == 0) return 0;
     const bool skinny = qe_gemm_skinny_ok(M, N, K, dt_a, dt_w);
     const bool tiled = qe_gemm_mfma_ok(M, N, K, dt_a, dt_w);
+    if (epilogue == EPI_SILU_MUL_IL && !skinny) {
+        QE_REQUIRE(N % 32 == 0 && qe_gemm_mfma_ok(M, 2 * N, K, dt_a, dt_w),
+                   "gemm: M=%d N=%d K=%d is not taken by a silu-mul kernel", M, N, K);
+        return qe_gemm_mfma(x, w, bias, out, M, 2 * N, K, dt_o, algo > ALGO_TILE ? algo - ALGO_TILE : 0, true, stream);
+    }
     if (epilogue != EPI_STORE) {
         QE_REQUIRE(skinny, "gemm: M=%d N=%d K=%d with these element types is not taken by the kernel for few rows", M, N, K);
         return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, epilogue, splits, stream);
@@ -40,11 +52,11 @@ extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* ou
     QE_REQUIRE(algo == ALGO_AUTO || algo == ALGO_GENERIC || algo == ALGO_MFMA || algo > ALGO_TILE, "gemm: unknown algo %d", algo);
     if (algo > ALGO_TILE) {
         QE_REQUIRE(tiled, "gemm: M=%d N=%d K=%d is not taken by the tiled MFMA kernel", M, N, K);
-        return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, algo - ALGO_TILE, stream);
+        return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, algo - ALGO_TILE, false, stream);
     }
     if (algo != ALGO_GENERIC) {
         if (skinny) return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, EPI_STORE, 1, stream);
-        if (tiled) return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, algo >= ALGO_TILE ? algo - ALGO_TILE : 0, stream);
+        if (tiled) return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, 0, false, stream);
         QE_REQUIRE(algo == ALGO_AUTO, "gemm: M=%d N=%d K=%d with these element types is not taken by an MFMA kernel", M, N, K);
     }
     return qe_gemm_generic(x, w, bias, out, M, N, K, dt_a, dt_w, dt_o, stream);

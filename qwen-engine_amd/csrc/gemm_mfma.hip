@@ -22,7 +22,10 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float floatx16;
 typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
 
-template <typename TO, int BM, int BN, int BK, int MINB>
+// SILU: W holds gate and up rows interleaved in blocks of 32 (gate 0..31, up 0..31, gate 32..63,
+// ...), N counts all of them, and the result is silu(gate) * up, N / 2 wide: the two MFMA tiles a
+// lane holds side by side are the gate and the up of the same outputs.
+template <typename TO, int BM, int BN, int BK, int MINB, bool SILU>
 __global__ __launch_bounds__(256, MINB) void gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TO* __restrict__ out, int M, int N, int K, int tiles_m) {
@@ -43,27 +46,30 @@ __global__ __launch_bounds__(256, MINB) void gemm_mfma_kernel(
 
     // A piece outside the matrices is loaded from a valid address all the same and replaced by
     // zeros only when it is stored to shared memory: a select right after the load would make
-    // the wave wait for the load before it computes.
+    // the wave wait for the load before it computes.  Addresses are formed once; a step adds BK.
+    const bf16_t* src[LD];
+    bool row_ok[LD];
+    int kofs[LD], dst[LD];
+#pragma unroll
+    for (int i = 0; i < LD; ++i) {
+        const int q = tid + 256 * i;
+        const int row = q / PPR, pc = q % PPR;
+        const bool is_a = row < BM;
+        const int grow = is_a ? m0 + row : n0 + row - BM;
+        row_ok[i] = grow < (is_a ? M : N);
+        kofs[i] = pc * 8;
+        src[i] = (is_a ? x : w) + (long)(row_ok[i] ? grow : 0) * K + pc * 8;
+        dst[i] = row * ROWB + pc * 16;
+    }
 #define LOAD_GLOBAL(kt_)                                                                 \
     _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                     \
-        const int q = tid + 256 * i;                                                     \
-        const int row = q / PPR, pc = q % PPR;                                           \
-        const int k = (kt_) * BK + pc * 8;                                               \
-        const bool is_a = row < BM;                                                      \
-        const int grow = is_a ? m0 + row : n0 + row - BM;                                \
-        const bool ok = k < K && grow < (is_a ? M : N);                                  \
-        const bf16_t* src = (is_a ? x : w) + (long)(ok ? grow : 0) * K + (ok ? k : 0);   \
-        stage[i] = *(const uint4_t*)src;                                                 \
+        const bool ok = (kt_) * BK + kofs[i] < K;                                        \
+        stage[i] = *(const uint4_t*)(ok ? src[i] + (kt_) * BK : src[i]);                 \
     }
 #define STORE_SHARED(buf_, kt_)                                                          \
     _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                     \
-        const int q = tid + 256 * i;                                                     \
-        const int row = q / PPR, pc = q % PPR;                                           \
-        const int k = (kt_) * BK + pc * 8;                                               \
-        const bool is_a = row < BM;                                                      \
-        const int grow = is_a ? m0 + row : n0 + row - BM;                                \
-        const bool ok = k < K && grow < (is_a ? M : N);                                  \
-        *(uint4_t*)(smem + (buf_) * (BM + BN) * ROWB + row * ROWB + pc * 16) =           \
+        const bool ok = row_ok[i] && (kt_) * BK + kofs[i] < K;                           \
+        *(uint4_t*)(smem + (buf_) * (BM + BN) * ROWB + dst[i]) =                         \
             ok ? stage[i] : uint4_t{0u, 0u, 0u, 0u};                                     \
     }
 
@@ -96,7 +102,7 @@ __global__ __launch_bounds__(256, MINB) void gemm_mfma_kernel(
             for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < NJ; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
         }
         if (kt + 1 < nk) { STORE_SHARED(buf ^ 1, kt + 1) }   // the other buffer: its readers finished before the last barrier
         __syncthreads();
@@ -104,28 +110,48 @@ __global__ __launch_bounds__(256, MINB) void gemm_mfma_kernel(
 #undef LOAD_GLOBAL
 #undef STORE_SHARED
 
-    // C of a 32x32 MFMA: lane holds column (lane % 32), rows 8 * b + 4 * (lane / 32) + r for e = 4 * b + r.
-    // With A = x rows and B = W rows that is: token row m, output column n = lane % 32.
+    // The MFMA is given the W rows as its first operand and the x rows as its second, so its
+    // result is the tile transposed: a lane holds, for the token row m = lane % 32, the outputs
+    // n = 8 b + 4 (lane / 32) + r (e = 4 b + r): four consecutive n at a time, one 8- or 16-byte store.
+    const int NO = SILU ? N / 2 : N;             // width of the output
+    const bool vec_ok = (NO % 4) == 0;
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
+    for (int i = 0; i < MI; ++i) {
+        const int m = m0 + wm + i * 32 + (lane & 31);
+        if (m >= M) continue;
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            const int n = n0 + wn + j * 32 + (lane & 31);
-            if (n >= N) continue;
-            const float bv = bias ? bias[n] : 0.f;
+        for (int j = 0; j < NJ; j += (SILU ? 2 : 1))
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int m = m0 + wm + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                if (m < M) Elem<TO>::store(out + (long)m * N + n, acc[i][j][e] + bv);
+            for (int bq = 0; bq < 4; ++bq) {
+                const int nw = n0 + wn + j * 32;                       // first weight row of the MFMA tile
+                const int n = (SILU ? nw / 2 : nw) + 8 * bq + 4 * (lane >> 5);
+                if (n >= NO) continue;
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (SILU) {
+                        const float gt = acc[i][j][4 * bq + r], up = acc[i][j + (SILU ? 1 : 0)][4 * bq + r];
+                        v[r] = gt / (1.f + __expf(-gt)) * up;
+                    } else {
+                        v[r] = acc[i][j][4 * bq + r] + ((bias && n + r < NO) ? bias[n + r] : 0.f);
+                    }
+                }
+                TO* o = out + (long)m * NO + n;
+                if (vec_ok) {
+                    Vec4<TO>::store(o, v);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) if (n + r < NO) Elem<TO>::store(o + r, v[r]);
+                }
             }
-        }
+    }
 }
 
 bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w) {
     return dt_a == QE_BF16 && dt_w == QE_BF16 && M > 64 && K % 8 == 0 && K >= 64;
 }
 
-template <typename TO, int BM, int BN, int BK, int MINB>
+template <typename TO, int BM, int BN, int BK, int MINB, bool SILU>
 static int launch_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                        hipStream_t stream) {
     const int tiles_m = qe_cdiv(M, BM), tiles_n = qe_cdiv(N, BN);
@@ -134,33 +160,39 @@ static int launch_mfma(const void* x, const void* w, const float* bias, void* ou
     const size_t shmem = 2 * (BM + BN) * (BK * 2 + 16);
     static bool attr_set = false;   // one flag per instantiation
     if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)gemm_mfma_kernel<TO, BM, BN, BK, MINB>,
+        (void)hipFuncSetAttribute((const void*)gemm_mfma_kernel<TO, BM, BN, BK, MINB, SILU>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         attr_set = true;
     }
-    gemm_mfma_kernel<TO, BM, BN, BK, MINB><<<(int)blocks, 256, shmem, stream>>>(
+    gemm_mfma_kernel<TO, BM, BN, BK, MINB, SILU><<<(int)blocks, 256, shmem, stream>>>(
         (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m);
     QE_LAUNCH_CHECK();
     return 0;
 }
 
-template <typename TO>
+template <typename TO, bool SILU>
 static int pick_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                      int tile, hipStream_t stream) {
     const long cus = 256;
     const long big = (long)qe_cdiv(M, 256) * qe_cdiv(N, 128), mid = (long)qe_cdiv(M, 128) * qe_cdiv(N, 128);
     // the largest tile that still gives every compute unit two blocks (one, for the middle size)
     if (tile == 0) tile = big >= 2 * cus ? 256 : (mid >= cus ? 128 : 64);
-    if (tile == 256) return launch_mfma<TO, 256, 128, 32, 2>(x, w, bias, out, M, N, K, stream);
-    if (tile == 128) return launch_mfma<TO, 128, 128, 64, 2>(x, w, bias, out, M, N, K, stream);
-    return launch_mfma<TO, 64, 128, 64, 2>(x, w, bias, out, M, N, K, stream);
+    if (tile == 256) return launch_mfma<TO, 256, 128, 32, 2, SILU>(x, w, bias, out, M, N, K, stream);
+    if (tile == 128) return launch_mfma<TO, 128, 128, 64, 2, SILU>(x, w, bias, out, M, N, K, stream);
+    return launch_mfma<TO, 64, 128, 64, 2, SILU>(x, w, bias, out, M, N, K, stream);
 }
 
-// tile: rows of the output tile (256, 128 or 64), 0 to choose by the shape
+// tile: rows of the output tile (256, 128 or 64), 0 to choose by the shape.  silu: w is [N, K] with
+// gate and up rows interleaved in blocks of 32, out is [M, N / 2] = silu(gate) * up.
 int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
-                 int tile, hipStream_t stream) {
+                 int tile, bool silu, hipStream_t stream) {
     QE_REQUIRE(K % 8 == 0, "mfma gemm: K=%d is no multiple of 8", K);
     QE_REQUIRE(tile == 0 || tile == 256 || tile == 128 || tile == 64, "mfma gemm: tile of %d rows", tile);
-    if (dt_o == QE_BF16) return pick_mfma<bf16_t>(x, w, bias, out, M, N, K, tile, stream);
-    return pick_mfma<float>(x, w, bias, out, M, N, K, tile, stream);
+    if (silu) {
+        QE_REQUIRE(!bias && N % 64 == 0, "mfma gemm: silu-mul takes no bias and gate|up rows in blocks of 32");
+        if (dt_o == QE_BF16) return pick_mfma<bf16_t, true>(x, w, bias, out, M, N, K, tile, stream);
+        return pick_mfma<float, true>(x, w, bias, out, M, N, K, tile, stream);
+    }
+    if (dt_o == QE_BF16) return pick_mfma<bf16_t, false>(x, w, bias, out, M, N, K, tile, stream);
+    return pick_mfma<float, false>(x, w, bias, out, M, N, K, tile, stream);
 }

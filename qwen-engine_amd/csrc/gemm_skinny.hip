@@ -17,7 +17,7 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 
-enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3 };
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3, EPI_SILU_MUL_IL = 4 };
 
 // grid (N / 16, S): block (bx, s) sums the chunks [s * cps, (s + 1) * cps) of K.  With S > 1 the
 // epilogue is EPI_PARTIAL: 32-bit partial products out[s][M][N] that the consumer adds up in the
@@ -26,8 +26,9 @@ template <int MT, int EPI, typename TO>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TO* __restrict__ out, int M, int N, int K, int cps) {
-    constexpr int NW = (EPI == EPI_SILU_MUL) ? 2 : 1;   // weight tiles per block
-    constexpr int U = (MT == 1 && EPI != EPI_SILU_MUL) ? 8 : ((MT <= 2) ? 4 : 2);   // chunks whose loads are issued together
+    constexpr bool SILU = EPI == EPI_SILU_MUL || EPI == EPI_SILU_MUL_IL;
+    constexpr int NW = SILU ? 2 : 1;   // weight tiles per block
+    constexpr int U = (MT == 1 && !SILU) ? 8 : ((MT <= 2) ? 4 : 2);   // chunks whose loads are issued together
     __shared__ float red[4][NW][MT][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r = lane & 15;
@@ -43,8 +44,12 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
         for (int j = 0; j < MT; ++j) acc[a][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     const bool row_ok = n0 + r < N;
-    const bf16_t* wrow0 = w + (long)(row_ok ? n0 + r : 0) * K + g * 8;
-    const bf16_t* wrow1 = (EPI == EPI_SILU_MUL) ? wrow0 + (long)N * K : wrow0;
+    // gate row n and up row n: N rows apart, or, with the rows interleaved in blocks of 32
+    // (gate 0..31, up 0..31, gate 32..63, ...), 32 rows apart inside the block of 64
+    const int nrow = row_ok ? n0 + r : 0;
+    const long wr = (EPI == EPI_SILU_MUL_IL) ? (long)(nrow >> 5) * 64 + (nrow & 31) : nrow;
+    const bf16_t* wrow0 = w + wr * K + g * 8;
+    const bf16_t* wrow1 = (EPI == EPI_SILU_MUL_IL) ? wrow0 + 32L * K : (SILU ? wrow0 + (long)N * K : wrow0);
     const bf16_t* xrow[MT];
     bool tok_ok[MT];
 #pragma unroll
@@ -61,7 +66,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
             const int cc = c + 4 * u;
             const bool ok = cc < c_end;
             a0[u] = (ok && row_ok) ? *(const bf16x8*)(wrow0 + cc * 32) : zero;
-            if (EPI == EPI_SILU_MUL) a1[u] = (ok && row_ok) ? *(const bf16x8*)(wrow1 + cc * 32) : zero;
+            if (SILU) a1[u] = (ok && row_ok) ? *(const bf16x8*)(wrow1 + cc * 32) : zero;
 #pragma unroll
             for (int j = 0; j < MT; ++j) b[u][j] = (ok && tok_ok[j]) ? *(const bf16x8*)(xrow[j] + cc * 32) : zero;
         }
@@ -70,7 +75,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
 #pragma unroll
             for (int j = 0; j < MT; ++j) {
                 acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[u], b[u][j], acc[0][j], 0, 0, 0);
-                if (EPI == EPI_SILU_MUL)
+                if (SILU)
                     acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[u], b[u][j], acc[1][j], 0, 0, 0);
             }
     }
@@ -96,7 +101,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
             const int n = n0 + g * 4 + i;
             if (n >= N) continue;
             float y = v[0][i];
-            if (EPI == EPI_SILU_MUL) {
+            if (SILU) {
                 y = y / (1.f + __expf(-y)) * v[1][i];
             } else if (bias && blockIdx.y == 0) {
                 y += bias[n];
@@ -150,6 +155,7 @@ int qe_gemm_skinny_splits(int N, int K) {
 
 // epilogue EPI_STORE: out [M, N] in dt_o.  EPI_RESIDUAL: out is the 32-bit stream [M, N], added to.
 // EPI_SILU_MUL: w is [2 N, K] (gate rows, then up rows), out [M, N] in dt_o.
+// EPI_SILU_MUL_IL: the same with gate and up rows interleaved in blocks of 32.
 // EPI_PARTIAL: out is float [splits, M, N]; the product is the sum over the first index.
 int qe_gemm_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                    int dt_o, int epilogue, int splits, hipStream_t stream) {
@@ -168,6 +174,11 @@ int qe_gemm_skinny(const void* x, const void* w, const float* bias, void* out, i
         QE_REQUIRE(!bias, "skinny gemm: silu-mul takes no bias");
         if (dt_o == QE_BF16) return launch_skinny<EPI_SILU_MUL, bf16_t>(x, w, bias, out, M, N, K, 1, stream);
         return launch_skinny<EPI_SILU_MUL, float>(x, w, bias, out, M, N, K, 1, stream);
+    }
+    if (epilogue == EPI_SILU_MUL_IL) {
+        QE_REQUIRE(!bias && N % 32 == 0, "skinny gemm: interleaved silu-mul takes no bias and N in blocks of 32");
+        if (dt_o == QE_BF16) return launch_skinny<EPI_SILU_MUL_IL, bf16_t>(x, w, bias, out, M, N, K, 1, stream);
+        return launch_skinny<EPI_SILU_MUL_IL, float>(x, w, bias, out, M, N, K, 1, stream);
     }
     QE_REQUIRE(epilogue == EPI_STORE, "skinny gemm: unknown epilogue %d", epilogue);
     if (dt_o == QE_BF16) return launch_skinny<EPI_STORE, bf16_t>(x, w, bias, out, M, N, K, 1, stream);

@@ -19,7 +19,7 @@ _DT = {torch.float32: F32, torch.bfloat16: BF16}
 
 ALGO_AUTO, ALGO_GENERIC, ALGO_FAST = 0, 1, 2
 ALGO_TILE = 1000   # ALGO_TILE + 256, 128 or 64: the tiled MFMA gemm with tiles of that many rows
-EPI_STORE, EPI_RESIDUAL, EPI_SILU_MUL, EPI_PARTIAL = 0, 1, 2, 3
+EPI_STORE, EPI_RESIDUAL, EPI_SILU_MUL, EPI_PARTIAL, EPI_SILU_MUL_IL = 0, 1, 2, 3, 4
 DECODE_SPLIT_KEYS = 128   # keys per split of the decode attention kernel
 
 
@@ -46,7 +46,8 @@ def load_library():
         "qe_rmsnorm": [vp, vp, i32, i32, i64, vp, vp, vp, i32, i32, f32, i32, vp],
         "qe_residual_add": [vp, vp, i64, i32, vp],
         "qe_scatter_int": [vp, vp, vp, i32, i64, vp],
-        "qe_silu_mul": [vp, vp, i32, i32, i32, vp],
+        "qe_silu_mul": [vp, vp, i32, i32, i32, i32, vp],
+        "qe_gemm_silu_supported": [i32, i32, i32, i32, i32],
         "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
         "qe_gemm_partial_splits": [i32, i32],
         "qe_gemm_fused_supported": [i32, i32, i32, i32, i32],
@@ -181,8 +182,16 @@ def scatter_int(table: torch.Tensor, idx: torch.Tensor, val: torch.Tensor) -> No
                               _stream()), "scatter_int")
 
 
-def silu_mul(gu: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """gu [T, 2 I] = gate | up  ->  silu(gate) * up  [T, I]."""
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """[I, K] gate and up weights -> [2 I, K] with the rows in alternating blocks of 32 (gate 0..31,
+    up 0..31, gate 32..63, ...): the layout of EPI_SILU_MUL_IL.  I must be a multiple of 32."""
+    I, K = gate.shape
+    return torch.stack([gate.view(I // 32, 32, K), up.view(I // 32, 32, K)], dim=1).reshape(2 * I, K).contiguous()
+
+
+def silu_mul(gu: torch.Tensor, out: Optional[torch.Tensor] = None, interleaved: bool = False) -> torch.Tensor:
+    """gu [T, 2 I] = gate | up (or, interleaved, gate and up in alternating blocks of 32)
+    ->  silu(gate) * up  [T, I]."""
     lib = load_library()
     _need(gu, "gu", _ACT, (None, None))
     T, I2 = gu.shape
@@ -192,7 +201,8 @@ def silu_mul(gu: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tens
     if out is None:
         out = torch.empty((T, I), dtype=gu.dtype, device=gu.device)
     _need(out, "out", gu.dtype, (T, I), gu.device)
-    _check(lib.qe_silu_mul(gu.data_ptr(), out.data_ptr(), T, I, _DT[gu.dtype], _stream()), "silu_mul")
+    _check(lib.qe_silu_mul(gu.data_ptr(), out.data_ptr(), T, I, int(interleaved), _DT[gu.dtype], _stream()),
+           "silu_mul")
     return out
 
 
@@ -202,6 +212,12 @@ def gemm_fused_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
     return bool(lib.qe_gemm_fused_supported(x.shape[0], w.shape[0], x.shape[1], _DT[x.dtype], _DT[w.dtype]))
 
 
+def gemm_silu_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """True if gemm can apply silu-mul itself over w = interleaved gate|up rows (EPI_SILU_MUL_IL)."""
+    lib = load_library()
+    return bool(lib.qe_gemm_silu_supported(x.shape[0], w.shape[0] // 2, x.shape[1], _DT[x.dtype], _DT[w.dtype]))
+
+
 def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
          out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
          algo: int = ALGO_AUTO, epilogue: int = EPI_STORE, splits: int = 0) -> torch.Tensor:
@@ -209,7 +225,8 @@ def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
 
     epilogue EPI_RESIDUAL: the product is added into ``out``, the 32-bit stream [M, N].
     epilogue EPI_SILU_MUL: w is [2 N, K] (gate rows, then up rows); the result is
-    silu(x . gate^T) * (x . up^T), [M, N].
+    silu(x . gate^T) * (x . up^T), [M, N].  EPI_SILU_MUL_IL: the same with the gate and up rows
+    interleaved in blocks of 32 (see interleave_gate_up); needs gemm_silu_supported(x, w).
     epilogue EPI_PARTIAL: the product is cut along K into ``splits`` (0: chosen for the shape)
     partial products, returned as float32 [splits, M, N]; their sum over the first index, taken
     in order, is the product.  All three need gemm_fused_supported(x, w)."""
@@ -218,7 +235,7 @@ def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
     M, K = x.shape
     _need(w, "w", _ACT, (None, K), x.device)
     N = w.shape[0]
-    if epilogue == EPI_SILU_MUL:
+    if epilogue in (EPI_SILU_MUL, EPI_SILU_MUL_IL):
         if N % 2:
             raise KernelError("gemm: gate|up weights have an odd number of rows")
         N //= 2

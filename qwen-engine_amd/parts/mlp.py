@@ -18,6 +18,7 @@ class SwiGLU:
         self.hidden = int(hidden_size)
         self.inter = int(spec.intermediate_size)
         self.w_gu = self.w_down = None
+        self.interleaved = False
 
     @staticmethod
     def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
@@ -32,15 +33,20 @@ class SwiGLU:
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gu = rt.place_matrix(torch.cat([g, u], dim=0))
+        # gate and up rows in alternating blocks of 32, so that a product's epilogue finds the gate
+        # and the up of an output side by side; widths that are no multiple of 32 keep gate | up
+        self.interleaved = self.inter % 32 == 0
+        self.w_gu = rt.place_matrix(ops.interleave_gate_up(g, u) if self.interleaved else torch.cat([g, u], dim=0))
         self.w_down = rt.place_matrix(tensors["down_proj.weight"])
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         """Returns the feed-forward output [T, H], or float32 partial products [S, T, H] of it."""
-        if ops.gemm_fused_supported(x, self.w_gu):
-            a = ops.gemm(x, self.w_gu, epilogue=ops.EPI_SILU_MUL)   # silu.mul in the product's epilogue
+        if self.interleaved and ops.gemm_silu_supported(x, self.w_gu):
+            a = ops.gemm(x, self.w_gu, epilogue=ops.EPI_SILU_MUL_IL)   # silu.mul in the product's epilogue
+        elif not self.interleaved and ops.gemm_fused_supported(x, self.w_gu):
+            a = ops.gemm(x, self.w_gu, epilogue=ops.EPI_SILU_MUL)
         else:
-            a = ops.silu_mul(ops.gemm(x, self.w_gu))
+            a = ops.silu_mul(ops.gemm(x, self.w_gu), interleaved=self.interleaved)
         if ops.gemm_fused_supported(a, self.w_down):
             return ops.gemm(a, self.w_down, epilogue=ops.EPI_PARTIAL)
         return ops.gemm(a, self.w_down)

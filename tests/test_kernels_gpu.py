@@ -509,3 +509,24 @@ def test_prefill_kernel_one_far_key_decides(ops, key_pos):
     close(out, want, bf)
     last_seen = max(key_pos, first) - first
     assert float((want[last_seen:, 0] - v[key_pos, 0].float()).abs().max()) < 0.05
+
+
+@pytest.mark.parametrize("M", [1, 8, 64, 65, 200, 1024])
+@pytest.mark.parametrize("I,K", [(160, 96), (192, 64), (3072, 1024)])
+def test_gemm_with_silu_mul_over_interleaved_rows(ops, M, I, K):
+    """gate and up rows in alternating blocks of 32: the kernel for few rows and the tiled one both
+    find the gate and the up of an output side by side; so does the separate silu.mul kernel."""
+    bf = torch.bfloat16
+    g, u = rand(I, K, seed=170, dtype=bf, scale=0.2), rand(I, K, seed=171, dtype=bf, scale=0.2)
+    x = rand(M, K, seed=172, dtype=bf)
+    w = ops.interleave_gate_up(g, u)
+    assert torch.equal(w[:32], g[:32]) and torch.equal(w[32:64], u[:32]) and torch.equal(w[64:96], g[32:64])
+    want = P.silu_mul(P.linear(x.double(), g.double()), P.linear(x.double(), u.double()))
+    assert ops.gemm_silu_supported(x.to(DEV), w.to(DEV)) == (K % 32 == 0 or M > 64)
+    if ops.gemm_silu_supported(x.to(DEV), w.to(DEV)):
+        close(ops.gemm(x.to(DEV), w.to(DEV), epilogue=ops.EPI_SILU_MUL_IL), want, bf)
+        if M > 64:
+            for rows in (64, 128, 256):
+                close(ops.gemm(x.to(DEV), w.to(DEV), epilogue=ops.EPI_SILU_MUL_IL, algo=ops.ALGO_TILE + rows), want, bf)
+    gu = ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_GENERIC)
+    close(ops.silu_mul(gu, interleaved=True), want, bf)

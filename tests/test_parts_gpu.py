@@ -71,17 +71,19 @@ def test_rotary_table_is_the_reference_formula():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_swiglu_part(dtype):
+@pytest.mark.parametrize("H,I,T", [(80, 112, 6), (96, 160, 6), (128, 192, 70)])
+def test_swiglu_part(dtype, H, I, T):
+    """Widths with and without gate|up interleaving (multiples of 32 or not), few and many rows."""
     from qwen_engine_amd.config import SwiGLUSpec
     from qwen_engine_amd.parts import Runtime, build_part
     rt = Runtime(DEV, dtype)
-    H, I = 80, 112
     part = build_part(SwiGLUSpec(intermediate_size=I), H)
     w = {"gate_proj.weight": rand(I, H, seed=3, scale=0.2, dtype=torch.bfloat16),
          "up_proj.weight": rand(I, H, seed=4, scale=0.2, dtype=torch.bfloat16),
          "down_proj.weight": rand(H, I, seed=5, scale=0.2, dtype=torch.bfloat16)}
     part.load(w, rt)
-    x = rand(6, H, seed=6, dtype=dtype)
+    x = rand(T, H, seed=6, dtype=dtype)
+    assert part.interleaved == (I % 32 == 0)
     got = branch(part.forward(x.to(DEV), None))
     act = None if dtype == torch.float32 else dtype
     want = P.mlp_block(x.float(), {f"p.mlp.{k}": v for k, v in w.items()}, "p", act_dtype=act)
