@@ -22,6 +22,8 @@ import hashlib
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
+
 
 class CacheError(RuntimeError):
     """A request for pages or slots that cannot be met, or a misuse of the manager."""
@@ -289,17 +291,24 @@ class CacheManager:
         rc.dirty[group] = []
         return out
 
-    def token_slots(self, req_id: Hashable, group: int, start: int, count: int) -> List[int]:
-        """page * page_size + offset for positions start .. start + count - 1."""
+    def token_slot_array(self, req_id: Hashable, group: int, start: int, count: int) -> np.ndarray:
+        """page * page_size + offset for positions start .. start + count - 1, as int32."""
         table = self.get(req_id).tables[group]
         P = self.page_size
-        out = []
-        for pos in range(start, start + count):
-            page = table[pos // P]
-            if page < 0:
-                raise CacheError(f"request {req_id!r} holds no page for position {pos} in group {group}")
-            out.append(page * P + pos % P)
-        return out
+        if count <= 0:
+            return np.zeros(0, dtype=np.int32)
+        first, last = start // P, (start + count - 1) // P
+        pages = np.asarray(table[first:last + 1], dtype=np.int64)
+        if len(pages) != last + 1 - first or (pages < 0).any():
+            missing = next(q for q in range(start, start + count)
+                           if q // P >= len(table) or table[q // P] < 0)
+            raise CacheError(f"request {req_id!r} holds no page for position {missing} in group {group}")
+        pos = np.arange(start, start + count, dtype=np.int64)
+        return (pages[pos // P - first] * P + pos % P).astype(np.int32)
+
+    def token_slots(self, req_id: Hashable, group: int, start: int, count: int) -> List[int]:
+        """The same as a list."""
+        return self.token_slot_array(req_id, group, start, count).tolist()
 
     # ---- prefix sharing ----------------------------------------------------------
     def match_prefix(self, req_id: Hashable, prompt: Sequence[int]) -> int:

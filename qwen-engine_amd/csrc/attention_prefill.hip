@@ -106,7 +106,10 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     // may have been given back) reads the other half's memory again; what lies outside
     // [kmin, kmax) is zeroed in the value tile (it may be unwritten memory, and anything times a
     // weight of 0 must still be 0) and masked in the scores.
-    Piece kst[KP], vst[VP];
+    // Two sets of staging registers in turn: the loads of a tile are issued two tiles ahead and
+    // stored to shared memory one tile ahead, so a load has a whole tile's computation to arrive
+    // (one tile of arithmetic is shorter than a trip to memory).
+    Piece kst[2][KP], vst[2][VP];
     // what a thread adds to (page base + offset-in-page scaled) to reach its pieces: constant over the loop
     long kconst[KP], vconst[VP];
     bool khalf[KP], vhalf[VP];
@@ -125,7 +128,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
         vconst[i] = ((long)(Hkv + kvh) * P) * D + (long)(rem >> 1) * P + (rem & 1) * 8;
     }
     const int pmask = P - 1;
-#define STAGE_LOAD(kk_)                                                                             \
+#define STAGE_LOAD(set_, kk_)                                                                       \
     {                                                                                               \
         const bool first_ = (kk_) + 16 > kmin, second_ = (kk_) + 16 < kmax;                         \
         const int ka_ = first_ ? (kk_) : (kk_) + 16;                                                \
@@ -134,54 +137,73 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
         const int oa_ = ka_ & pmask, ob_ = kb_ & pmask;                                             \
         const long ka_base = pa_ + (long)oa_ * D, kb_base = pb_ + (long)ob_ * D;                    \
         _Pragma("unroll") for (int i = 0; i < KP; ++i)                                              \
-            kst[i].q = *(const uint4_t*)(cache + (khalf[i] ? kb_base : ka_base) + kconst[i]);       \
+            kst[set_][i].q = *(const uint4_t*)(cache + (khalf[i] ? kb_base : ka_base) + kconst[i]); \
         _Pragma("unroll") for (int i = 0; i < VP; ++i)                                              \
-            vst[i].q = *(const uint4_t*)(cache + (vhalf[i] ? pb_ + ob_ : pa_ + oa_) + vconst[i]);   \
+            vst[set_][i].q = *(const uint4_t*)(cache + (vhalf[i] ? pb_ + ob_ : pa_ + oa_) + vconst[i]); \
+    }
+#define STAGE_STORE(buf_, set_, kk_)                                                                \
+    {                                                                                               \
         if ((kk_) + 32 > kmax || (kk_) < kmin) {                                                    \
             _Pragma("unroll") for (int i = 0; i < VP; ++i) {                                        \
                 const int id = tid + 256 * i;                                                       \
                 const int half = id / (2 * D), part = id & 1;                                       \
                 _Pragma("unroll") for (int e = 0; e < 8; ++e) {                                     \
                     const int key = (kk_) + 16 * half + 8 * part + e;                               \
-                    if (key < kmin || key >= kmax) vst[i].e[e] = 0;                                 \
+                    if (key < kmin || key >= kmax) vst[set_][i].e[e] = 0;                           \
                 }                                                                                   \
             }                                                                                       \
         }                                                                                           \
-    }
-#define STAGE_STORE(buf_)                                                                           \
-    {                                                                                               \
         unsigned char* ks_ = smem + (buf_) * BUF;                                                   \
         unsigned char* vs_ = ks_ + KBYTES;                                                          \
         _Pragma("unroll") for (int i = 0; i < KP; ++i) {                                            \
             const int id = tid + 256 * i;                                                           \
-            *(uint4_t*)(ks_ + (id / (D / 8)) * KROW + (id % (D / 8)) * 16) = kst[i].q;              \
+            *(uint4_t*)(ks_ + (id / (D / 8)) * KROW + (id % (D / 8)) * 16) = kst[set_][i].q;        \
         }                                                                                           \
         _Pragma("unroll") for (int i = 0; i < VP; ++i) {                                            \
             const int id = tid + 256 * i;                                                           \
             unsigned char* dst = vs_ + (id >> 1) * VROW + (id & 1) * 16;                            \
-            *(uint2*)dst = vst[i].u[0];                                                             \
-            *(uint2*)(dst + 8) = vst[i].u[1];                                                       \
+            *(uint2*)dst = vst[set_][i].u[0];                                                       \
+            *(uint2*)(dst + 8) = vst[set_][i].u[1];                                                 \
         }                                                                                           \
     }
 
+    // tile j (keys kk0 + 32 j ...) uses register set and shared buffer j % 2
     const int kk0 = (kmin / 32) * 32;
-    STAGE_LOAD(kk0)
-    STAGE_STORE(0)
+    STAGE_LOAD(0, kk0)
+    STAGE_STORE(0, 0, kk0)
+    if (kk0 + 32 < kmax) STAGE_LOAD(1, kk0 + 32)
     __syncthreads();
-    int buf = 0;
-    for (int kk = kk0; kk < kmax; kk += 32, buf ^= 1) {
-        const bool more = kk + 32 < kmax;
-        if (more) STAGE_LOAD(kk + 32)                     // travels while this tile is computed
+    for (int kk2 = kk0; kk2 < kmax; kk2 += 64) {
+#pragma unroll
+      for (int buf = 0; buf < 2; ++buf) {
+        const int kk = kk2 + 32 * buf;
+        if (kk >= kmax) break;                            // the same for all threads of the block
+        if (kk + 64 < kmax) STAGE_LOAD(buf, kk + 64)      // this set's tile went to shared memory a tile ago
         __builtin_amdgcn_sched_barrier(0);                // keep the loads ahead of the computation
         if (wave_on && kk < k_stop && kk + 32 > k_start) { // some row of the wave sees some key of the tile
             const unsigned char* ks_ = smem + buf * BUF + r * KROW + g * 16;
             const unsigned char* vs_ = smem + buf * BUF + KBYTES + r * VROW + g * 8;
+            // all key fragments are read before the first MFMA, all value fragments before the
+            // softmax: shared-memory latency then passes under the arithmetic instead of before it
+            bf16x8 kf[D / 16];
+#pragma unroll
+            for (int ks = 0; ks < D / 16; ++ks) kf[ks] = *(const bf16x8*)(ks_ + ks * 32);
+            __builtin_amdgcn_sched_barrier(0);
             floatx16 s;
 #pragma unroll
             for (int e = 0; e < 16; ++e) s[e] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < D / 16; ++ks)
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(ks_ + ks * 32), qreg[ks], s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qreg[ks], s, 0, 0, 0);
+            PackV vf[D / 32][2];
+#pragma unroll
+            for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const unsigned char* vp = vs_ + (h * D + db * 32) * VROW;
+                    vf[db][h].u[0] = *(const uint2*)vp;
+                    vf[db][h].u[1] = *(const uint2*)(vp + 16);
+                }
 
             float tmax = -INFINITY;
             if (kk >= all_lo && kk + 32 <= all_hi) {       // every column sees every key of the tile
@@ -220,17 +242,13 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 #pragma unroll
             for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    PackV vv;
-                    const unsigned char* vp = vs_ + (h * D + db * 32) * VROW;
-                    vv.u[0] = *(const uint2*)vp;
-                    vv.u[1] = *(const uint2*)(vp + 16);
-                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vv.v, pb[h].v, acc[db], 0, 0, 0);
-                }
+                for (int h = 0; h < 2; ++h)
+                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][h].v, pb[h].v, acc[db], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (more) STAGE_STORE(buf ^ 1)                    // its readers finished before the last barrier
+        if (kk + 32 < kmax) STAGE_STORE(buf ^ 1, buf ^ 1, kk + 32)   // that buffer's readers finished before the last barrier
         __syncthreads();
+      }
     }
 #undef STAGE_LOAD
 #undef STAGE_STORE

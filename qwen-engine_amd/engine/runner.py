@@ -12,9 +12,10 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
-from ..cache.manager import CacheManager
+from ..cache.manager import CacheManager, OutOfPages
 from ..cache.plan import CachePlan
 from ..config.registry import config_from_folder
 from ..kernels import ops
@@ -116,6 +117,9 @@ class ModelRunner:
         self.tables = [torch.full((max_requests, w), -1, dtype=torch.int32, device=dev) for w in self.table_width]
         self.use_graphs = (dt == torch.bfloat16 and not has_state) if use_graphs is None else bool(use_graphs)
         self._graphs = {}
+        self._stage: Optional[torch.Tensor] = None     # pinned host buffer of a step's integer arrays
+        self._stage_np = None
+        self._stage_event = torch.cuda.Event()
         self.steps_run = 0
         self.graph_steps = 0
 
@@ -130,22 +134,30 @@ class ModelRunner:
         return sum(t.numel() * t.element_size() for t in self.kv if t is not None)
 
     # ---- one step ----------------------------------------------------------------------
-    def _check_and_reserve(self, entries: Sequence[StepEntry]) -> None:
+    def _check_and_reserve(self, entries: Sequence[StepEntry]) -> List[np.ndarray]:
+        """Checks the entries, reserves their pages (all or none), and returns the entries'
+        tokens as int32 arrays."""
         cache = self.cache
         vocab = self.model.spec.vocab_size
         max_pos = self.model.spec.max_positions
         if not entries:
             raise ValueError("a step needs at least one entry")
         seen = set()
+        tokens: List[np.ndarray] = []
         for e in entries:
             if e.req_id in seen:
                 raise ValueError(f"request {e.req_id!r} appears twice in one step")
             seen.add(e.req_id)
             if len(e.tokens) == 0:
                 raise ValueError(f"request {e.req_id!r} brings no tokens")
-            for t in e.tokens:
-                if not 0 <= int(t) < vocab:
-                    raise ValueError(f"token id {t} of request {e.req_id!r} is outside the vocabulary of {vocab}")
+            arr = np.asarray(e.tokens)
+            if arr.ndim != 1 or arr.dtype.kind not in "iu":
+                raise ValueError(f"the tokens of request {e.req_id!r} are not a flat list of integers")
+            bad = (arr < 0) | (arr >= vocab)
+            if bad.any():
+                raise ValueError(f"token id {int(arr[bad][0])} of request {e.req_id!r} is outside the "
+                                 f"vocabulary of {vocab}")
+            tokens.append(arr.astype(np.int32))
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"request {e.req_id!r} wants logits at place {w} of {len(e.tokens)} tokens")
@@ -153,34 +165,31 @@ class ModelRunner:
             if rc.num_tokens + len(e.tokens) > max_pos:
                 raise ValueError(f"request {e.req_id!r} would pass the model's {max_pos} positions")
         if not cache.can_reserve([(e.req_id, cache.get(e.req_id).num_tokens + len(e.tokens)) for e in entries]):
-            from ..cache.manager import OutOfPages
             raise OutOfPages("the cache has too few free pages for this step")
         for e in entries:
             cache.reserve(e.req_id, cache.get(e.req_id).num_tokens + len(e.tokens))
+        return tokens
 
-    def _layout(self, entries: Sequence[StepEntry]):
-        """The batch as flat host lists: (seqs, named lists of ints, per-group lists)."""
+    def _layout(self, entries: Sequence[StepEntry], tokens: List[np.ndarray]):
+        """The batch as flat int32 host arrays: (seqs, token ids, positions, table row of each
+        token, wanted rows, and per group: cache slot of each token, changed table entries)."""
         cache = self.cache
         seqs: List[SeqInfo] = []
-        token_ids: List[int] = []
-        positions: List[int] = []
-        tok_seq: List[int] = []
-        rows: List[int] = []
+        positions, tok_seq, rows = [], [], []
         n_groups = len(cache.groups)
-        slots: List[List[int]] = [[] for _ in range(n_groups)]
+        slots: List[list] = [[] for _ in range(n_groups)]
         upd_idx: List[List[int]] = [[] for _ in range(n_groups)]
         upd_val: List[List[int]] = [[] for _ in range(n_groups)]
         q_start = 0
-        for e in entries:
+        for e, tok in zip(entries, tokens):
             rc = cache.get(e.req_id)
-            n = len(e.tokens)
+            n = len(tok)
             seqs.append(SeqInfo(e.req_id, q_start, n, rc.num_tokens, rc.state_slot, rc.new_request))
-            token_ids.extend(int(t) for t in e.tokens)
-            positions.extend(range(rc.num_tokens, rc.num_tokens + n))
-            tok_seq.extend([rc.state_slot] * n)          # the request's row in the device tables
-            rows.extend(q_start + int(w) for w in e.want)
+            positions.append(np.arange(rc.num_tokens, rc.num_tokens + n, dtype=np.int32))
+            tok_seq.append(np.full(n, rc.state_slot, dtype=np.int32))   # the request's row in the device tables
+            rows.append(np.asarray(e.want, dtype=np.int32).reshape(-1) + q_start)
             for g in range(n_groups):
-                slots[g].extend(cache.token_slots(e.req_id, g, rc.num_tokens, n))
+                slots[g].append(cache.token_slot_array(e.req_id, g, rc.num_tokens, n))
                 width = self.table_width[g]
                 for i, page in cache.take_dirty(e.req_id, g):
                     if i >= width:
@@ -188,44 +197,54 @@ class ModelRunner:
                     upd_idx[g].append(rc.state_slot * width + i)
                     upd_val[g].append(page)
             q_start += n
-        return seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val
+        cat = np.concatenate
+        return (seqs, cat(tokens), cat(positions), cat(tok_seq), cat(rows), [cat(x) for x in slots],
+                [np.asarray(u, dtype=np.int32) for u in upd_idx], [np.asarray(u, dtype=np.int32) for u in upd_val])
+
+    def _to_device(self, parts: List[np.ndarray]) -> List[torch.Tensor]:
+        """One copy of all the arrays to the device, through a pinned buffer that is kept and grown;
+        returns a device view for each part."""
+        total = sum(len(x) for x in parts)
+        if self._stage is None or self._stage.numel() < total:
+            self._stage = torch.empty(max(total, 4096), dtype=torch.int32).pin_memory()
+            self._stage_np = self._stage.numpy()
+        else:
+            self._stage_event.synchronize()               # the last copy out of the buffer is done
+        np.concatenate(parts, out=self._stage_np[:total])
+        dev = self._stage[:total].to(self.rt.device, non_blocking=True)
+        self._stage_event.record()
+        out, off = [], 0
+        for x in parts:
+            out.append(dev[off:off + len(x)])
+            off += len(x)
+        return out
 
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
         """Reserves pages for the entries' tokens, lays the batch out flat, and brings the
         device's block tables up to date (one copy to the device, one small kernel per group)."""
-        self._check_and_reserve(entries)
-        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(entries)
-        T, B, n_groups = len(token_ids), len(seqs), len(self.cache.groups)
-        dec_rows = [s.q_start for s in seqs if s.q_len == 1]
-        other_rows = [s.q_start + i for s in seqs if s.q_len > 1 for i in range(s.q_len)]
+        tokens = self._check_and_reserve(entries)
+        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(entries, tokens)
+        T, n_groups = len(token_ids), len(self.cache.groups)
+        i32 = np.int32
+        dec_rows = np.asarray([s.q_start for s in seqs if s.q_len == 1], dtype=i32)
+        other = [np.arange(s.q_start, s.q_start + s.q_len, dtype=i32) for s in seqs if s.q_len > 1]
+        other_rows = np.concatenate(other) if other else np.zeros(0, dtype=i32)
         max_dec = max([s.kv_before for s in seqs if s.q_len == 1], default=0)
-        parts = [token_ids, positions, tok_seq, rows, [s.state_slot for s in seqs], dec_rows, other_rows]
+        parts = [token_ids, positions, tok_seq, rows, np.asarray([s.state_slot for s in seqs], dtype=i32),
+                 dec_rows, other_rows]
         for g in range(n_groups):
             parts += [slots[g], upd_idx[g], upd_val[g]]
-        flat = [v for part in parts for v in part]
-        host = torch.tensor(flat, dtype=torch.int32).pin_memory()
-        dev = host.to(self.rt.device, non_blocking=True)
-        off = 0
-
-        def take(n):
-            nonlocal off
-            t = dev[off:off + n]
-            off += n
-            return t
-
-        d_tok, d_pos, d_seq = take(T), take(T), take(T)
-        d_rows, d_state = take(len(rows)), take(B)
-        d_dec, d_other = take(len(dec_rows)), take(len(other_rows))
+        dev = self._to_device(parts)
+        d_tok, d_pos, d_seq, d_rows, d_state, d_dec, d_other = dev[:7]
         d_slots = []
         for g in range(n_groups):
-            d_slots.append(take(T))
-            n_upd = len(upd_idx[g])
-            d_idx, d_val = take(n_upd), take(n_upd)
-            if n_upd:
+            d_slot, d_idx, d_val = dev[7 + 3 * g:10 + 3 * g]
+            d_slots.append(d_slot)
+            if len(d_idx):
                 ops.scatter_int(self.tables[g], d_idx, d_val)
         return StepContext(rt=self.rt, page_size=self.page_size, num_tokens=T, seqs=seqs, token_ids=d_tok,
                            positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
-                           logit_rows=d_rows, state_slots=d_state, max_position=max(positions),
+                           logit_rows=d_rows, state_slots=d_state, max_position=int(positions.max()),
                            dec_tokens=d_dec, other_tokens=d_other, max_dec_position=max_dec)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
@@ -248,21 +267,21 @@ class ModelRunner:
 
     # ---- decoding through a recorded graph ------------------------------------------------
     def _decode_step_with_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        self._check_and_reserve(entries)
-        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(entries)
+        tokens = self._check_and_reserve(entries)
+        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(entries, tokens)
         B, n_groups = len(seqs), len(self.cache.groups)
+        i32 = np.int32
         cap = 2 * B                                    # table updates a decode step can bring per group
-        splits = max(positions) // ops.DECODE_SPLIT_KEYS + 1
+        splits = int(positions.max()) // ops.DECODE_SPLIT_KEYS + 1
         bucket = (splits + self.SPLIT_BUCKET - 1) // self.SPLIT_BUCKET * self.SPLIT_BUCKET
         if any(len(u) > cap for u in upd_idx):
             # more table changes than the recorded step takes (the first decode step after a
             # preemption, say): bring the tables up to date apart, then go on with none
             for g in range(n_groups):
-                if upd_idx[g]:
-                    ops.scatter_int(self.tables[g],
-                                    torch.tensor(upd_idx[g], dtype=torch.int32).to(self.rt.device),
-                                    torch.tensor(upd_val[g], dtype=torch.int32).to(self.rt.device))
-                upd_idx[g], upd_val[g] = [], []
+                if len(upd_idx[g]):
+                    ops.scatter_int(self.tables[g], torch.from_numpy(upd_idx[g]).to(self.rt.device),
+                                    torch.from_numpy(upd_val[g]).to(self.rt.device))
+                upd_idx[g] = upd_val[g] = np.zeros(0, dtype=i32)
         key = (B, bucket)
         rec = self._graphs.pop(key, None)
         if rec is None:
@@ -270,13 +289,13 @@ class ModelRunner:
                 self._graphs.pop(next(iter(self._graphs)))     # dicts keep insertion order: the oldest use
             rec = self._record_decode_graph(B, bucket, cap)
         self._graphs[key] = rec                                # (re)inserted last = most recently used
-        parts = [token_ids, positions, tok_seq, list(range(B)), [s.state_slot for s in seqs], list(range(B))]
+        iota = np.arange(B, dtype=i32)
+        parts = [token_ids, positions, tok_seq, iota, np.asarray([s.state_slot for s in seqs], dtype=i32), iota]
         for g in range(n_groups):
             pad = cap - len(upd_idx[g])
-            parts += [slots[g], upd_idx[g] + [-1] * pad, upd_val[g] + [0] * pad]
-        flat = [v for part in parts for v in part]
+            parts += [slots[g], upd_idx[g], np.full(pad, -1, dtype=i32), upd_val[g], np.zeros(pad, dtype=i32)]
         rec["event"].synchronize()                     # the last copy out of the host buffer is done
-        rec["host"].copy_(torch.tensor(flat, dtype=torch.int32))
+        np.concatenate(parts, out=rec["host_np"])
         rec["meta"].copy_(rec["host"], non_blocking=True)
         rec["event"].record()
         rec["graph"].replay()
@@ -340,4 +359,5 @@ class ModelRunner:
             t[0, 0] = v
         event = torch.cuda.Event()
         event.record()
-        return {"graph": graph, "host": host, "meta": meta, "logits": logits, "event": event}
+        return {"graph": graph, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits,
+                "event": event}
