@@ -19,13 +19,10 @@ __device__ __forceinline__ float bf16_to_float(bf16_t v) {
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t bits16) {
     return __uint_as_float(bits16 << 16);
 }
-// round to nearest even; NaN stays NaN
+// round to nearest even; NaN stays NaN (the hardware conversion of gfx950, v_cvt_pk_bf16_f32)
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
     bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) { r.bits = (uint16_t)((u >> 16) | 0x0040u); return r; }
-    u += 0x7fffu + ((u >> 16) & 1u);
-    r.bits = (uint16_t)(u >> 16);
+    r.bits = __builtin_bit_cast(unsigned short, (__bf16)f);
     return r;
 }
 
@@ -57,10 +54,10 @@ template <> struct Vec4<bf16_t> {
         v[2] = bf16_bits_to_float(t.y & 0xffffu); v[3] = bf16_bits_to_float(t.y >> 16);
     }
     static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
-        uint2 t;
-        t.x = (uint32_t)float_to_bf16(v[0]).bits | ((uint32_t)float_to_bf16(v[1]).bits << 16);
-        t.y = (uint32_t)float_to_bf16(v[2]).bits | ((uint32_t)float_to_bf16(v[3]).bits << 16);
-        *(uint2*)p = t;
+        typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+        typedef __attribute__((ext_vector_type(4))) float floatx4_t;
+        const floatx4_t f = {v[0], v[1], v[2], v[3]};
+        *(bf16x4_t*)p = __builtin_convertvector(f, bf16x4_t);
     }
 };
 

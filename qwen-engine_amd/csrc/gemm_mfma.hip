@@ -28,50 +28,107 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
 template <typename TO, int BM, int BN, int BK, int MINB, bool SILU>
 __global__ __launch_bounds__(256, MINB) void gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    TO* __restrict__ out, int M, int N, int K, int tiles_m) {
+    TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n) {
     constexpr int ROWB = BK * 2 + 16;       // bytes of a staged row
     constexpr int PPR = BK / 8;             // 16-byte pieces per row
+    constexpr int RPI = 256 / PPR;          // rows the block stages with one piece per thread
     constexpr int WM = BM / 2, WN = BN / 2; // a wave's part
     constexpr int MI = WM / 32, NJ = WN / 32;
-    constexpr int LD = (BM + BN) * PPR / 256;   // pieces a thread stages per step
+    constexpr int LDA = BM / RPI, LD = (BM + BN) / RPI;   // pieces a thread stages per step: LDA of x, then of W
+    static_assert((LD == 12 || LD == 8 || LD == 6) && BM % RPI == 0 && BN % RPI == 0, "tile rows must be a multiple of the rows staged at once");
+    constexpr int BUF = (BM + BN) * ROWB;   // bytes of one buffer: the x rows, then the W rows
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    // buffer b: A rows at smem + b * (BM + BN) * ROWB, then B rows
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
+    // Consecutive blocks go to the eight XCDs in turn, and each XCD has an L2 of its own: the blocks
+    // of one XCD take a compact part of the tiles (an eighth of the tile columns, or of the tile
+    // rows), so that they share the rows of W and of x that they read through that L2.
+    int tile_m, tile_n;
+    {
+        const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
+        if (tiles_n % 8 == 0) {
+            tile_m = local % tiles_m;
+            tile_n = xcd * (tiles_n / 8) + local / tiles_m;
+        } else if (tiles_m % 8 == 0) {
+            tile_n = local % tiles_n;
+            tile_m = xcd * (tiles_m / 8) + local / tiles_n;
+        } else {
+            tile_m = blockIdx.x % tiles_m;
+            tile_n = blockIdx.x / tiles_m;
+        }
+    }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
 
     const int nk = (K + BK - 1) / BK;
-    uint4_t stage[LD];
+    // Two sets of staging registers in turn: a step's loads are issued two steps ahead and go to
+    // shared memory one step ahead, so a load has a whole step of MFMAs to arrive.
+    uint4_t stage[2][LD];
 
-    // A piece outside the matrices is loaded from a valid address all the same and replaced by
-    // zeros only when it is stored to shared memory: a select right after the load would make
-    // the wave wait for the load before it computes.  Addresses are formed once; a step adds BK.
-    const bf16_t* src[LD];
-    bool row_ok[LD];
-    int kofs[LD], dst[LD];
+    // Piece i of a thread is row (tid / PPR) of the i-th group of RPI rows, 16 bytes at k = 8 (tid % PPR).
+    // The loads are buffer loads: one descriptor for the tile's rows of x and one for its rows of W,
+    // each ending with the last row that exists, so that a row beyond the matrix is "out of range"
+    // and reads as zeros by itself.  The thread's byte offset never changes and the step's k offset
+    // is a scalar.  A thread whose piece lies beyond K (in a last step shorter than BK) picks an
+    // offset that is out of range.
+    //
+    // The loads and the waits for them are written as instructions: the compiler's own placing of
+    // waits joins what it knows at the loop's top and so waits for the youngest loads as well,
+    // which would undo the two steps of distance.  A set's registers pass through the wait
+    // statement as operands, so nothing that uses them can move ahead of it.
+    const int lrow = tid / PPR, pc = tid % PPR;
+    const int a_rows = M - m0 < BM ? M - m0 : BM, b_rows = N - n0 < BN ? N - n0 : BN;
+    const unsigned long a_addr = (unsigned long)(x + (long)m0 * K), b_addr = (unsigned long)(w + (long)n0 * K);
+    uint4_t rsrc_a, rsrc_b;   // base, base high 16 bits (stride 0), bytes, format: 32-bit raw buffer
+    rsrc_a[0] = (unsigned)a_addr; rsrc_a[1] = (unsigned)(a_addr >> 32) & 0xffffu;
+    rsrc_a[2] = (unsigned)(a_rows * K * 2); rsrc_a[3] = 0x00020000u;
+    rsrc_b[0] = (unsigned)b_addr; rsrc_b[1] = (unsigned)(b_addr >> 32) & 0xffffu;
+    rsrc_b[2] = (unsigned)(b_rows * K * 2); rsrc_b[3] = 0x00020000u;
 #pragma unroll
-    for (int i = 0; i < LD; ++i) {
-        const int q = tid + 256 * i;
-        const int row = q / PPR, pc = q % PPR;
-        const bool is_a = row < BM;
-        const int grow = is_a ? m0 + row : n0 + row - BM;
-        row_ok[i] = grow < (is_a ? M : N);
-        kofs[i] = pc * 8;
-        src[i] = (is_a ? x : w) + (long)(row_ok[i] ? grow : 0) * K + pc * 8;
-        dst[i] = row * ROWB + pc * 16;
+    for (int c = 0; c < 4; ++c) {   // the same in every lane: into scalar registers
+        rsrc_a[c] = __builtin_amdgcn_readfirstlane(rsrc_a[c]);
+        rsrc_b[c] = __builtin_amdgcn_readfirstlane(rsrc_b[c]);
     }
-#define LOAD_GLOBAL(kt_)                                                                 \
-    _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                     \
-        const bool ok = (kt_) * BK + kofs[i] < K;                                        \
-        stage[i] = *(const uint4_t*)(ok ? src[i] + (kt_) * BK : src[i]);                 \
+    int voff[LD];
+#pragma unroll
+    for (int i = 0; i < LD; ++i)
+        voff[i] = ((i < LDA ? RPI * i : RPI * (i - LDA)) + lrow) * K * 2 + pc * 16;
+    const int dst = lrow * ROWB + pc * 16;                 // where piece 0 goes in a buffer; piece i: + i RPI ROWB
+#define LOAD_GLOBAL(set_, kt_)                                                           \
+    {                                                                                    \
+        const bool k_ok = (kt_) * BK + pc * 8 < K;                                       \
+        const int soff = (kt_) * BK * 2;                                                 \
+        _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                 \
+            const int vo = k_ok ? voff[i] : 0x7fffffff;                                  \
+            if (i < LDA)                                                                 \
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                  \
+                             : "=&a"(stage[set_][i]) : "v"(vo), "s"(rsrc_a), "s"(soff) : "memory"); \
+            else                                                                         \
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                  \
+                             : "=&a"(stage[set_][i]) : "v"(vo), "s"(rsrc_b), "s"(soff) : "memory"); \
+        }                                                                                \
     }
-#define STORE_SHARED(buf_, kt_)                                                          \
-    _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                     \
-        const bool ok = row_ok[i] && (kt_) * BK + kofs[i] < K;                           \
-        *(uint4_t*)(smem + (buf_) * (BM + BN) * ROWB + dst[i]) =                         \
-            ok ? stage[i] : uint4_t{0u, 0u, 0u, 0u};                                     \
-    }
+    // waits until at most `younger_` loads are in flight; the set's registers are valid afterwards
+#define WAIT_LOADS(set_, younger_)                                                       \
+    if constexpr (LD == 12)                                                              \
+        asm volatile("s_waitcnt vmcnt(%12)"                                              \
+                     : "+a"(stage[set_][0]), "+a"(stage[set_][1]), "+a"(stage[set_][2]), "+a"(stage[set_][3]), \
+                       "+a"(stage[set_][4]), "+a"(stage[set_][5]), "+a"(stage[set_][6]), "+a"(stage[set_][7]), \
+                       "+a"(stage[set_][8 % LD]), "+a"(stage[set_][9 % LD]), "+a"(stage[set_][10 % LD]),       \
+                       "+a"(stage[set_][11 % LD])                                        \
+                     : "n"(younger_) : "memory");                                        \
+    else if constexpr (LD == 8)                                                          \
+        asm volatile("s_waitcnt vmcnt(%8)"                                               \
+                     : "+a"(stage[set_][0]), "+a"(stage[set_][1]), "+a"(stage[set_][2]), "+a"(stage[set_][3]), \
+                       "+a"(stage[set_][4]), "+a"(stage[set_][5]), "+a"(stage[set_][6 % LD]), "+a"(stage[set_][7 % LD]) \
+                     : "n"(younger_) : "memory");                                        \
+    else                                                                                 \
+        asm volatile("s_waitcnt vmcnt(%6)"                                               \
+                     : "+a"(stage[set_][0]), "+a"(stage[set_][1]), "+a"(stage[set_][2]), "+a"(stage[set_][3]), \
+                       "+a"(stage[set_][4]), "+a"(stage[set_][5])                        \
+                     : "n"(younger_) : "memory");
+#define STORE_SHARED(buf_)                                                               \
+    _Pragma("unroll") for (int i = 0; i < LD; ++i)                                       \
+        *(uint4_t*)(smem + (buf_) * BUF + dst + i * RPI * ROWB) = stage[buf_][i];
 
     floatx16 acc[MI][NJ];
 #pragma unroll
@@ -81,69 +138,131 @@ __global__ __launch_bounds__(256, MINB) void gemm_mfma_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    LOAD_GLOBAL(0)
-    STORE_SHARED(0, 0)
-    __syncthreads();
     const int fr = lane & 31;          // row of the fragment this lane holds
     const int fk = (lane >> 5) * 16;   // byte offset of its 8 k values within a 16-wide k step
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) { LOAD_GLOBAL(kt + 1) }
-        const unsigned char* a_base = smem + buf * (BM + BN) * ROWB + (wm + fr) * ROWB + fk;
-        const unsigned char* b_base = smem + buf * (BM + BN) * ROWB + (BM + wn + fr) * ROWB + fk;
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 a[MI], b[NJ];
-#pragma unroll
-            for (int i = 0; i < MI; ++i) a[i] = *(const bf16x8*)(a_base + i * 32 * ROWB + ks * 32);
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) b[j] = *(const bf16x8*)(b_base + j * 32 * ROWB + ks * 32);
-#pragma unroll
-            for (int i = 0; i < MI; ++i)
-#pragma unroll
-                for (int j = 0; j < NJ; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nk) { STORE_SHARED(buf ^ 1, kt + 1) }   // the other buffer: its readers finished before the last barrier
-        __syncthreads();
+    const unsigned char* a_frag = smem + (wm + fr) * ROWB + fk;
+    const unsigned char* b_frag = smem + (BM + wn + fr) * ROWB + fk;
+    // One step on buffer buf_ (a constant, so every shared-memory address is base + immediate).
+    // The fragments of k step ks + 1 are read while the MFMAs of ks run, and the stores of the
+    // next step's tile are issued before the last MFMAs, whose time then covers them.
+#define READ_FRAGS(buf_, ks_, a_, b_)                                                    \
+    _Pragma("unroll") for (int i = 0; i < MI; ++i)                                       \
+        a_[i] = *(const bf16x8*)(a_frag + (buf_) * BUF + i * 32 * ROWB + (ks_) * 32);    \
+    _Pragma("unroll") for (int j = 0; j < NJ; ++j)                                       \
+        b_[j] = *(const bf16x8*)(b_frag + (buf_) * BUF + j * 32 * ROWB + (ks_) * 32);
+#define MFMAS(a_, b_)                                                                    \
+    _Pragma("unroll") for (int i = 0; i < MI; ++i)                                       \
+        _Pragma("unroll") for (int j = 0; j < NJ; ++j)                                   \
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_[j], a_[i], acc[i][j], 0, 0, 0);
+#define K_STEP(buf_, kt_)                                                                \
+    {                                                                                    \
+        bf16x8 fa[2][MI], fb[2][NJ];                                                     \
+        READ_FRAGS(buf_, 0, fa[0], fb[0])                                                \
+        LOAD_GLOBAL(buf_, (kt_) + 2)   /* this set went to shared memory a step ago */   \
+        __builtin_amdgcn_sched_barrier(0);                                               \
+        _Pragma("unroll") for (int ks = 0; ks < BK / 16 - 1; ++ks) {                     \
+            READ_FRAGS(buf_, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1])                 \
+            __builtin_amdgcn_sched_barrier(0);   /* keep the reads ahead of the MFMAs */ \
+            MFMAS(fa[ks & 1], fb[ks & 1])                                                \
+            __builtin_amdgcn_sched_barrier(0);                                           \
+        }                                                                                \
+        /* the other buffer: its readers finished before the last barrier (after the last step  \
+           this stores a step that does not exist, which nobody reads) */                    \
+        WAIT_LOADS((buf_) ^ 1, LD)   /* the LD loads just issued may stay in flight */   \
+        STORE_SHARED((buf_) ^ 1)                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                               \
+        MFMAS(fa[(BK / 16 - 1) & 1], fb[(BK / 16 - 1) & 1])                              \
+        __builtin_amdgcn_sched_barrier(0);                                               \
+        __syncthreads();                                                                 \
     }
+
+    // step kt uses buffer and register set kt % 2
+    LOAD_GLOBAL(0, 0)
+    LOAD_GLOBAL(1, 1)
+    WAIT_LOADS(0, LD)
+    STORE_SHARED(0)
+    __syncthreads();
+    // (two steps in a body without branches, and an odd last step after the loop)
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+        K_STEP(0, kt)
+        K_STEP(1, kt + 1)
+    }
+    if (kt < nk) K_STEP(0, kt)
+    // The loads past the end are still in flight and the compiler does not know of them: their
+    // registers pass through a last wait, so that they stay reserved until the loads have landed
+    // (a register whose value nobody uses would be handed out again at once).
+    WAIT_LOADS(0, 0)
+    WAIT_LOADS(1, 0)
+#undef K_STEP
+#undef READ_FRAGS
+#undef MFMAS
 #undef LOAD_GLOBAL
+#undef WAIT_LOADS
 #undef STORE_SHARED
 
     // The MFMA is given the W rows as its first operand and the x rows as its second, so its
     // result is the tile transposed: a lane holds, for the token row m = lane % 32, the outputs
-    // n = 8 b + 4 (lane / 32) + r (e = 4 b + r): four consecutive n at a time, one 8- or 16-byte store.
-    const int NO = SILU ? N / 2 : N;             // width of the output
-    const bool vec_ok = (NO % 4) == 0;
+    // n = 8 b + 4 (lane / 32) + r (e = 4 b + r), four consecutive n at a time.  Stored from there,
+    // one instruction would touch 32 rows with 16 bytes each.  So each wave turns its part round
+    // in shared memory, a strip of 32 rows at a time (the staging buffers are free: every wave has
+    // passed the loop's last barrier): it writes the strip as rows and reads it back 16 bytes a
+    // lane, so that a store instruction covers whole rows of the strip.
+    const int NO = SILU ? N / 2 : N;                       // width of the output
+    constexpr int WNO = SILU ? WN / 2 : WN;                // output columns of a wave's strip
+    constexpr int ESZ = (int)sizeof(TO);
+    constexpr int CH = 16 / ESZ;                           // outputs in 16 bytes
+    constexpr int CPR = WNO / CH;                          // 16-byte chunks in a row of the strip
+    constexpr int SROW = WNO * ESZ + 16;                   // bytes of a staged row
+    static_assert(4 * 32 * SROW <= 2 * BUF, "the strips of the four waves must fit the staging buffers");
+    unsigned char* strip = smem + wave * 32 * SROW;
+    const int no0 = SILU ? (n0 + wn) / 2 : n0 + wn;        // first output column of the wave's strip
+    const bool vec_ok = (NO % CH) == 0 && (((unsigned long)out) & 15) == 0;
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
-        const int m = m0 + wm + i * 32 + (lane & 31);
-        if (m >= M) continue;
+        __builtin_amdgcn_sched_barrier(0);   // one strip after the other: nothing of the next is computed early
 #pragma unroll
         for (int j = 0; j < NJ; j += (SILU ? 2 : 1))
 #pragma unroll
             for (int bq = 0; bq < 4; ++bq) {
-                const int nw = n0 + wn + j * 32;                       // first weight row of the MFMA tile
-                const int n = (SILU ? nw / 2 : nw) + 8 * bq + 4 * (lane >> 5);
-                if (n >= NO) continue;
+                const int nl = (SILU ? j * 16 : j * 32) + 8 * bq + 4 * (lane >> 5);   // column within the strip
                 float v[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     if (SILU) {
                         const float gt = acc[i][j][4 * bq + r], up = acc[i][j + (SILU ? 1 : 0)][4 * bq + r];
-                        v[r] = gt / (1.f + __expf(-gt)) * up;
+                        v[r] = gt * __builtin_amdgcn_rcpf(1.f + __expf(-gt)) * up;   // rcp: within 1 ulp
                     } else {
-                        v[r] = acc[i][j][4 * bq + r] + ((bias && n + r < NO) ? bias[n + r] : 0.f);
+                        v[r] = acc[i][j][4 * bq + r];
                     }
                 }
-                TO* o = out + (long)m * NO + n;
-                if (vec_ok) {
-                    Vec4<TO>::store(o, v);
-                } else {
+                if (!SILU && bias) {                       // (a column beyond the output is never stored: any bias does)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) if (n + r < NO) Elem<TO>::store(o + r, v[r]);
+                    for (int r = 0; r < 4; ++r) v[r] += bias[no0 + nl + r < NO ? no0 + nl + r : NO - 1];
                 }
+                Vec4<TO>::store((TO*)(strip + (lane & 31) * SROW) + nl, v);
             }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the wave's writes before its reads
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int c = lane; c < 32 * CPR; c += 64) {
+            const int row = c / CPR, col = (c % CPR) * CH;
+            const int m = m0 + wm + i * 32 + row, n = no0 + col;
+            if (m >= M || n >= NO) continue;
+            const uint4_t piece = *(const uint4_t*)(strip + row * SROW + col * ESZ);
+            TO* o = out + (long)m * NO + n;
+            if (vec_ok) {
+                *(uint4_t*)o = piece;                      // n + CH <= NO: both are multiples of CH
+            } else {
+                const TO* pv = (const TO*)&piece;
+#pragma unroll
+                for (int e = 0; e < CH; ++e) if (n + e < NO) o[e] = pv[e];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the reads before the next strip's writes
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 }
 
@@ -165,7 +284,7 @@ static int launch_mfma(const void* x, const void* w, const float* bias, void* ou
         attr_set = true;
     }
     gemm_mfma_kernel<TO, BM, BN, BK, MINB, SILU><<<(int)blocks, 256, shmem, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m);
+        (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n);
     QE_LAUNCH_CHECK();
     return 0;
 }
@@ -177,7 +296,7 @@ static int pick_mfma(const void* x, const void* w, const float* bias, void* out,
     const long big = (long)qe_cdiv(M, 256) * qe_cdiv(N, 128), mid = (long)qe_cdiv(M, 128) * qe_cdiv(N, 128);
     // the largest tile that still gives every compute unit two blocks (one, for the middle size)
     if (tile == 0) tile = big >= 2 * cus ? 256 : (mid >= cus ? 128 : 64);
-    if (tile == 256) return launch_mfma<TO, 256, 128, 32, 2, SILU>(x, w, bias, out, M, N, K, stream);
+    if (tile == 256) return launch_mfma<TO, 256, 128, 64, 1, SILU>(x, w, bias, out, M, N, K, stream);
     if (tile == 128) return launch_mfma<TO, 128, 128, 64, 2, SILU>(x, w, bias, out, M, N, K, stream);
     return launch_mfma<TO, 64, 128, 64, 2, SILU>(x, w, bias, out, M, N, K, stream);
 }
@@ -186,7 +305,7 @@ static int pick_mfma(const void* x, const void* w, const float* bias, void* out,
 // gate and up rows interleaved in blocks of 32, out is [M, N / 2] = silu(gate) * up.
 int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
                  int tile, bool silu, hipStream_t stream) {
-    QE_REQUIRE(K % 8 == 0, "mfma gemm: K=%d is no multiple of 8", K);
+    QE_REQUIRE(K % 8 == 0 && K >= 64 && K < (1 << 22), "mfma gemm: K=%d is no multiple of 8 in [64, 2^22)", K);
     QE_REQUIRE(tile == 0 || tile == 256 || tile == 128 || tile == 64, "mfma gemm: tile of %d rows", tile);
     if (silu) {
         QE_REQUIRE(!bias && N % 64 == 0, "mfma gemm: silu-mul takes no bias and gate|up rows in blocks of 32");
