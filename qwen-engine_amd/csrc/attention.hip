@@ -20,7 +20,7 @@ int qe_attention_decode(const void* q, void* out, const void* cache, const int* 
 
 int qe_attention_prefill(const void* q, void* out, const void* cache, const int* tiles, int num_tiles,
                          const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
-                         int Hq, int Hkv, int D, int P, float scale, int window, hipStream_t stream);
+                         int Hq, int Hkv, int D, int P, float scale, int window, int groups, hipStream_t stream);
 
 int qe_attention_prefill_tile_rows(int Hq, int Hkv);
 
@@ -31,14 +31,15 @@ extern "C" int qe_attention_prefill_rows(int Hq, int Hkv) {
 }
 
 // tiles: num_tiles pairs (first row of q, rows <= qe_attention_prefill_rows) of consecutive new
-// tokens of one request.  Takes what qe_attention_prefill_supported takes.
+// tokens of one request.  Takes what qe_attention_prefill_supported takes.  groups: wave groups
+// a block that share the key tiles between them, 1 or 2, or 0 to choose by the number of blocks.
 extern "C" int qe_attention_prefill_run(const void* q, void* out, const void* cache, const int* tiles,
                                         int num_tiles, const int* positions, const int* tok_seq,
                                         const int* block_table, int max_blocks, int Hq, int Hkv, int D, int P,
-                                        float scale, int window, hipStream_t stream) {
+                                        float scale, int window, int groups, hipStream_t stream) {
     QE_REQUIRE(num_tiles >= 0 && Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0, "prefill attention: bad sizes");
     return qe_attention_prefill(q, out, cache, tiles, num_tiles, positions, tok_seq, block_table, max_blocks,
-                                Hq, Hkv, D, P, scale, window, stream);
+                                Hq, Hkv, D, P, scale, window, groups, stream);
 }
 
 // tokens: null for all T rows of q, else n_tokens row indices.

@@ -19,6 +19,12 @@
 //       because value tiles are stored transposed ([D][P]) the A operand is two 8-byte reads
 // The causal and window limits are applied per column, so the order of the sums for a row
 // depends on its position and the window only.
+//
+// With NG = 2 a block has two such groups of four waves on the same four row tiles: group 0 takes
+// the even key tiles and group 1 the odd ones, each through shared buffers of its own, and at the
+// end group 0 merges the two partial results (maxima, sums, accumulators) through shared memory.
+// That halves the length of the longest block, which is what the time of a causal prompt hangs on
+// when there are no more blocks than compute units.  The longest blocks are started first.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -38,10 +44,10 @@ union Piece {   // a staged 16-byte piece, addressable by element for masking
 
 #define VROW 40   // bytes of a staged value row: 16 keys = 32 bytes of data + 8 of padding
 
-// Two blocks per compute unit (at most 256 registers a lane): while one block waits for its next
-// tile or at its barrier, the other computes.
-template <int D>
-__global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
+// Two waves per SIMD (at most 256 registers a lane), as two blocks of one group or one block of
+// two: while one wave waits for its next tile or at its barrier, the other computes.
+template <int D, int NG>
+__global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ tiles, const int* __restrict__ positions, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int max_blocks,
@@ -50,9 +56,11 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     constexpr int KBYTES = 32 * KROW, VBYTES = 2 * D * VROW, BUF = KBYTES + VBYTES;
     constexpr int KP = 32 * (D / 8) / 256;           // 16-byte key pieces per thread (2 for D = 128)
     constexpr int VP = 2 * D * 2 / 256;              // 16-byte value pieces per thread
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
+    __shared__ __attribute__((aligned(16))) unsigned char smem_all[NG * 2 * BUF];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = threadIdx.x / 256;                     // which half of the key tiles (NG = 2)
+    const int tid = threadIdx.x % 256, lane = tid & 63, wave = tid >> 6;
+    unsigned char* smem = smem_all + grp * 2 * BUF;
     const int g = lane >> 5, r = lane & 31;
     const int G = Hq / Hkv;
     const int GH = 32 / R;                                 // heads per wave
@@ -60,7 +68,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const int head = kvh * G + (blockIdx.y % (G / GH)) * GH + r / R;   // this lane's column: head and row
 
     // the block's four tiles belong to one request, in ascending rows; tiles of 0 rows pad the group
-    const int* bt4 = tiles + 8 * blockIdx.x;
+    const int* bt4 = tiles + 8 * (gridDim.x - 1 - blockIdx.x);   // later rows see more keys: they start first
     const int row_first = bt4[0];
     int last = 0;
 #pragma unroll
@@ -167,20 +175,29 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
         }                                                                                           \
     }
 
-    // tile j (keys kk0 + 32 j ...) uses register set and shared buffer j % 2
+    // The group's i-th tile holds the keys from kk0 + 32 (NG i + grp) on and uses register set and
+    // shared buffer i % 2.  All groups make the same number of rounds (the barriers are the
+    // block's); a round whose tile lies beyond the keys brings and computes nothing.
     const int kk0 = (kmin / 32) * 32;
-    STAGE_LOAD(0, kk0)
-    STAGE_STORE(0, 0, kk0)
-    if (kk0 + 32 < kmax) STAGE_LOAD(1, kk0 + 32)
+    const int rounds = ((kmax - kk0 + 31) / 32 + NG - 1) / NG;
+#define TILE_KEY(i_) (kk0 + 32 * (NG * (i_) + grp))
+    const int kk_first = TILE_KEY(0), kk_second = TILE_KEY(1);
+    if (kk_first < kmax) {
+        STAGE_LOAD(0, kk_first)
+        STAGE_STORE(0, 0, kk_first)
+    }
+    if (kk_second < kmax) STAGE_LOAD(1, kk_second)
     __syncthreads();
-    for (int kk2 = kk0; kk2 < kmax; kk2 += 64) {
+    for (int i2 = 0; i2 < rounds; i2 += 2) {
 #pragma unroll
       for (int buf = 0; buf < 2; ++buf) {
-        const int kk = kk2 + 32 * buf;
-        if (kk >= kmax) break;                            // the same for all threads of the block
-        if (kk + 64 < kmax) STAGE_LOAD(buf, kk + 64)      // this set's tile went to shared memory a tile ago
+        const int i = i2 + buf;
+        if (i >= rounds) break;                           // the same for all threads of the block
+        const int kk = TILE_KEY(i);
+        const int kk_1 = TILE_KEY(i + 1), kk_2 = TILE_KEY(i + 2);   // (values, not expressions in i: the macros have loops over i)
+        if (kk_2 < kmax) STAGE_LOAD(buf, kk_2)            // this set's tile went to shared memory a round ago
         __builtin_amdgcn_sched_barrier(0);                // keep the loads ahead of the computation
-        if (wave_on && kk < k_stop && kk + 32 > k_start) { // some row of the wave sees some key of the tile
+        if (wave_on && kk < k_stop && kk + 32 > k_start) { // some row of the wave sees some key of the tile (none beyond kmax)
             const unsigned char* ks_ = smem + buf * BUF + r * KROW + g * 16;
             const unsigned char* vs_ = smem + buf * BUF + KBYTES + r * VROW + g * 8;
             // all key fragments are read before the first MFMA, all value fragments before the
@@ -205,23 +222,22 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
                     vf[db][h].u[1] = *(const uint2*)(vp + 16);
                 }
 
+            // (the scores stay unscaled: the scale is positive, so it is applied to the maximum, and
+            // to each score by the multiply-add that also subtracts the maximum)
             float tmax = -INFINITY;
             if (kk >= all_lo && kk + 32 <= all_hi) {       // every column sees every key of the tile
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    s[e] *= scale_log2;
-                    tmax = fmaxf(tmax, s[e]);
-                }
+                for (int e = 0; e < 16; ++e) tmax = fmaxf(tmax, s[e]);
             } else {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int key = kk + 8 * (e >> 2) + 4 * g + (e & 3);
-                    s[e] = (key >= lo && key < hi) ? s[e] * scale_log2 : -INFINITY;
+                    s[e] = (key >= lo && key < hi) ? s[e] : -INFINITY;
                     tmax = fmaxf(tmax, s[e]);
                 }
             }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-            const float mn = fmaxf(m, tmax);
+            const float mn = fmaxf(m, tmax * scale_log2);
             const float ref = (mn == -INFINITY) ? 0.f : mn;   // a column that has seen no key yet: all weights 0
             if (__any(mn > m)) {                              // some column's maximum moved: rescale
                 const float alpha = __builtin_amdgcn_exp2f(m - ref);
@@ -234,7 +250,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
             float psum = 0.f;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const float pe = __builtin_amdgcn_exp2f(s[e] - ref);   // 0 for keys that are not seen
+                const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], scale_log2, -ref));   // 0 for keys that are not seen
                 psum += pe;
                 pb[e >> 3].v[e & 7] = (__bf16)pe;
             }
@@ -246,13 +262,44 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
                     acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][h].v, pb[h].v, acc[db], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (kk + 32 < kmax) STAGE_STORE(buf ^ 1, buf ^ 1, kk + 32)   // that buffer's readers finished before the last barrier
+        if (kk_1 < kmax) STAGE_STORE(buf ^ 1, buf ^ 1, kk_1)   // that buffer's readers finished before the last barrier
         __syncthreads();
       }
     }
 #undef STAGE_LOAD
 #undef STAGE_STORE
+#undef TILE_KEY
     l += __shfl_xor(l, 32, 64);
+    if (NG == 2) {
+        // group 1 hands its maxima, sums and accumulators to group 0, 16 values of every lane at a
+        // time, through the staging memory (free after the loop's last barrier): [wave][value][lane]
+        float* xch = (float*)smem_all + wave * 18 * 64 + lane;
+        float a_own = 1.f, a_other = 0.f;
+        if (grp == 1) { xch[0] = m; xch[64] = l; }
+        __syncthreads();
+        if (grp == 0) {
+            const float m1 = xch[0], l1 = xch[64];
+            const float mt = fmaxf(m, m1);
+            const float ref = (mt == -INFINITY) ? 0.f : mt;
+            a_own = __builtin_amdgcn_exp2f(m - ref);       // 0 for a side that has seen no key
+            a_other = __builtin_amdgcn_exp2f(m1 - ref);
+            l = l * a_own + l1 * a_other;
+        }
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db) {
+            if (grp == 1) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) xch[(2 + e) * 64] = acc[db][e];
+            }
+            __syncthreads();
+            if (grp == 0) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[db][e] = acc[db][e] * a_own + xch[(2 + e) * 64] * a_other;
+            }
+            __syncthreads();
+        }
+        if (grp == 1) return;
+    }
     if (col_ok) {
         const float inv = 1.f / l;
         bf16_t* orow = out + ((long)row * Hq + head) * D + 4 * g;
@@ -280,7 +327,7 @@ int qe_attention_prefill_tile_rows(int Hq, int Hkv) {
 // through the group; a group is filled up with pairs of 0 rows.  num_tiles is a multiple of 4.
 int qe_attention_prefill(const void* q, void* out, const void* cache, const int* tiles, int num_tiles,
                          const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
-                         int Hq, int Hkv, int D, int P, float scale, int window, hipStream_t stream) {
+                         int Hq, int Hkv, int D, int P, float scale, int window, int groups, hipStream_t stream) {
     QE_REQUIRE((D == 64 || D == 128) && P >= 16 && (P & (P - 1)) == 0 && Hq % Hkv == 0,
                "prefill attention: sizes not taken");
     int log2P = 0;
@@ -292,14 +339,17 @@ int qe_attention_prefill(const void* q, void* out, const void* cache, const int*
     QE_REQUIRE(Hkv * waves_per_kv <= 65535, "prefill attention: too many heads");
     dim3 grid(num_tiles / 4, Hkv * waves_per_kv);
     const float scale_log2 = scale * 1.4426950408889634f;
-    if (D == 128)
-        attention_prefill_kernel<128><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache,
-                                                                tiles, positions, tok_seq, block_table,
-                                                                max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R);
-    else
-        attention_prefill_kernel<64><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache,
-                                                               tiles, positions, tok_seq, block_table,
-                                                               max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R);
+    // two groups a block where the blocks do not fill the compute units twice anyway
+    // (groups: 0 = choose, 1 or 2)
+    if (groups == 0) groups = (long)grid.x * grid.y <= 256 ? 2 : 1;
+    QE_REQUIRE(groups == 1 || groups == 2, "prefill attention: %d groups a block", groups);
+#define QE_PREFILL(D_, NG_)                                                                         \
+    attention_prefill_kernel<D_, NG_><<<grid, 256 * NG_, 0, stream>>>(                              \
+        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, tiles, positions, tok_seq, block_table, \
+        max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R)
+    if (D == 128) { if (groups == 2) QE_PREFILL(128, 2); else QE_PREFILL(128, 1); }
+    else          { if (groups == 2) QE_PREFILL(64, 2); else QE_PREFILL(64, 1); }
+#undef QE_PREFILL
     QE_LAUNCH_CHECK();
     return 0;
 }

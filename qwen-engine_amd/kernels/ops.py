@@ -54,7 +54,7 @@ def load_library():
         "qe_attention_decode_supported": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_supported": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_rows": [i32, i32],
-        "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, vp],
+        "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
         "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
         "qe_qk_rope_store": [vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
@@ -336,7 +336,7 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
               out: Optional[torch.Tensor] = None, algo: int = ALGO_AUTO,
               dec_tokens: Optional[torch.Tensor] = None, max_dec_position: int = 0,
               other_tokens: Optional[torch.Tensor] = None,
-              other_tiles: Optional[torch.Tensor] = None) -> torch.Tensor:
+              other_tiles: Optional[torch.Tensor] = None, prefill_groups: int = 0) -> torch.Tensor:
     """q [T, Hq, D]; cache [pages, 2, Hkv, P, D] (key tiles [P][D], value tiles transposed [D][P]);
     positions, tok_seq int32 [T]; block_table int32 [B, max_blocks].  Token t sees the keys at
     positions max(0, p - window + 1) .. p of request tok_seq[t] (window 0: all).  The caller
@@ -346,7 +346,7 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
     their positions being max_dec_position) go to the decode kernel where it takes the sizes;
     other_tokens are the remaining rows, and other_tiles (int32 [tiles, 2]: first row, number of
     rows <= prefill_tile_rows(Hq, Hkv), consecutive tokens of one request) the same rows cut
-    for the prefill kernel.
+    for the prefill kernel (prefill_groups: its wave groups a block, 1 or 2, 0 to let it choose).
     Without the lists every row is treated alike."""
     lib = load_library()
     _need(q, "q", _ACT, (None, None, None))
@@ -394,7 +394,8 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
             _check(lib.qe_attention_prefill_run(q.data_ptr(), out.data_ptr(), cache.data_ptr(),
                                                 other_tiles.data_ptr(), other_tiles.shape[0],
                                                 positions.data_ptr(), tok_seq.data_ptr(), block_table.data_ptr(),
-                                                max_blocks, Hq, Hkv, D, P, float(scale), int(window), _stream()),
+                                                max_blocks, Hq, Hkv, D, P, float(scale), int(window),
+                                                int(prefill_groups), _stream()),
                    "attention (prefill)")
         else:
             generic(other_tokens)

@@ -480,11 +480,12 @@ def test_prefill_attention_kernel(ops, hq, hkv, d, page, window):
     for b, t in enumerate(tables):
         table[b, :len(t)] = t
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
-    out = ops.attention(torch.cat(qs).to(DEV), torch.cat(caches).to(DEV), i32(pos), i32(seq), table.to(DEV), scale,
-                        window=window, dec_tokens=i32(dec), max_dec_position=33, other_tokens=i32(other),
-                        other_tiles=i32(tiles))
-    assert not torch.isnan(out.float()).any()
-    close(out, torch.cat(want), bf)
+    for groups in (0, 1, 2):                     # wave groups a block: chosen by the kernel, one, two
+        out = ops.attention(torch.cat(qs).to(DEV), torch.cat(caches).to(DEV), i32(pos), i32(seq), table.to(DEV), scale,
+                            window=window, dec_tokens=i32(dec), max_dec_position=33, other_tokens=i32(other),
+                            other_tiles=i32(tiles), prefill_groups=groups)
+        assert not torch.isnan(out.float()).any()
+        close(out, torch.cat(want), bf)
 
 
 @pytest.mark.parametrize("key_pos", [0, 15, 16, 200, 255, 256, 299])
@@ -503,10 +504,12 @@ def test_prefill_kernel_one_far_key_decides(ops, key_pos):
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
     from qwen_engine_amd.engine.batch import prefill_tiles
     tiles = torch.tensor(prefill_tiles([(0, n)], ops.prefill_tile_rows(hq, hkv)), dtype=torch.int32).view(-1, 2).tolist()
-    out = ops.attention(q.to(DEV), cache.to(DEV), i32(list(range(first, L))), i32([0] * n), ids[None].to(DEV),
-                        1 / math.sqrt(d), dec_tokens=i32([]), other_tokens=i32(list(range(n))), other_tiles=i32(tiles))
     want = P.attention(q.float(), k.float(), v.float(), 1 / math.sqrt(d))
-    close(out, want, bf)
+    for groups in (1, 2):
+        out = ops.attention(q.to(DEV), cache.to(DEV), i32(list(range(first, L))), i32([0] * n), ids[None].to(DEV),
+                            1 / math.sqrt(d), dec_tokens=i32([]), other_tokens=i32(list(range(n))),
+                            other_tiles=i32(tiles), prefill_groups=groups)
+        close(out, want, bf)
     last_seen = max(key_pos, first) - first
     assert float((want[last_seen:, 0] - v[key_pos, 0].float()).abs().max()) < 0.05
 
