@@ -86,6 +86,14 @@ __global__ __launch_bounds__(64) void qk_rope_store_kernel(
 // taken by D / 8 lanes, each with 4 features of the first half and the 4 features 64... D / 2
 // further that rotate with them, so a wave works on 512 / D heads at a time with 8-byte
 // accesses and the norm's sum needs log2(D / 8) shuffles.  One block of 256 threads per token.
+//
+// Values go to the cache by tiles: a value tile is stored transposed, [D][P], so one token's
+// values are a column of single elements.  The blocks of 16 consecutive tokens share the work
+// on those tokens' values: each takes some of the key/value heads, reads the 16 tokens' values
+// of that head, turns them round in shared memory and writes, per feature, the run of 16
+// elements that are neighbours in the tile.  That needs the 16 tokens to lie side by side in
+// one page (consecutive slots), which is how the tokens of a prompt lie; a block of tokens that
+// do not is written element by element.
 template <typename TA>
 __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
     const TA* __restrict__ qkv, const int* __restrict__ positions,
@@ -101,7 +109,8 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
     const int width = nheads * D;
     const int s = slot ? slot[t] : -1;
     const float* cs = table ? table + (long)positions[t] * D : nullptr;
-    for (int head = threadIdx.x / lph; head < nheads; head += heads_per_pass) {
+    const int nloop = packed_out ? nheads : Hq + Hkv;   // (values go to the cache by tiles, further down)
+    for (int head = threadIdx.x / lph; head < nloop; head += heads_per_pass) {
         const bool is_q = head < Hq;
         const bool is_k = !is_q && head < Hq + Hkv;
         const TA* src = qkv + t * width + (long)head * D;
@@ -118,14 +127,7 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
             const int kh = is_k ? head - Hq : head - Hq - Hkv;
             if (is_k) {
                 dst = cache + page * (2L * Hkv * P * D) + ((long)kh * P + off) * D;
-            } else {   // value tile is [D][P]: a column of single elements
-                TA* vt = cache + page * (2L * Hkv * P * D) + ((long)(Hkv + kh) * P) * D + off;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    Elem<TA>::store(vt + (long)(4 * j + e) * P, a[e]);
-                    Elem<TA>::store(vt + (long)(half + 4 * j + e) * P, b[e]);
-                }
-            }
+            }                                               // (values: below, by tiles)
         }
         const bool is_v = !is_q && !is_k;
         if (is_v) {
@@ -164,6 +166,54 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
             Vec4<TA>::store(dst + half + 4 * j, b);
         }
     }
+    if (packed_out || !slot) return;
+
+    // ---- values of the 16 tokens t0 .. t0 + n - 1, key/value heads t - t0, t - t0 + n, ... ----
+    extern __shared__ __attribute__((aligned(16))) unsigned char vsh[];   // [D][16] elements + 16 bytes a row
+    const int srow = 16 * (int)sizeof(TA) + 16;
+    const long t0 = t / 16 * 16;
+    const int n = (int)((long)gridDim.x - t0 < 16 ? (long)gridDim.x - t0 : 16);
+    const int s0 = slot[t0];
+    bool run = s0 >= 0 && s0 % P + n <= P;                 // side by side in one page?
+    for (int i = 1; i < n; ++i) run = run && slot[t0 + i] == s0 + i;
+    const int cpr = D / 8;                                 // 8-element chunks in a head
+    for (int kh = (int)(t - t0); kh < Hkv; kh += n) {
+        const TA* src = qkv + t0 * width + (long)(Hq + Hkv + kh) * D;
+        if (run) {
+            __syncthreads();                               // the last head's readers are done
+            for (int idx = threadIdx.x; idx < n * cpr; idx += 256) {
+                const int i = idx / cpr, c = idx % cpr;
+                float x[8];
+                Vec4<TA>::load(src + (long)i * width + 8 * c, *(float(*)[4])x);
+                Vec4<TA>::load(src + (long)i * width + 8 * c + 4, *(float(*)[4])(x + 4));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) Elem<TA>::store((TA*)(vsh + (8 * c + e) * srow) + i, x[e]);
+            }
+            __syncthreads();
+            TA* vt = cache + (long)(s0 / P) * (2L * Hkv * P * D) + ((long)(Hkv + kh) * P) * D + s0 % P;
+            const bool vec = n == 16 && P % 4 == 0 && (s0 % P) % 4 == 0;   // whole aligned groups of four
+            for (int idx = threadIdx.x; idx < D * 4; idx += 256) {  // feature d, tokens 4 q .. 4 q + 3
+                const int d = idx / 4, q4 = idx % 4;
+                const TA* from = (const TA*)(vsh + d * srow) + 4 * q4;
+                TA* to = vt + (long)d * P + 4 * q4;
+                if (vec) {
+                    float x[4];
+                    Vec4<TA>::load(from, x);
+                    Vec4<TA>::store(to, x);
+                } else {
+                    for (int e = 0; e < 4; ++e) if (4 * q4 + e < n) to[e] = from[e];
+                }
+            }
+        } else {
+            for (int idx = threadIdx.x; idx < n * D; idx += 256) {
+                const int i = idx / D, d = idx % D;
+                const int si = slot[t0 + i];
+                if (si >= 0)
+                    cache[(long)(si / P) * (2L * Hkv * P * D) + ((long)(Hkv + kh) * P) * D + (long)d * P + si % P] =
+                        src[(long)i * width + d];
+            }
+        }
+    }
 }
 
 extern "C" int qe_qk_rope_store(const void* qkv, const int* positions, const float* q_w, const float* k_w,
@@ -183,11 +233,11 @@ extern "C" int qe_qk_rope_store(const void* qkv, const int* positions, const flo
     if ((long)T * (Hq + 2 * Hkv) > 2048 && D % 8 == 0 && lph >= 1 && lph <= 64 && (lph & (lph - 1)) == 0 &&
         (!table || rotary_dim == D)) {
         if (dt_a == QE_F32)
-            qk_rope_store_vec_kernel<float><<<T, 256, 0, stream>>>(
+            qk_rope_store_vec_kernel<float><<<T, 256, (size_t)D * (16 * 4 + 16), stream>>>(
                 (const float*)qkv, positions, q_w, k_w, eps, table, slot, (float*)cache, (float*)q_out,
                 (float*)packed_out, Hq, Hkv, D, P);
         else if (dt_a == QE_BF16)
-            qk_rope_store_vec_kernel<bf16_t><<<T, 256, 0, stream>>>(
+            qk_rope_store_vec_kernel<bf16_t><<<T, 256, (size_t)D * (16 * 2 + 16), stream>>>(
                 (const bf16_t*)qkv, positions, q_w, k_w, eps, table, slot, (bf16_t*)cache, (bf16_t*)q_out,
                 (bf16_t*)packed_out, Hq, Hkv, D, P);
         else

@@ -242,6 +242,55 @@ def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, page):
     close(no_norm, P.apply_rope(table, pos, q), dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,d,page", [(16, 8, 128, 16), (4, 2, 64, 32), (12, 4, 16, 16), (6, 1, 128, 20), (20, 20, 32, 8)])
+def test_qk_norm_rope_store_of_many_tokens(ops, dtype, hq, hkv, d, page):
+    """Enough tokens for the kernel that takes a token per block and writes values by tiles of 16
+    tokens: a prompt from a page's start, one from the middle of a page, tokens whose slots are
+    scattered, tokens without a slot, and a last tile of fewer than 16 tokens."""
+    eps = 1e-6
+    lens = [(0, 150), (page // 2 + 1, 100), (3, 16)]                  # (first position, tokens) of three requests
+    T = sum(n for _, n in lens) + 24
+    width = (hq + 2 * hkv) * d
+    assert T * (hq + 2 * hkv) > 2048
+    qkv = rand(T, width, seed=73, dtype=dtype)
+    qw, kw = 1 + rand(d, seed=74, scale=0.1), 1 + rand(d, seed=75, scale=0.1)
+    table = P.rope_table(10000.0, d, 256)
+    pages = 40
+    perm = torch.randperm(pages, generator=torch.Generator().manual_seed(76)).tolist()
+    pos, slots = [], []
+    for first, n in lens:                                             # consecutive slots through pages of its own
+        mine = [perm.pop() for _ in range((first + n + page - 1) // page)]
+        for p_ in range(first, first + n):
+            pos.append(p_)
+            slots.append(mine[p_ // page] * page + p_ % page)
+    free = [pg * page + o for pg in perm[:4] for o in range(page)]
+    g = torch.Generator().manual_seed(77)
+    pick = torch.randperm(len(free), generator=g)[:24].tolist()
+    for i in range(24):                                               # scattered, and every fifth without a slot
+        pos.append(100 + i)
+        slots.append(-1 if i % 5 == 4 else free[pick[i]])
+    pos, slots = torch.tensor(pos, dtype=torch.int32), torch.tensor(slots, dtype=torch.int32)
+    cache = torch.zeros(pages, 2, hkv, page, d, dtype=dtype, device=DEV)
+    q_out = ops.qk_rope_store(qkv.to(DEV), hq, hkv, d, pos.to(DEV), qw.to(DEV), kw.to(DEV), eps,
+                              table.to(DEV), slots.to(DEV), cache, page)
+    x = qkv.float()
+    q = x[:, :hq * d].view(T, hq, d)
+    k = x[:, hq * d:(hq + hkv) * d].view(T, hkv, d)
+    v = x[:, (hq + hkv) * d:].view(T, hkv, d)
+    close(q_out, P.apply_rope(table, pos, P.rms_norm(q, qw, eps)), dtype)
+    k_ref = P.apply_rope(table, pos, P.rms_norm(k, kw, eps))
+    want = torch.zeros(pages, 2, hkv, page, d)
+    want_vt = want[:, 1].view(pages, hkv, d, page)
+    for t in range(T):
+        s = int(slots[t])
+        if s >= 0:
+            want[s // page, 0, :, s % page] = k_ref[t]
+            want_vt[s // page, :, :, s % page] = v[t]
+    close(cache, want, dtype)
+    assert torch.equal(cache[:, 1].float().cpu(), want[:, 1].to(dtype).float())      # values are copied exactly
+
+
 def test_argmax_takes_the_lowest_index_on_ties(ops):
     logits = rand(5, 50000, seed=80)
     logits[0, 49999] = 9.0
