@@ -33,7 +33,8 @@ extern "C" int qe_gemm_partial_splits(int N, int K) { return qe_gemm_skinny_spli
 // 4: as 2 with the gate and up rows of w interleaved in blocks of 32 (gate 0..31, up 0..31, ...);
 //    taken by the kernel for few rows and by the tiled one.
 // algo: 0 = choose, 1 = the generic 32-bit kernel, 2 = an MFMA kernel (the one for few rows up to
-// 64 rows, the tiled one above) or an error if neither takes the operands.
+// 64 rows, except against a very wide matrix from 17 rows on; else the tiled one) or an error if
+// neither takes the operands.
 extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                        int dt_a, int dt_w, int dt_o, int algo, int epilogue, int splits, hipStream_t stream) {
     QE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -55,7 +56,11 @@ extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* ou
         return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, algo - ALGO_TILE, false, stream);
     }
     if (algo != ALGO_GENERIC) {
-        if (skinny) return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, EPI_STORE, 1, stream);
+        // more than 16 rows against a very wide matrix (the logits of a large batch): the kernel for
+        // few rows passes over the weights once per 16 rows' worth of arithmetic and falls behind
+        // the memory there; the tiled kernel streams them once
+        if (skinny && !(tiled && M > 16 && N >= 32768))
+            return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, EPI_STORE, 1, stream);
         if (tiled) return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, 0, false, stream);
         QE_REQUIRE(algo == ALGO_AUTO, "gemm: M=%d N=%d K=%d with these element types is not taken by an MFMA kernel", M, N, K);
     }

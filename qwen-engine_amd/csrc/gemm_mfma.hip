@@ -267,7 +267,7 @@ __global__ __launch_bounds__(256, MINB) void gemm_mfma_kernel(
 }
 
 bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w) {
-    return dt_a == QE_BF16 && dt_w == QE_BF16 && M > 64 && K % 8 == 0 && K >= 64;
+    return dt_a == QE_BF16 && dt_w == QE_BF16 && M > 16 && K % 8 == 0 && K >= 64;
 }
 
 template <typename TO, int BM, int BN, int BK, int MINB, bool SILU>
@@ -295,7 +295,7 @@ static int pick_mfma(const void* x, const void* w, const float* bias, void* out,
     const long cus = 256;
     const long big = (long)qe_cdiv(M, 256) * qe_cdiv(N, 128), mid = (long)qe_cdiv(M, 128) * qe_cdiv(N, 128);
     // the largest tile that still gives every compute unit two blocks (one, for the middle size)
-    if (tile == 0) tile = big >= 2 * cus ? 256 : (mid >= cus ? 128 : 64);
+    if (tile == 0) tile = (big >= 2 * cus && M > 128) ? 256 : ((mid >= cus && M > 64) ? 128 : 64);   // never taller than the rows need
     if (tile == 256) return launch_mfma<TO, 256, 128, 64, 1, SILU>(x, w, bias, out, M, N, K, stream);
     if (tile == 128) return launch_mfma<TO, 128, 128, 64, 2, SILU>(x, w, bias, out, M, N, K, stream);
     return launch_mfma<TO, 64, 128, 64, 2, SILU>(x, w, bias, out, M, N, K, stream);

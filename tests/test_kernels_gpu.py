@@ -470,7 +470,7 @@ def test_decode_kernel_one_far_key_decides(ops, key_pos):
 
 
 @pytest.mark.parametrize("M,N,K", [(65, 64, 64), (128, 128, 64), (200, 331, 96), (257, 500, 160), (2048, 1024, 1024),
-                                   (300, 3072, 1024), (130, 152, 2048)])
+                                   (300, 3072, 1024), (130, 152, 2048), (17, 200, 64), (33, 40000, 96)])
 def test_gemm_tiled_mfma(ops, M, N, K):
     bf = torch.bfloat16
     x, w = rand(M, K, seed=110, dtype=bf), rand(N, K, seed=111, dtype=bf, scale=0.1)
