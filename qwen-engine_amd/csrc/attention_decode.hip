@@ -84,6 +84,207 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     }
 }
 
+// ---- the same with the step before it folded in ---------------------------------------------
+// The q/k norm, the rotation and the cache write of the new token cost a kernel of their own
+// that runs a few microseconds for a few kilobytes.  Here every wave norms and rotates the query
+// heads it needs itself, straight from the q|k|v rows (the pairs d, d + D/2 of the rotation lie in
+// the same lane in the MFMA operand layout), and the wave whose split holds the token's own
+// position also norms and rotates the new key, takes it and the new value into its softmax from
+// registers (the cached keys it reads stop before that position), and writes both to the cache.
+// Roundings are where the separate kernels have them: q and k to bfloat16 after the rotation,
+// the probability to bfloat16 before it meets the value.
+
+// One head's features c * 32 + g * 8 + e in the MFMA operand layout: fetch() issues the loads (the
+// head, the norm's weights, the position's row [cos | sin] of the table), finish() does the
+// RMSNorm (w) and the rotation (cs), each optional, and rounds to bfloat16.  Apart, so that the
+// loads of the first key tiles can be issued between the two.
+template <int D>
+struct NormRotate {
+    static constexpr int H = D / 64;                       // chunk c and chunk c + H rotate together
+    bf16x8 raw[D / 32];
+    float wv[D / 32][8], co[H][8], sn[H][8];
+    __device__ __forceinline__ void fetch(const bf16_t* __restrict__ src, bool active, const float* __restrict__ w,
+                                          const float* __restrict__ cs, int g) {
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c) {
+            raw[c] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (active) raw[c] = *(const bf16x8*)(src + c * 32 + g * 8);
+        }
+        if (w) {
+#pragma unroll
+            for (int c = 0; c < D / 32; ++c) {
+                Vec4<float>::load(w + c * 32 + g * 8, *(float(*)[4])wv[c]);
+                Vec4<float>::load(w + c * 32 + g * 8 + 4, *(float(*)[4])(wv[c] + 4));
+            }
+        }
+        if (cs) {
+#pragma unroll
+            for (int c = 0; c < H; ++c) {
+                Vec4<float>::load(cs + c * 32 + g * 8, *(float(*)[4])co[c]);
+                Vec4<float>::load(cs + c * 32 + g * 8 + 4, *(float(*)[4])(co[c] + 4));
+                Vec4<float>::load(cs + D / 2 + c * 32 + g * 8, *(float(*)[4])sn[c]);
+                Vec4<float>::load(cs + D / 2 + c * 32 + g * 8 + 4, *(float(*)[4])(sn[c] + 4));
+            }
+        }
+    }
+    __device__ __forceinline__ void finish(bf16x8 (&out)[D / 32], bool has_w, float eps, bool has_cs) {
+        float x[D / 32][8];
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[c][e] = (float)raw[c][e];
+        if (has_w) {
+            float ss = 0.f;
+#pragma unroll
+            for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss += x[c][e] * x[c][e];
+            ss += __shfl_xor(ss, 16, 64);
+            ss += __shfl_xor(ss, 32, 64);
+            const float rstd = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+            for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[c][e] = x[c][e] * rstd * wv[c][e];
+        }
+        if (has_cs) {
+#pragma unroll
+            for (int c = 0; c < H; ++c)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float x1 = x[c][e], x2 = x[c + H][e];
+                    x[c][e] = co[c][e] * x1 - sn[c][e] * x2;
+                    x[c + H][e] = sn[c][e] * x1 + co[c][e] * x2;
+                }
+        }
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) out[c][e] = (__bf16)x[c][e];
+    }
+};
+
+template <int D, int SPLIT>
+__global__ __launch_bounds__(64) void attention_decode_fused_split_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* cache,
+    const int* __restrict__ dec_tokens, const int* __restrict__ positions, const int* __restrict__ tok_seq,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ slots,
+    const float* __restrict__ q_w, const float* __restrict__ k_w, float eps, const float* __restrict__ table,
+    float* __restrict__ part_acc, float* __restrict__ part_ml,
+    int Hq, int Hkv, int P, float scale, int window, int num_splits) {
+    const int lane = threadIdx.x, g = lane >> 4, n = lane & 15;
+    const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
+    const int G = Hq / Hkv;
+    const int t = dec_tokens[di];
+    const int p = positions[t];
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const bool own = split == p / SPLIT;                   // this wave takes the token's own key and value
+    const int k_begin = max(split * SPLIT, lo);
+    const int k_end = min((split + 1) * SPLIT, p);         // cached keys: the token's own is not among them
+    const int head = kvh * G + n;
+    const bool head_ok = n < G;
+    float* pacc = part_acc + (((long)di * Hq + head) * num_splits + split) * D;
+    float* pml = part_ml + (((long)di * Hq + head) * num_splits + split) * 2;
+    if (k_begin >= k_end && !own) {   // nothing of this split is seen by the token
+        if (head_ok && g == 0) { pml[0] = -INFINITY; pml[1] = 0.f; }
+        return;
+    }
+    const long width = (long)(Hq + 2 * Hkv) * D;
+    const float* cs = table ? table + (long)p * D : nullptr;
+    const long page_stride = 2L * Hkv * P * D;
+
+    AttnState<D> st;
+    st.init();
+    bf16x8 qreg[D / 32];
+    if (k_begin < k_end) {
+        const int* bt = block_table + (long)tok_seq[t] * max_blocks;
+        const int tile0 = (k_begin - split * SPLIT) / 16;
+        const int tile1 = (k_end - split * SPLIT + 15) / 16;
+        int my_page = 0;
+        if (lane >= tile0 && lane < tile1) my_page = bt[(split * SPLIT + lane * 16) / P];
+#define LOAD(buf_, i_) load_tile<D>(buf_, cache, __builtin_amdgcn_readlane(my_page, (i_)), page_stride, kvh, Hkv, P, \
+                                    (split * SPLIT + (i_) * 16) % P, g, n)
+#define STEP(buf_, i_) attn_tile_step<D>(st, buf_, qreg, scale, split * SPLIT + (i_) * 16, g, k_begin, k_end, k_begin, k_end)
+        KVTile<D> ta, tb;
+        int i = tile0;
+        NormRotate<D> nq;
+        nq.fetch(qkv + t * width + (long)head * D, head_ok, q_w, cs, g);
+        LOAD(ta, i);                                       // the first tiles travel while q is prepared
+        if (i + 1 < tile1) LOAD(tb, i + 1);
+        nq.finish(qreg, q_w != nullptr, eps, cs != nullptr);
+        while (true) {
+            STEP(ta, i);
+            if (++i >= tile1) break;
+            if (i + 1 < tile1) LOAD(ta, i + 1);
+            STEP(tb, i);
+            if (++i >= tile1) break;
+            if (i + 1 < tile1) LOAD(tb, i + 1);
+        }
+#undef LOAD
+#undef STEP
+    } else {
+        NormRotate<D> nq;
+        nq.fetch(qkv + t * width + (long)head * D, head_ok, q_w, cs, g);
+        nq.finish(qreg, q_w != nullptr, eps, cs != nullptr);
+    }
+    if (own) {
+        bf16x8 kreg[D / 32];
+        NormRotate<D> nk;
+        nk.fetch(qkv + t * width + (long)(Hq + kvh) * D, true, k_w, cs, g);
+        nk.finish(kreg, k_w != nullptr, eps, cs != nullptr);
+        float dot = 0.f;
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dot += (float)qreg[c][e] * (float)kreg[c][e];
+        dot += __shfl_xor(dot, 16, 64);
+        dot += __shfl_xor(dot, 32, 64);
+        const float s_new = dot * scale;
+        const float mn = fmaxf(st.m, s_new);
+        const float alpha = __expf(st.m - mn);             // 0 when no cached key was seen
+        const float pn = __expf(s_new - mn);
+        const float pn_b = (float)(__bf16)pn;
+        st.l = st.l * alpha + (g == 0 ? pn : 0.f);         // (a lane's share of the sum: once per column)
+        st.m = mn;
+        const bf16_t* vsrc = qkv + t * width + (long)(Hq + Hkv + kvh) * D;
+#pragma unroll
+        for (int db = 0; db < D / 16; ++db) {
+            const short4_t vv = *(const short4_t*)(vsrc + db * 16 + g * 4);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                st.acc[db][j] = st.acc[db][j] * alpha + pn_b * bf16_bits_to_float((unsigned short)vv[j]);
+        }
+        const int slot = slots ? slots[t] : -1;
+        if (slot >= 0) {
+            const long page = slot / P;
+            const int off = slot % P;
+            if (n == 0) {
+#pragma unroll
+                for (int c = 0; c < D / 32; ++c)
+                    *(bf16x8*)(cache + page * page_stride + ((long)kvh * P + off) * D + c * 32 + g * 8) = kreg[c];
+            }
+            if (n < D / 16) {                              // the value tile is [D][P]: a column of single elements
+                bf16_t* vt = cache + page * page_stride + ((long)(Hkv + kvh) * P) * D + off;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int d = n * 16 + g * 4 + j;
+                    vt[(long)d * P] = vsrc[d];
+                }
+            }
+        }
+    }
+    float l = st.l;
+    const float m = st.m;
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (head_ok) {
+#pragma unroll
+        for (int db = 0; db < D / 16; ++db)
+            *(floatx4*)(pacc + db * 16 + g * 4) = st.acc[db];
+        if (g == 0) { pml[0] = m; pml[1] = l; }
+    }
+}
+
 // out[t, head, :] = sum_s e^{m_s - M} acc_s / sum_s e^{m_s - M} l_s,  M = max_s m_s.
 // One block of 256 threads per (token, head): wave w sums the splits w, w + 4, ... in ascending
 // order, the four sums are added in the order of the waves.
@@ -175,6 +376,43 @@ int qe_attention_decode(const void* q, void* out, const void* cache, const int* 
     else if (split_keys == 128) QE_DECODE(64, 128);
     else QE_DECODE(64, 256);
 #undef QE_DECODE
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// The fused form: qkv [T, (Hq + 2 Hkv) D] as the projection left it; q_w, k_w (per-head norm weights)
+// and table (rows [cos | sin] of D floats per position) may be null; slots: the cache slot of each
+// row's own key and value (negative: not written).  Every row named in dec_tokens brings exactly
+// its own new key; the cache holds the keys before it.
+int qe_attention_decode_fused(const void* qkv, void* out, void* cache, const int* dec_tokens, int n_dec,
+                              const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
+                              const int* slots, const float* q_w, const float* k_w, float eps, const float* table,
+                              int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
+                              int split_keys, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    QE_REQUIRE(qe_attention_decode_ok(Hq, Hkv, D, P, QE_BF16), "decode attention: sizes not taken");
+    QE_REQUIRE(split_keys == 128 || split_keys == 256, "decode attention: splits of 128 or 256 keys, not %d", split_keys);
+    if (n_dec == 0) return 0;
+    const int num_splits = max_position / split_keys + 1;
+    QE_REQUIRE(num_splits <= 65535 && n_dec <= 65535, "decode attention: too many splits or tokens");
+    QE_REQUIRE(workspace_bytes >= qe_attention_decode_workspace(n_dec, Hq, D, num_splits),
+               "decode attention: workspace of %zu bytes is too small", workspace_bytes);
+    float* part_acc = (float*)workspace;
+    float* part_ml = part_acc + (size_t)n_dec * Hq * num_splits * D;
+    dim3 grid(num_splits, Hkv, n_dec);
+    dim3 mgrid(n_dec, Hq);
+#define QE_DECODE_FUSED(D_, S_)                                                                         \
+    do {                                                                                                \
+        attention_decode_fused_split_kernel<D_, S_><<<grid, 64, 0, stream>>>(                           \
+            (const bf16_t*)qkv, (bf16_t*)cache, dec_tokens, positions, tok_seq, block_table, max_blocks, \
+            slots, q_w, k_w, eps, table, part_acc, part_ml, Hq, Hkv, P, scale, window, num_splits);     \
+        attention_decode_merge_kernel<D_><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, dec_tokens,     \
+                                                                     (bf16_t*)out, Hq, num_splits);     \
+    } while (0)
+    if (D == 128 && split_keys == 128) QE_DECODE_FUSED(128, 128);
+    else if (D == 128) QE_DECODE_FUSED(128, 256);
+    else if (split_keys == 128) QE_DECODE_FUSED(64, 128);
+    else QE_DECODE_FUSED(64, 256);
+#undef QE_DECODE_FUSED
     QE_LAUNCH_CHECK();
     return 0;
 }

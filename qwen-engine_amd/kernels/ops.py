@@ -56,6 +56,8 @@ def load_library():
         "qe_attention_prefill_rows": [i32, i32],
         "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
         "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
+        "qe_attention_decode_fused_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, f32, vp,
+                                          i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
         "qe_qk_rope_store": [vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
         "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
@@ -399,6 +401,66 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
                    "attention (prefill)")
         else:
             generic(other_tokens)
+    return out
+
+
+def attention_decode_fused_supported(qkv: torch.Tensor, cache: torch.Tensor, num_heads: int,
+                                     table: Optional[torch.Tensor]) -> bool:
+    """True if attention_decode_fused takes these operands: the sizes of the decode kernel, and a
+    rotation (if any) over the whole head."""
+    lib = load_library()
+    D = cache.shape[4]
+    return (qkv.dtype == torch.bfloat16 and (table is None or table.shape[1] == D) and
+            bool(lib.qe_attention_decode_supported(num_heads, cache.shape[2], D, cache.shape[3], _DT[qkv.dtype])))
+
+
+def attention_decode_fused(qkv: torch.Tensor, num_heads: int, cache: torch.Tensor, positions: torch.Tensor,
+                           tok_seq: torch.Tensor, block_table: torch.Tensor, scale: float, window: int,
+                           dec_tokens: torch.Tensor, max_dec_position: int,
+                           q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                           table: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention of single new tokens with the step before it inside: per-head q/k RMSNorm
+    (weights or None), half-split rotation from ``table`` (rows [cos | sin] of the head size, or
+    None) and the write of each token's key and value to cache slot ``slots[t]`` (negative or no
+    slots: not written).  qkv [T, (Hq + 2 Hkv) D] bfloat16; the rows ``dec_tokens`` are computed
+    into out [T, Hq, D]; the cache holds each request's keys before the token's own position."""
+    lib = load_library()
+    _need(qkv, "qkv", torch.bfloat16, (None, None))
+    T, dev = qkv.shape[0], qkv.device
+    _need(cache, "cache", torch.bfloat16, (None, 2, None, None, None), dev)
+    Hkv, P, D = cache.shape[2], cache.shape[3], cache.shape[4]
+    Hq = int(num_heads)
+    if qkv.shape[1] != (Hq + 2 * Hkv) * D:
+        raise KernelError(f"attention_decode_fused: qkv rows of {qkv.shape[1]} are not ({Hq} + 2 * {Hkv}) * {D}")
+    if not attention_decode_fused_supported(qkv, cache, Hq, table):
+        raise KernelError("attention_decode_fused: sizes not taken")
+    _need(positions, "positions", torch.int32, (T,), dev)
+    _need(tok_seq, "tok_seq", torch.int32, (T,), dev)
+    _need(block_table, "block_table", torch.int32, (None, None), dev)
+    _need(dec_tokens, "dec_tokens", torch.int32, (None,), dev)
+    if q_weight is not None:
+        _need(q_weight, "q_weight", torch.float32, (D,), dev)
+    if k_weight is not None:
+        _need(k_weight, "k_weight", torch.float32, (D,), dev)
+    if table is not None:
+        _need(table, "table", torch.float32, (None, D), dev)
+    if slots is not None:
+        _need(slots, "slots", torch.int32, (T,), dev)
+    if out is None:
+        out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=dev)
+    _need(out, "out", torch.bfloat16, (T, Hq, D), dev)
+    n_dec = dec_tokens.shape[0]
+    if n_dec == 0:
+        return out
+    nbytes = lib.qe_attention_decode_workspace_bytes(n_dec, Hq, D, int(max_dec_position), DECODE_SPLIT_KEYS)
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+    _check(lib.qe_attention_decode_fused_run(qkv.data_ptr(), out.data_ptr(), cache.data_ptr(), dec_tokens.data_ptr(),
+                                             n_dec, positions.data_ptr(), tok_seq.data_ptr(), block_table.data_ptr(),
+                                             block_table.shape[1], _ptr(slots), _ptr(q_weight), _ptr(k_weight),
+                                             float(eps), _ptr(table), Hq, Hkv, D, P, float(scale), int(window),
+                                             int(max_dec_position), DECODE_SPLIT_KEYS, ws.data_ptr(), nbytes,
+                                             _stream()), "attention (decode, fused)")
     return out
 
 

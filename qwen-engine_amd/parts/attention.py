@@ -18,6 +18,12 @@ from .base import CacheBinding, Runtime, TensorInfo
 from .registry import build_part, register_part
 
 
+# Up to this many single new tokens in a step, the decode attention kernel norms, rotates and
+# writes the cache itself; above, the separate kernel is quicker (every wave of the attention
+# kernel repeats the preparation of q, which then outweighs the kernel saved).
+FUSED_DECODE_MAX_TOKENS = 16
+
+
 class PagedAttention:
     def __init__(self, spec, hidden_size: int):
         self.spec = spec
@@ -91,6 +97,16 @@ class PagedAttention:
             if table is not None and ctx.max_position >= table.shape[0]:
                 raise RuntimeError(f"position {ctx.max_position} is beyond the rotation table "
                                    f"({table.shape[0]} positions)")
+            only_new_tokens = (ctx.dec_tokens is not None and ctx.dec_tokens.shape[0] == T and
+                               (ctx.other_tokens is None or ctx.other_tokens.shape[0] == 0))
+            if (only_new_tokens and T <= FUSED_DECODE_MAX_TOKENS and binding.write and
+                    ops.attention_decode_fused_supported(qkv, cache, self.hq, table)):
+                # every row is the one new token of its request: norm, rotation and cache write
+                # happen inside the attention kernel
+                o = ops.attention_decode_fused(qkv, self.hq, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g],
+                                               self.scale, self.window, ctx.dec_tokens, ctx.max_dec_position,
+                                               self.q_norm, self.k_norm, eps, table, slots)
+                return self._project_out(o.view(T, self.hq * self.d))
             q = ops.qk_rope_store(qkv, self.hq, self.hkv, self.d, ctx.positions, self.q_norm, self.k_norm,
                                   eps, table, slots, cache, ctx.page_size)
         else:
@@ -105,7 +121,9 @@ class PagedAttention:
                           dec_tokens=ctx.dec_tokens, max_dec_position=ctx.max_dec_position,
                           other_tokens=ctx.other_tokens,
                           other_tiles=ctx.other_tiles(ops.prefill_tile_rows(self.hq, self.hkv)))
-        o = o.view(T, self.hq * self.d)
+        return self._project_out(o.view(T, self.hq * self.d))
+
+    def _project_out(self, o: torch.Tensor) -> torch.Tensor:
         if ops.gemm_fused_supported(o, self.w_o):
             # few rows: the product is cut along K to fill the chip; the norm that follows adds the parts
             return ops.gemm(o, self.w_o, epilogue=ops.EPI_PARTIAL)

@@ -451,6 +451,91 @@ def test_decode_attention_kernel(ops, hq, hkv, d, page, window):
     close(out2, torch.cat(want), bf)
 
 
+@pytest.mark.parametrize("hq,hkv,d,page", [(16, 8, 128, 16), (4, 4, 64, 16), (8, 1, 128, 32), (6, 2, 64, 48), (16, 1, 64, 16)])
+@pytest.mark.parametrize("window", [0, 40])
+@pytest.mark.parametrize("norm,rope", [(True, True), (False, True), (True, False)])
+def test_decode_attention_with_norm_rotation_and_cache_write_inside(ops, hq, hkv, d, page, window, norm, rope):
+    """Single new tokens at positions that are first in the cache, first of a page, first and last
+    of a split of 128 keys and in the middle of one: the kernel that norms and rotates q and k
+    itself, takes the new key and value from registers and writes them to the cache, against the
+    plain functions; and against the separate kernels on the same operands."""
+    bf = torch.bfloat16
+    scale, eps = 1 / math.sqrt(d), 1e-6
+    positions = [0, 1, page, 127, 128, 129, 255, 256, 300, 700]
+    B = len(positions)
+    width = (hq + 2 * hkv) * d
+    qkv = rand(B, width, seed=510, dtype=bf)
+    qw = 1 + rand(d, seed=511, scale=0.1) if norm else None
+    kw = 1 + rand(d, seed=512, scale=0.1) if norm else None
+    table = P.rope_table(10000.0, d, 1024) if rope else None
+    caches, tables, slots, want, k_new, base = [], [], [], [], [], 0
+    for b, p in enumerate(positions):
+        L = p + 1
+        k, v = rand(L, hkv, d, seed=520 + b, dtype=bf), rand(L, hkv, d, seed=540 + b, dtype=bf)
+        x = qkv[b].float()
+        q_b = x[:hq * d].view(1, hq, d)
+        k_b = x[hq * d:(hq + hkv) * d].view(1, hkv, d)
+        v_b = x[(hq + hkv) * d:].view(1, hkv, d)
+        pos_b = torch.tensor([p], dtype=torch.int32)
+        if norm:
+            q_b, k_b = P.rms_norm(q_b, qw, eps), P.rms_norm(k_b, kw, eps)
+        if rope:
+            q_b, k_b = P.apply_rope(table, pos_b, q_b), P.apply_rope(table, pos_b, k_b)
+        q_b, k_b = q_b.to(bf).float(), k_b.to(bf).float()
+        k_new.append(k_b[0])
+        keys = torch.cat([k[:p].float(), k_b]) if p else k_b
+        vals = torch.cat([v[:p].float(), v_b]) if p else v_b
+        want.append(P.attention(q_b, keys, vals, scale, window=window or None))
+        # the cache holds the keys before p; the slot of p itself holds NaN until the kernel writes it
+        k[p], v[p] = float("nan"), float("nan")
+        cache, ids = paged_cache(k, v, page, 560 + b, bf)
+        tables.append(ids + base)
+        slots.append(int(ids[p // page] + base) * page + p % page)
+        base += cache.shape[0]
+        caches.append(cache)
+    slots[4] = -1                                            # one token without a slot: nothing is written for it
+    cache = torch.cat(caches)
+    width_t = max(len(t) for t in tables)
+    tab = torch.full((B, width_t), -1, dtype=torch.int32)
+    for b, t in enumerate(tables):
+        tab[b, :len(t)] = t
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    dev = lambda t: None if t is None else t.to(DEV)
+    cd = cache.to(DEV)
+    assert ops.attention_decode_fused_supported(qkv.to(DEV), cd, hq, dev(table))
+    out = ops.attention_decode_fused(qkv.to(DEV), hq, cd, i32(positions), i32(list(range(B))), tab.to(DEV), scale,
+                                     window, i32(list(range(B))), max(positions), dev(qw), dev(kw), eps, dev(table),
+                                     i32(slots))
+    assert not torch.isnan(out.float()).any()
+    close(out, torch.cat(want), bf)
+    # the cache afterwards: the new key (normed, rotated) and value at the slot, nothing else touched
+    after = cd.cpu()
+    vt_after = after[:, 1].reshape(after.shape[0], hkv, d, page)
+    x = qkv.float()
+    for b, p in enumerate(positions):
+        s = slots[b]
+        if s < 0:
+            continue
+        close(after[s // page, 0, :, s % page], k_new[b], bf)
+        assert torch.equal(vt_after[s // page, :, :, s % page].float(), x[b, (hq + hkv) * d:].view(hkv, d))
+    untouched = torch.ones_like(cache, dtype=torch.bool)
+    vt_mask = untouched[:, 1].view(cache.shape[0], hkv, d, page)
+    for s in slots:
+        if s >= 0:
+            untouched[s // page, 0, :, s % page] = False
+            vt_mask[s // page, :, :, s % page] = False
+    same = (after == cache) | (torch.isnan(after.float()) & torch.isnan(cache.float()))
+    assert bool(same[untouched].all())
+    # the separate kernels on the same operands give the same rows (to rounding of the norm's sum)
+    cd2 = cache.to(DEV)
+    q2 = ops.qk_rope_store(qkv.to(DEV), hq, hkv, d, i32(positions) if rope else None, dev(qw), dev(kw), eps, dev(table),
+                           i32(slots), cd2, page)
+    out2 = ops.attention(q2, cd2, i32(positions), i32(list(range(B))), tab.to(DEV), scale, window=window,
+                         dec_tokens=i32([b for b in range(B) if slots[b] >= 0]), max_dec_position=max(positions))
+    rows = [b for b in range(B) if slots[b] >= 0]
+    close(out[rows], out2[rows].float().cpu(), bf)
+
+
 @pytest.mark.parametrize("key_pos", [0, 15, 16, 127, 128, 255, 256, 1000, 1023])
 def test_decode_kernel_one_far_key_decides(ops, key_pos):
     bf = torch.bfloat16
