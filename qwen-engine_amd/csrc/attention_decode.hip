@@ -306,15 +306,33 @@ __global__ __launch_bounds__(256) void attention_decode_merge_kernel(
     float o[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) o[i] = 0.f;
-    for (int s = wave; s < num_splits; s += 4) {
-        const float ms = pml[2 * s];
-        if (ms == -INFINITY) continue;          // an empty split: its accumulator was never written
-        const float wgt = __expf(ms - M);
-        denom += wgt * pml[2 * s + 1];
+    // eight of the wave's splits at a time: their maxima, sums and accumulator rows are all asked
+    // for before the first is used (one trip to memory for eight); added in ascending order
+    for (int s0 = wave; s0 < num_splits; s0 += 32) {
+        float ms[8], ls[8], a[8][PER];
 #pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int d = lane + i * 64;
-            if (d < D) o[i] += wgt * pacc[(long)s * D + d];
+        for (int k = 0; k < 8; ++k) {
+            const int s = s0 + 4 * k;
+            ms[k] = s < num_splits ? pml[2 * s] : -INFINITY;
+            ls[k] = s < num_splits ? pml[2 * s + 1] : 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int s = s0 + 4 * k;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                const int d = lane + i * 64;
+                // an empty split's accumulator was never written: not read
+                a[k][i] = (ms[k] != -INFINITY && d < D) ? pacc[(long)s * D + d] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            if (ms[k] == -INFINITY) continue;
+            const float wgt = __expf(ms[k] - M);
+            denom += wgt * ls[k];
+#pragma unroll
+            for (int i = 0; i < PER; ++i) o[i] += wgt * a[k][i];
         }
     }
 #pragma unroll

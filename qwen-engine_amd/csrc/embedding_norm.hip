@@ -83,12 +83,19 @@ __global__ void rmsnorm_regs_kernel(float* __restrict__ h, const TD* __restrict_
         if (c < H) {
             Vec4<float>::load(hr + c, v[i]);
             if (dr) {
-#pragma unroll 4
-                for (int s = 0; s < n_delta; ++s) {
-                    float d[4];
-                    Vec4<TD>::load(dr + s * delta_stride + c, d);
+                // the parts are asked for eight at a time, all before the first is added (one trip
+                // to memory for eight), and added in ascending order
+                for (int s0 = 0; s0 < n_delta; s0 += 8) {
+                    float d[8][4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[i][e] += d[e];
+                    for (int s = 0; s < 8; ++s)
+                        if (s0 + s < n_delta) Vec4<TD>::load(dr + (s0 + s) * delta_stride + c, d[s]);
+#pragma unroll
+                    for (int s = 0; s < 8; ++s)
+                        if (s0 + s < n_delta) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[i][e] += d[s][e];
+                        }
                 }
             }
 #pragma unroll
