@@ -1,16 +1,19 @@
 // Matrix product for many rows of activations (prefill): out[M, N] = x[M, K] . W[N, K]^T (+ bias),
 // bfloat16 in, 32-bit accumulation with v_mfma_f32_32x32x16_bf16, output bfloat16 or float32.
 //
-// A block of 256 threads (4 waves, 2 x 2) computes a BM x BN tile of the output; each wave a
-// quarter as (BM / 64) x (BN / 64) MFMA tiles.  K is walked in steps of BK through shared memory
-// with two buffers: while the MFMAs of one step run, the 16-byte global loads of the next are in
-// flight.  Both operands are K-contiguous in memory, so they are staged alike: a row of BK
+// A block of NW waves (NW / 2 down, 2 across) computes a BM x BN tile of the output; each wave its
+// part as MFMA tiles of 32 x 32.  K is walked in steps of BK through shared memory with two
+// buffers.  Both operands are K-contiguous in memory, so they are staged alike: a row of BK
 // bfloat16 is padded by 16 bytes, which makes the 16-byte fragment reads of the 32 rows of an
 // MFMA operand fall into distinct banks.
 //
-// The kernel is bound by shared-memory traffic rather than by the MFMA units unless a wave's
-// part is large (an operand fragment read once serves several MFMAs): 256 x 128 tiles are used
-// where they still give every compute unit a block, 128 x 128 and 64 x 128 for smaller products.
+// What the time of such a block goes to, as measured on this chip (cycle counters in a copy of
+// the kernel, hardware counters): not to the MFMA units alone.  A compute unit takes 64 bytes a
+// cycle from its L1, so a 128 x 128 x 64 step (32 KB) costs as many cycles to load as its MFMAs
+// take; loads have to be in flight two steps ahead to arrive in time; and the result has to be
+// stored as whole rows.  128 x 128 tiles (four waves, two blocks a compute unit) are the default,
+// 64 x 128 where there would be too few blocks otherwise, 256 x 128 (eight waves) where even
+// those give every compute unit two blocks.
 //
 // Rows of x beyond M and rows of W beyond N are read as zero and never stored; K must be a
 // multiple of 8 (16-byte loads), a tail shorter than BK is filled with zeros.
@@ -25,14 +28,14 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
 // SILU: W holds gate and up rows interleaved in blocks of 32 (gate 0..31, up 0..31, gate 32..63,
 // ...), N counts all of them, and the result is silu(gate) * up, N / 2 wide: the two MFMA tiles a
 // lane holds side by side are the gate and the up of the same outputs.
-template <typename TO, int BM, int BN, int BK, int MINB, bool SILU>
-__global__ __launch_bounds__(256, MINB) void gemm_mfma_kernel(
+template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU>
+__global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n) {
     constexpr int ROWB = BK * 2 + 16;       // bytes of a staged row
     constexpr int PPR = BK / 8;             // 16-byte pieces per row
-    constexpr int RPI = 256 / PPR;          // rows the block stages with one piece per thread
-    constexpr int WM = BM / 2, WN = BN / 2; // a wave's part
+    constexpr int RPI = 64 * NW / PPR;      // rows the block stages with one piece per thread
+    constexpr int WM = BM / (NW / 2), WN = BN / 2;   // a wave's part: NW / 2 waves down, 2 across
     constexpr int MI = WM / 32, NJ = WN / 32;
     constexpr int LDA = BM / RPI, LD = (BM + BN) / RPI;   // pieces a thread stages per step: LDA of x, then of W
     static_assert((LD == 12 || LD == 8 || LD == 6) && BM % RPI == 0 && BN % RPI == 0, "tile rows must be a multiple of the rows staged at once");
@@ -214,7 +217,7 @@ __global__ __launch_bounds__(256, MINB) void gemm_mfma_kernel(
     constexpr int CH = 16 / ESZ;                           // outputs in 16 bytes
     constexpr int CPR = WNO / CH;                          // 16-byte chunks in a row of the strip
     constexpr int SROW = WNO * ESZ + 16;                   // bytes of a staged row
-    static_assert(4 * 32 * SROW <= 2 * BUF, "the strips of the four waves must fit the staging buffers");
+    static_assert(NW * 32 * SROW <= 2 * BUF, "the strips of the waves must fit the staging buffers");
     unsigned char* strip = smem + wave * 32 * SROW;
     const int no0 = SILU ? (n0 + wn) / 2 : n0 + wn;        // first output column of the wave's strip
     const bool vec_ok = (NO % CH) == 0 && (((unsigned long)out) & 15) == 0;
@@ -270,7 +273,7 @@ bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w) {
     return dt_a == QE_BF16 && dt_w == QE_BF16 && M > 16 && K % 8 == 0 && K >= 64;
 }
 
-template <typename TO, int BM, int BN, int BK, int MINB, bool SILU>
+template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU>
 static int launch_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                        hipStream_t stream) {
     const int tiles_m = qe_cdiv(M, BM), tiles_n = qe_cdiv(N, BN);
@@ -279,11 +282,11 @@ static int launch_mfma(const void* x, const void* w, const float* bias, void* ou
     const size_t shmem = 2 * (BM + BN) * (BK * 2 + 16);
     static bool attr_set = false;   // one flag per instantiation
     if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)gemm_mfma_kernel<TO, BM, BN, BK, MINB, SILU>,
+        (void)hipFuncSetAttribute((const void*)gemm_mfma_kernel<TO, BM, BN, BK, NW, MINB, SILU>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         attr_set = true;
     }
-    gemm_mfma_kernel<TO, BM, BN, BK, MINB, SILU><<<(int)blocks, 256, shmem, stream>>>(
+    gemm_mfma_kernel<TO, BM, BN, BK, NW, MINB, SILU><<<(int)blocks, 64 * NW, shmem, stream>>>(
         (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n);
     QE_LAUNCH_CHECK();
     return 0;
@@ -296,9 +299,9 @@ static int pick_mfma(const void* x, const void* w, const float* bias, void* out,
     const long big = (long)qe_cdiv(M, 256) * qe_cdiv(N, 128), mid = (long)qe_cdiv(M, 128) * qe_cdiv(N, 128);
     // the largest tile that still gives every compute unit two blocks (one, for the middle size)
     if (tile == 0) tile = (big >= 2 * cus && M > 128) ? 256 : ((mid >= cus && M > 64) ? 128 : 64);   // never taller than the rows need
-    if (tile == 256) return launch_mfma<TO, 256, 128, 64, 1, SILU>(x, w, bias, out, M, N, K, stream);
-    if (tile == 128) return launch_mfma<TO, 128, 128, 64, 2, SILU>(x, w, bias, out, M, N, K, stream);
-    return launch_mfma<TO, 64, 128, 64, 2, SILU>(x, w, bias, out, M, N, K, stream);
+    if (tile == 256) return launch_mfma<TO, 256, 128, 64, 8, 1, SILU>(x, w, bias, out, M, N, K, stream);
+    if (tile == 128) return launch_mfma<TO, 128, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, stream);
+    return launch_mfma<TO, 64, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, stream);
 }
 
 // tile: rows of the output tile (256, 128 or 64), 0 to choose by the shape.  silu: w is [N, K] with
