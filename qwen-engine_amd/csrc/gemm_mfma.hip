@@ -17,8 +17,7 @@
 //
 // Rows of x beyond M and rows of W beyond N are read as zero and never stored; K must be a
 // multiple of 8 (16-byte loads), a tail shorter than BK is filled with zeros.
-// blockIdx.x walks the tiles so that consecutive blocks share the same rows of W (one
-// column of tiles after the other), which keeps an XCD's L2 on few weight rows at a time.
+// The blocks of one XCD (every eighth block) take a compact part of the tiles, see the kernel.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
