@@ -13,6 +13,16 @@ line is printed:
   prefill    one 2048-token prompt in one step: tokens a second, and flops / time / peak
   roofline   the decode step's bytes (every weight once + the live requests' cache) / time / 8 TB/s
   points     decoded tokens a second at batch 1 and at batch 64
+
+Other sizes and workloads (not what the default line reports):
+
+  --model 8b|32b            the layer sizes of Qwen3-8B / Qwen3-32B (BASELINE.json configs[3], [4]); with
+                            --layers L fewer layers than the model has (the line names both numbers)
+  --workload serving        N requests (--requests, default 64) with prompt lengths uniform in [128, 2048]
+                            and 256 new tokens each through the scheduler: continuous batching, prompt
+                            portions of 512 tokens beside decoded tokens.  value = generated tokens a second
+  --workload shared-prefix  N requests (default 32) that share a 1024-token prefix, each with 1024 tokens
+                            of its own and 512 new tokens; the prefix's pages are shared
 """
 import argparse
 import json
@@ -33,6 +43,15 @@ QWEN3_0_6B = dict(
     max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True)
 
 
+SIZES = {
+    "0.6b": QWEN3_0_6B,
+    "8b": dict(QWEN3_0_6B, hidden_size=4096, intermediate_size=12288, num_hidden_layers=36,
+               num_attention_heads=32, num_key_value_heads=8, tie_word_embeddings=False),
+    "32b": dict(QWEN3_0_6B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64,
+                num_attention_heads=64, num_key_value_heads=8, tie_word_embeddings=False),
+}
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -46,7 +65,74 @@ def parse():
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--model", default="0.6b", choices=sorted(SIZES), help="whose layer sizes")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "shared-prefix"])
+    ap.add_argument("--requests", type=int, default=None, help="requests of the serving workloads")
     return ap.parse_args()
+
+
+def serving_run(args, cfg, model, layers, full_layers) -> int:
+    """The scheduler's workloads: every request through LLMEngine.submit / step until all have finished."""
+    import torch
+    from qwen_engine_amd import EngineConfig
+    from qwen_engine_amd.engine.llm_engine import LLMEngine
+
+    g = torch.Generator().manual_seed(args.seed + 2)
+    V = cfg.vocab_size
+    if args.workload == "serving":
+        n = args.requests or 64
+        lens = torch.randint(128, 2049, (n,), generator=g).tolist()
+        prompts = [torch.randint(0, V, (k,), generator=g).tolist() for k in lens]
+        new_tokens, sharing = 256, False
+        what = f"{n} requests, prompts uniform in [128, 2048], {new_tokens} new tokens each, portions of 512"
+    else:
+        n = args.requests or 32
+        prefix = torch.randint(0, V, (1024,), generator=g).tolist()
+        prompts = [prefix + torch.randint(0, V, (1024,), generator=g).tolist() for _ in range(n)]
+        new_tokens, sharing = 512, True
+        what = f"{n} requests sharing a 1024-token prefix, 1024 tokens of their own, {new_tokens} new tokens each"
+    longest = max(len(p) for p in prompts) + new_tokens
+    P = args.block_size
+    pages = n * ((longest + P - 1) // P + 1)
+    ecfg = EngineConfig(dtype="bfloat16" if args.dtype == "bf16" else "float32", block_size=P, num_blocks=pages,
+                        max_num_seqs=n, max_model_len=longest, max_step_tokens=2048, prefill_chunk=512,
+                        enable_prefix_sharing=sharing, seed=args.seed)
+    engine = LLMEngine(model, None, ecfg)
+    engine.submit(prompts, max_new_tokens=new_tokens, ignore_eos=True)
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    steps = 0
+    last = t
+    while engine.scheduler.has_work():
+        engine.step()
+        steps += 1
+        if time.perf_counter() - last > 30:
+            last = time.perf_counter()
+            print(f"[bench] {steps} steps, {engine.stats()}", file=sys.stderr, flush=True)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t
+    stats = engine.stats()
+    results = engine.run()
+    assert all(len(r.token_ids) == new_tokens for r in results), "a request did not run to its length"
+    generated = n * new_tokens
+    prompt_tokens = sum(len(p) for p in prompts)
+    line = {
+        "metric": f"generated tok/s, {args.workload} workload (Qwen3-{args.model.upper()} sizes)",
+        "value": round(generated / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 0,
+        "ms_per_step": round(dt / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform-random token ids",
+        "config": {"model": f"Qwen3-{args.model.upper()} sizes (random weights)", "layers": layers,
+                   "layers_of_model": full_layers, "hidden_size": cfg.hidden_size,
+                   "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
+                   "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": V,
+                   "workload": what, "requests": n, "page_size": P, "prefix_sharing": sharing,
+                   "parallelism": "single GPU"},
+        "seconds": round(dt, 3), "prompt_tokens": prompt_tokens, "generated_tokens": generated,
+        "all_tokens_per_s": round((prompt_tokens + generated) / dt, 1),
+        "scheduler": {k: v for k, v in stats.items() if isinstance(v, (int, float))},
+    }
+    print(json.dumps(line), flush=True)
+    return 0
 
 
 def main() -> int:
@@ -62,9 +148,10 @@ def main() -> int:
     from qwen_engine_amd.parts import DecoderModel, Runtime
     from qwen_engine_amd.weights import random_tensors
 
-    full_layers = QWEN3_0_6B["num_hidden_layers"]
+    sizes = SIZES[args.model]
+    full_layers = sizes["num_hidden_layers"]
     layers = args.layers or full_layers
-    cfg = Qwen3Config.from_dict(dict(QWEN3_0_6B, num_hidden_layers=layers))
+    cfg = Qwen3Config.from_dict(dict(sizes, num_hidden_layers=layers))
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -74,6 +161,9 @@ def main() -> int:
     model = DecoderModel(cfg.to_model_spec())
     model.load(random_tensors(cfg, args.seed, dtype=torch.bfloat16), Runtime(dev, dtype))
     print(f"[bench] random weights for {layers} layers in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+
+    if args.workload != "decode":
+        return serving_run(args, cfg, model, layers, full_layers)
 
     P = args.block_size
     itemsize = 2 if args.dtype == "bf16" else 4
@@ -155,7 +245,7 @@ def main() -> int:
             print(f"[bench] decode batch {b}: {r}", file=sys.stderr, flush=True)
 
     line = {
-        "metric": "decode tok/s @ batch 8 (Qwen3-0.6B sizes, context 4096)",
+        "metric": f"decode tok/s @ batch {args.batch} (Qwen3-{args.model.upper()} sizes, context {args.context})",
         "value": round(main_run["tok_s"], 1),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -168,9 +258,9 @@ def main() -> int:
         "dtype": args.dtype,
         "data": "synthetic: random weights N(0, 0.02), uniform-random token ids",
         "config": {
-            "model": "Qwen3-0.6B sizes (random weights)", "layers": layers, "layers_of_model": full_layers,
+            "model": f"Qwen3-{args.model.upper()} sizes (random weights)", "layers": layers, "layers_of_model": full_layers,
             "hidden_size": H, "num_attention_heads": Hq, "num_key_value_heads": Hkv, "head_dim": D,
-            "intermediate_size": I, "vocab_size": V, "tie_word_embeddings": True,
+            "intermediate_size": I, "vocab_size": V, "tie_word_embeddings": cfg.tie_word_embeddings,
             "global_batch": args.batch, "seq_len": args.context, "page_size": P,
             "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU",
         },
