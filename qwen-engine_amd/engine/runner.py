@@ -201,6 +201,60 @@ class ModelRunner:
         return (seqs, cat(tokens), cat(positions), cat(tok_seq), cat(rows), [cat(x) for x in slots],
                 [np.asarray(u, dtype=np.int32) for u in upd_idx], [np.asarray(u, dtype=np.int32) for u in upd_val])
 
+    def _single_token_layout(self, entries: Sequence[StepEntry]):
+        """What _check_and_reserve and _layout do, for entries of one token each, with plain
+        integers: a decode step's host time is per request, and an array per request costs
+        more than the request's whole bookkeeping."""
+        cache = self.cache
+        vocab, max_pos, P = self.model.spec.vocab_size, self.model.spec.max_positions, self.page_size
+        n_groups = len(cache.groups)
+        seen = set()
+        rcs, wants = [], []
+        for e in entries:
+            if e.req_id in seen:
+                raise ValueError(f"request {e.req_id!r} appears twice in one step")
+            seen.add(e.req_id)
+            t = e.tokens[0]
+            if not isinstance(t, (int, np.integer)) or not 0 <= t < vocab:
+                raise ValueError(f"token id {t} of request {e.req_id!r} is outside the vocabulary of {vocab}")
+            rc = cache.get(e.req_id)
+            if rc.num_tokens + 1 > max_pos:
+                raise ValueError(f"request {e.req_id!r} would pass the model's {max_pos} positions")
+            rcs.append(rc)
+            if any(len(table) * P <= rc.num_tokens for table in rc.tables):   # its next position has no page yet
+                wants.append((e.req_id, rc.num_tokens + 1))
+        if wants:
+            if not cache.can_reserve(wants):
+                raise OutOfPages("the cache has too few free pages for this step")
+            for req_id, new_len in wants:
+                cache.reserve(req_id, new_len)
+        B = len(entries)
+        seqs = []
+        tok, pos, seq = [0] * B, [0] * B, [0] * B
+        slots = [[0] * B for _ in range(n_groups)]
+        upd_idx: List[List[int]] = [[] for _ in range(n_groups)]
+        upd_val: List[List[int]] = [[] for _ in range(n_groups)]
+        for i, (e, rc) in enumerate(zip(entries, rcs)):
+            n = rc.num_tokens
+            seqs.append(SeqInfo(e.req_id, i, 1, n, rc.state_slot, rc.new_request))
+            tok[i], pos[i], seq[i] = int(e.tokens[0]), n, rc.state_slot
+            for g in range(n_groups):
+                page = rc.tables[g][n // P]
+                if page < 0:
+                    raise RuntimeError(f"request {e.req_id!r} holds no page for position {n} in group {g}")
+                slots[g][i] = page * P + n % P
+                if rc.dirty[g]:
+                    width = self.table_width[g]
+                    for j, pg in cache.take_dirty(e.req_id, g):
+                        if j >= width:
+                            raise RuntimeError("a request holds more pages than its table row has entries")
+                        upd_idx[g].append(rc.state_slot * width + j)
+                        upd_val[g].append(pg)
+        i32 = np.int32
+        return (seqs, np.asarray(tok, dtype=i32), np.asarray(pos, dtype=i32), np.asarray(seq, dtype=i32),
+                np.arange(B, dtype=i32), [np.asarray(x, dtype=i32) for x in slots],
+                [np.asarray(u, dtype=i32) for u in upd_idx], [np.asarray(u, dtype=i32) for u in upd_val])
+
     def _to_device(self, parts: List[np.ndarray]) -> List[torch.Tensor]:
         """One copy of all the arrays to the device, through a pinned buffer that is kept and grown;
         returns a device view for each part."""
@@ -267,8 +321,7 @@ class ModelRunner:
 
     # ---- decoding through a recorded graph ------------------------------------------------
     def _decode_step_with_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        tokens = self._check_and_reserve(entries)
-        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(entries, tokens)
+        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._single_token_layout(entries)
         B, n_groups = len(seqs), len(self.cache.groups)
         i32 = np.int32
         cap = 2 * B                                    # table updates a decode step can bring per group
