@@ -13,6 +13,7 @@ line is printed:
   prefill    one 2048-token prompt in one step: tokens a second, and flops / time / peak
   roofline   the decode step's bytes (every weight once + the live requests' cache) / time / 8 TB/s
   points     decoded tokens a second at batch 1 and at batch 64
+  measured_copy_gbs   what a plain copy of 1 GiB reaches on this device (read + write), for scale
 
 Other sizes and workloads (not what the default line reports):
 
@@ -233,6 +234,22 @@ def main() -> int:
         torch.cuda.empty_cache()
         return dict(value=T / best, tokens=T, ms=best * 1e3, frac=flops / best / PEAK_FLOPS[args.dtype])
 
+    def copy_gbs():
+        """What a plain device-to-device copy of 1 GiB reaches (read + write), for scale beside the 8 TB/s."""
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t) / 10
+        del src, dst
+        torch.cuda.empty_cache()
+        return 2 * (1 << 30) / dt / 1e9
+
     main_run = decode_run(args.batch, args.context, args.steps, args.warmup)
     print(f"[bench] decode batch {args.batch}: {main_run}", file=sys.stderr, flush=True)
     prefill = prefill_run(args.prefill_tokens)
@@ -269,6 +286,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(main_run["gbs"], 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(main_run["gbs"] / HBM_PEAK_GBS, 4)},
         "points": points,
+        "measured_copy_gbs": round(copy_gbs(), 1),
     }
     print(json.dumps(line), flush=True)
     return 0
