@@ -85,6 +85,10 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
 }
 
 // ---- the same with the step before it folded in ---------------------------------------------
+// (Folding the output projection into the merge kernel, a block per head and 128 output features
+// that merges the head's splits for all tokens and multiplies with its part of W_o, was tried for
+// few tokens: it takes as long as the two kernels it replaces.)
+//
 // The q/k norm, the rotation and the cache write of the new token cost a kernel of their own
 // that runs a few microseconds for a few kilobytes.  Here every wave norms and rotates the query
 // heads it needs itself, straight from the q|k|v rows (the pairs d, d + D/2 of the rotation lie in
