@@ -9,7 +9,7 @@ int qe_gemm_skinny(const void* x, const void* w, const float* bias, void* out, i
 int qe_gemm_skinny_splits(int N, int K);
 bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w);
 int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
-                 int tile, bool silu, hipStream_t stream);
+                 int tile, bool silu, int splits, hipStream_t stream);
 
 enum { ALGO_AUTO = 0, ALGO_GENERIC = 1, ALGO_MFMA = 2, ALGO_TILE = 1000 };   // ALGO_TILE + rows: the tiled kernel with that tile
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3, EPI_SILU_MUL_IL = 4 };
@@ -24,8 +24,26 @@ extern "C" int qe_gemm_silu_supported(int M, int N, int K, int dt_a, int dt_w) {
     return (N % 32 == 0 && (qe_gemm_skinny_ok(M, N, K, dt_a, dt_w) || qe_gemm_mfma_ok(M, 2 * N, K, dt_a, dt_w))) ? 1 : 0;
 }
 
+// More than 16 rows against a large matrix: the kernel for few rows, in which every wave reads the
+// activations of its chunks itself, reads several times more activations than weights there and
+// falls well behind the memory; the tiled kernel shares them through shared memory and streams
+// the weights at the memory's rate.  (Against a small matrix the tiled kernel has too few tiles.)
+static bool tiled_for_few_rows(int M, int N, int K, int dt_a, int dt_w) {
+    return M > 16 && (long)N * K >= (16L << 20) && qe_gemm_mfma_ok(M, N, K, dt_a, dt_w);
+}
+
 // number of partial products that epilogue 3 should be asked for
-extern "C" int qe_gemm_partial_splits(int N, int K) { return qe_gemm_skinny_splits(N, K); }
+extern "C" int qe_gemm_partial_splits(int M, int N, int K) {
+    if (tiled_for_few_rows(M, N, K, QE_BF16, QE_BF16)) {
+        const int tiles = qe_cdiv(N, 128);                 // (tiles of 64 rows: M <= 64 here)
+        int s = qe_cdiv(256, tiles);
+        const int most = K / 256;
+        if (s > most) s = most;
+        if (s > 16) s = 16;
+        return s < 1 ? 1 : s;
+    }
+    return qe_gemm_skinny_splits(N, K);
+}
 
 // out[M, N] = x[M, K] . w[N, K]^T (+ bias).  epilogue 0: store in dt_o.  1: add into out, the
 // 32-bit stream.  2: w is [2 N, K], gate rows then up rows; out = silu(x.gate^T) * (x.up^T).
@@ -41,10 +59,14 @@ extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* ou
     if (M == 0) return 0;
     const bool skinny = qe_gemm_skinny_ok(M, N, K, dt_a, dt_w);
     const bool tiled = qe_gemm_mfma_ok(M, N, K, dt_a, dt_w);
-    if (epilogue == EPI_SILU_MUL_IL && !skinny) {
+    if (epilogue == EPI_SILU_MUL_IL && (!skinny || tiled_for_few_rows(M, 2 * N, K, dt_a, dt_w))) {
         QE_REQUIRE(N % 32 == 0 && qe_gemm_mfma_ok(M, 2 * N, K, dt_a, dt_w),
                    "gemm: M=%d N=%d K=%d is not taken by a silu-mul kernel", M, N, K);
-        return qe_gemm_mfma(x, w, bias, out, M, 2 * N, K, dt_o, algo > ALGO_TILE ? algo - ALGO_TILE : 0, true, stream);
+        return qe_gemm_mfma(x, w, bias, out, M, 2 * N, K, dt_o, algo > ALGO_TILE ? algo - ALGO_TILE : 0, true, 1, stream);
+    }
+    if (epilogue == EPI_PARTIAL && tiled_for_few_rows(M, N, K, dt_a, dt_w)) {
+        QE_REQUIRE(dt_o == QE_F32, "gemm: partial products are 32-bit");
+        return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, 0, false, splits, stream);
     }
     if (epilogue != EPI_STORE) {
         QE_REQUIRE(skinny, "gemm: M=%d N=%d K=%d with these element types is not taken by the kernel for few rows", M, N, K);
@@ -53,15 +75,12 @@ extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* ou
     QE_REQUIRE(algo == ALGO_AUTO || algo == ALGO_GENERIC || algo == ALGO_MFMA || algo > ALGO_TILE, "gemm: unknown algo %d", algo);
     if (algo > ALGO_TILE) {
         QE_REQUIRE(tiled, "gemm: M=%d N=%d K=%d is not taken by the tiled MFMA kernel", M, N, K);
-        return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, algo - ALGO_TILE, false, stream);
+        return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, algo - ALGO_TILE, false, 1, stream);
     }
     if (algo != ALGO_GENERIC) {
-        // more than 16 rows against a very wide matrix (the logits of a large batch): the kernel for
-        // few rows passes over the weights once per 16 rows' worth of arithmetic and falls behind
-        // the memory there; the tiled kernel streams them once
-        if (skinny && !(tiled && M > 16 && N >= 32768))
+        if (skinny && !tiled_for_few_rows(M, N, K, dt_a, dt_w))
             return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, EPI_STORE, 1, stream);
-        if (tiled) return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, 0, false, stream);
+        if (tiled) return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, 0, false, 1, stream);
         QE_REQUIRE(algo == ALGO_AUTO, "gemm: M=%d N=%d K=%d with these element types is not taken by an MFMA kernel", M, N, K);
     }
     return qe_gemm_generic(x, w, bias, out, M, N, K, dt_a, dt_w, dt_o, stream);

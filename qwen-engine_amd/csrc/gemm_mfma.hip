@@ -30,7 +30,7 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
 template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU>
 __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n) {
+    TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n, int k_per_split) {
     constexpr int ROWB = BK * 2 + 16;       // bytes of a staged row
     constexpr int PPR = BK / 8;             // 16-byte pieces per row
     constexpr int RPI = 64 * NW / PPR;      // rows the block stages with one piece per thread
@@ -61,7 +61,11 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
 
-    const int nk = (K + BK - 1) / BK;
+    // blockIdx.y cuts K: this block sums the k values [k0, k0 + klen) and writes the partial product
+    // number blockIdx.y (out is then [splits][M][N]); without a cut k_per_split = K
+    const int k0 = blockIdx.y * k_per_split;
+    const int klen = K - k0 < k_per_split ? K - k0 : k_per_split;
+    const int nk = (klen + BK - 1) / BK;
     // Two sets of staging registers in turn: a step's loads are issued two steps ahead and go to
     // shared memory one step ahead, so a load has a whole step of MFMAs to arrive.
     uint4_t stage[2][LD];
@@ -79,12 +83,12 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     // statement as operands, so nothing that uses them can move ahead of it.
     const int lrow = tid / PPR, pc = tid % PPR;
     const int a_rows = M - m0 < BM ? M - m0 : BM, b_rows = N - n0 < BN ? N - n0 : BN;
-    const unsigned long a_addr = (unsigned long)(x + (long)m0 * K), b_addr = (unsigned long)(w + (long)n0 * K);
+    const unsigned long a_addr = (unsigned long)(x + (long)m0 * K + k0), b_addr = (unsigned long)(w + (long)n0 * K + k0);
     uint4_t rsrc_a, rsrc_b;   // base, base high 16 bits (stride 0), bytes, format: 32-bit raw buffer
     rsrc_a[0] = (unsigned)a_addr; rsrc_a[1] = (unsigned)(a_addr >> 32) & 0xffffu;
-    rsrc_a[2] = (unsigned)(a_rows * K * 2); rsrc_a[3] = 0x00020000u;
+    rsrc_a[2] = (unsigned)(((a_rows - 1) * K + klen) * 2); rsrc_a[3] = 0x00020000u;   // up to the last row's last k of this cut
     rsrc_b[0] = (unsigned)b_addr; rsrc_b[1] = (unsigned)(b_addr >> 32) & 0xffffu;
-    rsrc_b[2] = (unsigned)(b_rows * K * 2); rsrc_b[3] = 0x00020000u;
+    rsrc_b[2] = (unsigned)(((b_rows - 1) * K + klen) * 2); rsrc_b[3] = 0x00020000u;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {   // the same in every lane: into scalar registers
         rsrc_a[c] = __builtin_amdgcn_readfirstlane(rsrc_a[c]);
@@ -97,7 +101,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const int dst = lrow * ROWB + pc * 16;                 // where piece 0 goes in a buffer; piece i: + i RPI ROWB
 #define LOAD_GLOBAL(set_, kt_)                                                           \
     {                                                                                    \
-        const bool k_ok = (kt_) * BK + pc * 8 < K;                                       \
+        const bool k_ok = (kt_) * BK + pc * 8 < klen;                                    \
         const int soff = (kt_) * BK * 2;                                                 \
         _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                 \
             const int vo = k_ok ? voff[i] : 0x7fffffff;                                  \
@@ -238,7 +242,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
                         v[r] = acc[i][j][4 * bq + r];
                     }
                 }
-                if (!SILU && bias) {                       // (a column beyond the output is never stored: any bias does)
+                if (!SILU && bias && blockIdx.y == 0) {                       // (a column beyond the output is never stored: any bias does)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) v[r] += bias[no0 + nl + r < NO ? no0 + nl + r : NO - 1];
                 }
@@ -253,7 +257,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
             const int m = m0 + wm + i * 32 + row, n = no0 + col;
             if (m >= M || n >= NO) continue;
             const uint4_t piece = *(const uint4_t*)(strip + row * SROW + col * ESZ);
-            TO* o = out + (long)m * NO + n;
+            TO* o = out + ((long)blockIdx.y * M + m) * NO + n;
             if (vec_ok) {
                 *(uint4_t*)o = piece;                      // n + CH <= NO: both are multiples of CH
             } else {
@@ -274,7 +278,7 @@ bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w) {
 
 template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU>
 static int launch_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                       hipStream_t stream) {
+                       int splits, hipStream_t stream) {
     const int tiles_m = qe_cdiv(M, BM), tiles_n = qe_cdiv(N, BN);
     const long blocks = (long)tiles_m * tiles_n;
     QE_REQUIRE(blocks <= 2147483647L, "mfma gemm: too many tiles");
@@ -285,35 +289,41 @@ static int launch_mfma(const void* x, const void* w, const float* bias, void* ou
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         attr_set = true;
     }
-    gemm_mfma_kernel<TO, BM, BN, BK, NW, MINB, SILU><<<(int)blocks, 64 * NW, shmem, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n);
+    // a cut of K is a multiple of BK long (the last may be shorter)
+    const int k_per_split = splits > 1 ? qe_cdiv(qe_cdiv(K, splits), BK) * BK : K;
+    QE_REQUIRE(splits >= 1 && splits <= 65535 && (long)(splits - 1) * k_per_split < K,
+               "mfma gemm: K=%d cannot be cut into %d parts", K, splits);
+    gemm_mfma_kernel<TO, BM, BN, BK, NW, MINB, SILU><<<dim3((unsigned)blocks, (unsigned)splits), 64 * NW, shmem, stream>>>(
+        (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n, k_per_split);
     QE_LAUNCH_CHECK();
     return 0;
 }
 
 template <typename TO, bool SILU>
 static int pick_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                     int tile, hipStream_t stream) {
+                     int tile, int splits, hipStream_t stream) {
     const long cus = 256;
-    const long big = (long)qe_cdiv(M, 256) * qe_cdiv(N, 128), mid = (long)qe_cdiv(M, 128) * qe_cdiv(N, 128);
+    const long big = (long)qe_cdiv(M, 256) * qe_cdiv(N, 128) * splits, mid = (long)qe_cdiv(M, 128) * qe_cdiv(N, 128) * splits;
     // the largest tile that still gives every compute unit two blocks (one, for the middle size)
     if (tile == 0) tile = (big >= 2 * cus && M > 128) ? 256 : ((mid >= cus && M > 64) ? 128 : 64);   // never taller than the rows need
-    if (tile == 256) return launch_mfma<TO, 256, 128, 64, 8, 1, SILU>(x, w, bias, out, M, N, K, stream);
-    if (tile == 128) return launch_mfma<TO, 128, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, stream);
-    return launch_mfma<TO, 64, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, stream);
+    if (tile == 256) return launch_mfma<TO, 256, 128, 64, 8, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
+    if (tile == 128) return launch_mfma<TO, 128, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, splits, stream);
+    return launch_mfma<TO, 64, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, splits, stream);
 }
 
 // tile: rows of the output tile (256, 128 or 64), 0 to choose by the shape.  silu: w is [N, K] with
 // gate and up rows interleaved in blocks of 32, out is [M, N / 2] = silu(gate) * up.
+// splits > 1: out is float [splits, M, N], partial products along K (no silu then).
 int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
-                 int tile, bool silu, hipStream_t stream) {
+                 int tile, bool silu, int splits, hipStream_t stream) {
+    QE_REQUIRE(splits >= 1 && (splits == 1 || (!silu && dt_o == QE_F32)), "mfma gemm: partial products are 32-bit and plain");
     QE_REQUIRE(K % 8 == 0 && K >= 64 && K < (1 << 22), "mfma gemm: K=%d is no multiple of 8 in [64, 2^22)", K);
     QE_REQUIRE(tile == 0 || tile == 256 || tile == 128 || tile == 64, "mfma gemm: tile of %d rows", tile);
     if (silu) {
         QE_REQUIRE(!bias && N % 64 == 0, "mfma gemm: silu-mul takes no bias and gate|up rows in blocks of 32");
-        if (dt_o == QE_BF16) return pick_mfma<bf16_t, true>(x, w, bias, out, M, N, K, tile, stream);
-        return pick_mfma<float, true>(x, w, bias, out, M, N, K, tile, stream);
+        if (dt_o == QE_BF16) return pick_mfma<bf16_t, true>(x, w, bias, out, M, N, K, tile, splits, stream);
+        return pick_mfma<float, true>(x, w, bias, out, M, N, K, tile, splits, stream);
     }
-    if (dt_o == QE_BF16) return pick_mfma<bf16_t, false>(x, w, bias, out, M, N, K, tile, stream);
-    return pick_mfma<float, false>(x, w, bias, out, M, N, K, tile, stream);
+    if (dt_o == QE_BF16) return pick_mfma<bf16_t, false>(x, w, bias, out, M, N, K, tile, splits, stream);
+    return pick_mfma<float, false>(x, w, bias, out, M, N, K, tile, splits, stream);
 }

@@ -49,7 +49,7 @@ def load_library():
         "qe_silu_mul": [vp, vp, i32, i32, i32, i32, vp],
         "qe_gemm_silu_supported": [i32, i32, i32, i32, i32],
         "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
-        "qe_gemm_partial_splits": [i32, i32],
+        "qe_gemm_partial_splits": [i32, i32, i32],
         "qe_gemm_fused_supported": [i32, i32, i32, i32, i32],
         "qe_attention_decode_supported": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_supported": [i32, i32, i32, i32, i32],
@@ -252,7 +252,7 @@ def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
     out_dtype = out_dtype or x.dtype
     shape = (M, N)
     if epilogue == EPI_PARTIAL:
-        splits = splits or lib.qe_gemm_partial_splits(N, K)
+        splits = splits or lib.qe_gemm_partial_splits(M, N, K)
         out_dtype, shape = torch.float32, (splits, M, N)
     else:
         splits = 1

@@ -576,6 +576,42 @@ def test_gemm_tiled_mfma(ops, M, N, K):
         ops.gemm(torch.zeros(100, 76, dtype=bf, device=DEV), torch.zeros(8, 76, dtype=bf, device=DEV), algo=ops.ALGO_FAST)
 
 
+@pytest.mark.parametrize("M", [17, 40, 64])
+def test_gemm_of_few_rows_against_a_large_matrix(ops, M):
+    """17 to 64 rows against a matrix of 16 M elements or more go through the tiled kernel (the one
+    for few rows reads mostly activations there): plain, cut along K into partial products, and
+    with silu.mul over interleaved gate|up rows."""
+    bf = torch.bfloat16
+    N, K = 4224, 4096
+    x, w = rand(M, K, seed=180, dtype=bf), rand(N, K, seed=181, dtype=bf, scale=0.05)
+    bias = rand(N, seed=182)
+    want = P.linear(x.double(), w.double())
+    xd, wd = x.to(DEV), w.to(DEV)
+    close(ops.gemm(xd, wd), want, bf)
+    close(ops.gemm(xd, wd, bias.to(DEV), out_dtype=torch.float32), want + bias.double(), torch.float32,
+          scale=float(want.abs().max()))
+    for splits in (0, 1, 5, 16):
+        parts = ops.gemm(xd, wd, epilogue=ops.EPI_PARTIAL, splits=splits)
+        assert parts.dtype == torch.float32 and parts.dim() == 3 and (splits == 0 or parts.shape[0] == splits)
+        close(parts.sum(0), want, torch.float32, scale=float(want.abs().max()))
+    # the norm adds the parts up, as after the attention and the feed-forward
+    h = rand(M, N, seed=183)
+    hd = h.to(DEV)
+    nw = 1 + rand(N, seed=184, scale=0.1)
+    parts = ops.gemm(xd, wd, epilogue=ops.EPI_PARTIAL)
+    normed = ops.rmsnorm(hd, nw.to(DEV), 1e-6, bf, delta=parts)
+    total = h.double() + parts.double().cpu().sum(0)
+    close(hd, total, torch.float32)
+    close(normed, P.rms_norm(total.float(), nw, 1e-6), bf)
+    # gate|up: 2 * 2112 rows of 4096
+    I = N // 2
+    g, u = w[:I], w[I:]
+    wil = ops.interleave_gate_up(g.to(DEV), u.to(DEV))
+    assert ops.gemm_silu_supported(xd, wil)
+    got = ops.gemm(xd, wil, epilogue=ops.EPI_SILU_MUL_IL)
+    close(got, P.silu_mul(P.linear(x.double(), g.double()), P.linear(x.double(), u.double())), bf)
+
+
 @pytest.mark.parametrize("hq,hkv,d,page", [(16, 8, 128, 16), (4, 4, 64, 16), (8, 1, 128, 32), (6, 2, 64, 64), (8, 2, 128, 48)])
 @pytest.mark.parametrize("window", [0, 40, 17])
 def test_prefill_attention_kernel(ops, hq, hkv, d, page, window):
