@@ -15,10 +15,16 @@ when a request ends (the reference waits for the whole queue, llm_engine.py:147-
 a page is registered for sharing only once all its tokens are computed, and the map
 from page to hash is kept, so that a freed page leaves the registry
 (kvcache.py:163-165 pops a map that nothing fills); a reservation is all or nothing.
+
+With ``keep_freed_prefixes`` the registered pages of a request that ends are not freed at once:
+they stay registered, held by nobody, until a later request with the same beginning takes them
+over or a reservation needs their memory (then the one kept longest goes first, and of one
+request's pages the last before the first, so that no kept page outlives the pages before it).
 """
 from __future__ import annotations
 
 import hashlib
+from collections import OrderedDict
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
@@ -69,16 +75,32 @@ class PagePool:
             raise CacheError(f"cannot retain page {page}: it is free")
         self.refcount[page] += 1
 
-    def release(self, page: int) -> bool:
-        """Drop one reference; True if the page became free."""
+    def release(self, page: int, to_free_list: bool = True) -> bool:
+        """Drop one reference; True if nobody holds the page any more (it then goes to the free
+        list, unless the caller keeps it aside)."""
         self._check_id(page)
         if self.refcount[page] <= 0:
             raise CacheError(f"cannot release page {page}: it is free already")
         self.refcount[page] -= 1
         if self.refcount[page] == 0:
-            self.free.append(page)
+            if to_free_list:
+                self.free.append(page)
             return True
         return False
+
+    def revive(self, page: int) -> None:
+        """A page that was kept aside with no holder gets its first holder again."""
+        self._check_id(page)
+        if self.refcount[page] != 0:
+            raise CacheError(f"page {page} is held: it cannot be revived")
+        self.refcount[page] = 1
+
+    def give_back(self, page: int) -> None:
+        """A page that was kept aside with no holder goes to the free list."""
+        self._check_id(page)
+        if self.refcount[page] != 0:
+            raise CacheError(f"page {page} is held: it cannot be given back")
+        self.free.append(page)
 
     def _check_id(self, page: int) -> None:
         if not 0 <= page < self.num_pages:
@@ -146,7 +168,7 @@ class _SharedEntry:
 
 class CacheManager:
     def __init__(self, groups: Sequence[GroupSpec], num_pages, page_size: int, max_requests: int,
-                 prefix_sharing: bool = False):
+                 prefix_sharing: bool = False, keep_freed_prefixes: bool = False):
         if page_size <= 0:
             raise CacheError("page_size must be positive")
         self.groups = list(groups)
@@ -166,7 +188,11 @@ class CacheManager:
             all(g.window is None for g in self.groups)
         self._shared: Dict[int, _SharedEntry] = {}
         self._page_hash: Dict[int, int] = {}   # page id of group 0 -> hash it is registered under
-        self.stats = {"pages_allocated": 0, "pages_freed": 0, "shared_page_hits": 0}
+        self.keep_freed = bool(keep_freed_prefixes) and self.prefix_sharing
+        # registered entries that nobody holds, by hash; the first is the next to go
+        self._kept: "OrderedDict[int, _SharedEntry]" = OrderedDict()
+        self.stats = {"pages_allocated": 0, "pages_freed": 0, "shared_page_hits": 0, "kept_page_hits": 0,
+                      "kept_pages_evicted": 0}
 
     # ---- requests -------------------------------------------------------------
     def add_request(self, req_id: Hashable) -> RequestCache:
@@ -186,6 +212,24 @@ class CacheManager:
 
     def free_request(self, req_id: Hashable) -> None:
         rc = self.get(req_id)
+        kept: List[int] = []
+        if self.keep_freed:
+            # registered pages go index by index, the pages of all groups together: an entry that
+            # nobody holds any more is kept instead of freed
+            for i, page0 in enumerate(rc.tables[0]):
+                h = self._page_hash.get(page0) if page0 >= 0 else None
+                entry = self._shared.get(h) if h is not None else None
+                if entry is None or any(i >= len(t) or t[i] != entry.pages[g] for g, t in enumerate(rc.tables)):
+                    continue
+                unheld = [self.pools[g].release(p, to_free_list=False) for g, p in enumerate(entry.pages)]
+                if all(unheld):
+                    kept.append(h)
+                elif any(unheld):
+                    raise CacheError("the pages of a shared entry have different counts")
+                for t in rc.tables:
+                    t[i] = -1
+            for h in reversed(kept):               # the request's last page first: it is the first to go
+                self._kept[h] = self._shared[h]
         for g, table in enumerate(rc.tables):
             for page in table:
                 if page >= 0:
@@ -222,7 +266,27 @@ class CacheManager:
         for req_id, new_len in wants:
             for g, n in enumerate(self.pages_needed(req_id, new_len)):
                 total[g] += n
-        return all(total[g] <= self.pools[g].num_free for g in range(len(self.groups)))
+        return all(total[g] <= self.available(g) for g in range(len(self.groups)))
+
+    def available(self, group: int = 0) -> int:
+        """Pages a reservation can get: the free ones and the kept ones (a kept entry has a page in every group)."""
+        return self.pools[group].num_free + len(self._kept)
+
+    @property
+    def num_kept(self) -> int:
+        """Registered entries that nobody holds (each has a page in every group)."""
+        return len(self._kept)
+
+    def _allocate(self, g: int) -> int:
+        while not self.pools[g].free and self._kept:
+            h, entry = self._kept.popitem(last=False)
+            del self._shared[h]
+            del self._page_hash[entry.pages[0]]
+            for gg, page in enumerate(entry.pages):
+                self.pools[gg].give_back(page)
+                self.stats["pages_freed"] += 1
+            self.stats["kept_pages_evicted"] += 1
+        return self.pools[g].allocate()
 
     def reserve(self, req_id: Hashable, new_len: int) -> None:
         """Give the request pages for every position it will hold up to new_len - 1.
@@ -232,9 +296,9 @@ class CacheManager:
             raise CacheError("a request's length cannot shrink")
         need = self.pages_needed(req_id, new_len)
         for g, n in enumerate(need):
-            if n > self.pools[g].num_free:
+            if n > self.available(g):
                 raise OutOfPages(f"group {g} needs {n} pages for request {req_id!r}, "
-                                 f"{self.pools[g].num_free} are free")
+                                 f"{self.available(g)} are free")
         hi = (new_len + self.page_size - 1) // self.page_size
         for g, table in enumerate(rc.tables):
             lo = self._first_live_page(g, rc.num_tokens)
@@ -242,7 +306,7 @@ class CacheManager:
             while len(table) < start:              # behind the window from the start: never held
                 table.append(-1)
             for i in range(start, hi):
-                table.append(self.pools[g].allocate())
+                table.append(self._allocate(g))
                 rc.dirty[g].append(i)
                 self.stats["pages_allocated"] += 1
 
@@ -334,9 +398,14 @@ class CacheManager:
             taken.append(entry)
             hashes.append(h)
             parent = h
-        for entry in taken:
+        for h, entry in zip(hashes, taken):
+            was_kept = self._kept.pop(h, None) is not None    # held by nobody until now
+            self.stats["kept_page_hits"] += int(was_kept)
             for g, page in enumerate(entry.pages):
-                self.pools[g].retain(page)
+                if was_kept:
+                    self.pools[g].revive(page)
+                else:
+                    self.pools[g].retain(page)
                 rc.dirty[g].append(len(rc.tables[g]))
                 rc.tables[g].append(page)
         n = len(taken) * P
@@ -363,11 +432,15 @@ class CacheManager:
 
     # ---- whole-manager views -------------------------------------------------------
     def num_free_pages(self, group: int = 0) -> int:
-        return self.pools[group].num_free
+        return self.available(group)
 
     def reset(self) -> None:
         for req_id in list(self.requests):
             self.free_request(req_id)
+        for entry in self._kept.values():
+            for g, page in enumerate(entry.pages):
+                self.pools[g].give_back(page)
+        self._kept.clear()
         self._shared.clear()
         self._page_hash.clear()
 
@@ -387,17 +460,23 @@ class CacheManager:
             free = set(pool.free)
             if len(free) != len(pool.free):
                 raise CacheError(f"group {g}: a page is in the free list twice")
+            kept = [entry.pages[g] for entry in self._kept.values()]
+            if len(set(kept)) != len(kept) or free & set(kept):
+                raise CacheError(f"group {g}: a page is kept twice, or kept and free")
             for page in range(pool.num_pages):
                 rcnt = pool.refcount[page]
                 if rcnt != held.get(page, 0):
                     raise CacheError(f"group {g}: page {page} has count {rcnt}, "
                                      f"{held.get(page, 0)} requests hold it")
-                if (rcnt == 0) != (page in free):
-                    raise CacheError(f"group {g}: page {page} count {rcnt}, in free list: {page in free}")
+                if (rcnt == 0) != (page in free or page in kept):
+                    raise CacheError(f"group {g}: page {page} count {rcnt}, free: {page in free}, kept: {page in kept}")
+        for h, entry in self._kept.items():
+            if self._shared.get(h) is not entry:
+                raise CacheError("a kept entry is not registered")
         for h, entry in self._shared.items():
             for g, page in enumerate(entry.pages):
-                if self.pools[g].refcount[page] <= 0:
-                    raise CacheError(f"registered page {page} of group {g} is free")
+                if (self.pools[g].refcount[page] <= 0) != (h in self._kept):
+                    raise CacheError(f"registered page {page} of group {g}: held by nobody and not kept, or kept and held")
             if self._page_hash.get(entry.pages[0]) != h:
                 raise CacheError("the two maps of the prefix registry disagree")
         owners = [o for o in self.slots.owner if o is not None]

@@ -17,6 +17,7 @@ class EngineConfig:
     max_step_tokens: int = 2048      # token budget of one step
     prefill_chunk: int = 512         # largest portion of one prompt in a step
     enable_prefix_sharing: bool = True
+    keep_freed_prefixes: bool = True   # shared pages of finished requests stay until their memory is needed
     seed: int = 0
 
     def pages_per_group(self) -> int:

@@ -41,7 +41,8 @@ class LLMEngine:
         self.tokenizer = tokenizer
         cfg = self.config
         self.runner = ModelRunner(model, page_size=cfg.block_size, num_pages=cfg.pages_per_group(),
-                                  max_requests=cfg.max_num_seqs, prefix_sharing=cfg.enable_prefix_sharing)
+                                  max_requests=cfg.max_num_seqs, prefix_sharing=cfg.enable_prefix_sharing,
+                                  keep_freed_prefixes=cfg.keep_freed_prefixes)
         max_len = min(cfg.max_model_len, model.spec.max_positions)
         self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs, max_len, cfg.max_step_tokens,
                                    cfg.prefill_chunk, model.spec.eos_token_ids)
@@ -133,6 +134,7 @@ class LLMEngine:
         d = dict(self.scheduler.stats)
         d.update(self.runner.cache.stats)
         d["free_pages"] = [p.num_free for p in self.runner.cache.pools]
+        d["kept_pages"] = self.runner.cache.num_kept
         return d
 
 

@@ -72,7 +72,8 @@ class ModelRunner:
     MAX_GRAPHS = 24       # recorded graphs kept (each holds its own activations); the least recently used goes first
 
     def __init__(self, model: DecoderModel, page_size: int, num_pages, max_requests: int,
-                 prefix_sharing: bool = False, use_graphs: Optional[bool] = None):
+                 prefix_sharing: bool = False, use_graphs: Optional[bool] = None,
+                 keep_freed_prefixes: bool = False):
         if model.rt is None:
             raise RuntimeError("the model has no weights yet")
         self.model = model
@@ -82,7 +83,8 @@ class ModelRunner:
         self.plan: CachePlan = cache_plan(model.spec)
         has_state = any(s is not None for s in self.plan.entry_state)
         self.cache = CacheManager(self.plan.groups or [], num_pages, page_size, max_requests,
-                                  prefix_sharing=prefix_sharing and not has_state) \
+                                  prefix_sharing=prefix_sharing and not has_state,
+                                  keep_freed_prefixes=keep_freed_prefixes) \
             if self.plan.groups else CacheManager([], [], page_size, max_requests)
         dev, dt = self.rt.device, self.rt.dtype
         self.kv: List[Optional[torch.Tensor]] = []

@@ -94,7 +94,7 @@ def test_random_orders_keep_every_invariant():
         P = rng.choice([1, 4, 8])
         groups = [GroupSpec()] if trial % 2 else [GroupSpec(), GroupSpec(window=rng.choice([3, 9, 17]))]
         m = CacheManager(groups, rng.choice([6, 12, 40]), page_size=P, max_requests=4,
-                         prefix_sharing=(trial % 2 == 1))
+                         prefix_sharing=(trial % 2 == 1), keep_freed_prefixes=(trial % 4 == 3))
         live, next_id = {}, 0
         common = [rng.randrange(50) for _ in range(3 * P)]
         for _ in range(200):
@@ -130,8 +130,13 @@ def test_random_orders_keep_every_invariant():
         for rid in list(live):
             m.free_request(rid)
         m.check_invariants()
+        assert all(m.available(g) == pool.num_pages for g, pool in enumerate(m.pools))   # free, or kept and free to take
+        if m.keep_freed:
+            assert len(m._shared) == len(m._kept) == len(m._page_hash)
+            m.reset()
+            m.check_invariants()
         assert all(pool.num_free == pool.num_pages for pool in m.pools)
-        assert not m._shared and not m._page_hash
+        assert not m._shared and not m._page_hash and not m._kept
 
 
 def test_prefix_is_shared_by_full_pages_only_and_one_token_is_left():
@@ -161,6 +166,44 @@ def test_prefix_is_shared_by_full_pages_only_and_one_token_is_left():
     assert m.num_free_pages() == 16 and not m._shared   # a freed page leaves the registry
     m.add_request("d")
     assert m.match_prefix("d", prompt) == 0
+
+
+def test_freed_prefixes_are_kept_until_their_memory_is_needed():
+    P = 2
+    m = CacheManager([GroupSpec()], 8, page_size=P, max_requests=2, prefix_sharing=True, keep_freed_prefixes=True)
+    prompt = [1, 2, 3, 4, 5, 6, 7]                       # 3 full pages and one token
+    m.add_request("a")
+    m.reserve("a", 7)
+    m.commit("a", prompt)
+    pages_a = list(m.block_table("a", 0))
+    m.free_request("a")
+    m.check_invariants()
+    assert m.pools[0].num_free == 5 and m.available() == 8          # three pages kept, one freed
+    assert all(m.pools[0].refcount[p] == 0 for p in pages_a)
+    # a later request with the same beginning takes the kept pages over
+    m.add_request("b")
+    assert m.match_prefix("b", prompt) == 6
+    assert m.block_table("b", 0) == pages_a[:3] and m.stats["kept_page_hits"] == 3
+    assert all(m.pools[0].refcount[p] == 1 for p in pages_a[:3])
+    m.check_invariants()
+    m.free_request("b")
+    assert len(m._kept) == 3
+    # a reservation that needs more than the free pages takes kept ones: the last page of the prefix first
+    m.add_request("c")
+    m.reserve("c", 12)                                   # 6 pages: 5 free + 1 kept
+    m.check_invariants()
+    assert m.stats["kept_pages_evicted"] == 1 and len(m._kept) == 2
+    assert pages_a[2] in m.block_table("c", 0) and pages_a[0] not in m.block_table("c", 0)
+    m.add_request("d")
+    assert m.match_prefix("d", prompt) == 4              # the first two pages are still there
+    assert not m.can_reserve([("d", 7)])                 # nothing free, nothing kept
+    with pytest.raises(OutOfPages):
+        m.reserve("d", 7)
+    m.free_request("c")
+    m.free_request("d")
+    m.check_invariants()
+    m.reset()
+    assert m.pools[0].num_free == 8 and not m._shared and not m._kept
 
 
 def test_a_different_token_breaks_the_chain():

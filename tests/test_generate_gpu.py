@@ -58,10 +58,17 @@ def test_outputs_do_not_depend_on_the_engine_sizes(folders, sizes):
     res = eng.run()
     assert [r.token_ids for r in res] == want
     eng.runner.cache.check_invariants()
-    assert all(pool.num_free == pool.num_pages for pool in eng.runner.cache.pools)
+    cache = eng.runner.cache                                  # (pages kept for later requests count as free to take)
+    assert all(cache.available(g) == pool.num_pages for g, pool in enumerate(cache.pools))
     # temperature: the same tokens as a run of each request alone with the same seed
+    hits_before = eng.stats()["kept_page_hits"]
     eng.submit(p, max_new_tokens=10, temperature=0.7, seed=11, ignore_eos=True)
     together = [r.token_ids for r in eng.run()]
+    # the second run found full pages of the first run's prompts, kept though those requests had ended
+    if sizes.get("enable_prefix_sharing", True):
+        assert eng.stats()["kept_page_hits"] > hits_before
+    else:
+        assert eng.stats()["kept_page_hits"] == 0 and cache.num_kept == 0
     ref_engine = LLMEngine.from_folder(folders["B"], EngineConfig(dtype="float32", block_size=8, max_num_seqs=1,
                                                                   max_model_len=48))
     alone = []
@@ -90,7 +97,8 @@ def test_bfloat16_generation_on_the_mfma_kernels(folders, sizes):
     if "num_blocks" in sizes:
         assert eng.stats()["preemptions"] > 0
     eng.runner.cache.check_invariants()
-    assert all(pool.num_free == pool.num_pages for pool in eng.runner.cache.pools)
+    cache = eng.runner.cache                                  # (pages kept for later requests count as free to take)
+    assert all(cache.available(g) == pool.num_pages for g, pool in enumerate(cache.pools))
     for r, prompt in zip(res, prompts):
         assert r.finish_reason == "length" and len(r.token_ids) == 40
         logits = P.forward_logits(cfg, w, prompt + r.token_ids[:-1], act_dtype=torch.bfloat16)
