@@ -16,7 +16,9 @@
 //       scale * log2 e once); the accumulator is rescaled only when a maximum moved
 //   O^T[d, col] += V^T[d, key] . P^T[key, col]    v_mfma_f32_32x32x16_bf16, 2 * D / 32 of them;
 //       the 8 probabilities of a half tile that a lane holds are its B operand as they lie, and
-//       because value tiles are stored transposed ([D][P]) the A operand is two 8-byte reads
+//       because value tiles are stored transposed ([D][P]) the A operand is the same 8 keys of
+//       one row of V^T: the staged rows hold the keys in the order 0-3, 8-11, 4-7, 12-15, so that
+//       it is one 16-byte read
 // The causal and window limits are applied per column, so the order of the sums for a row
 // depends on its position and the window only.
 //
@@ -32,7 +34,7 @@ typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(16))) float floatx16;
 typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
 
-union PackV {   // two 8-byte pieces of a value row as one MFMA operand
+union PackV {   // an MFMA operand, also addressable as two 8-byte pieces
     bf16x8 v;
     uint2 u[2];
 };
@@ -42,7 +44,17 @@ union Piece {   // a staged 16-byte piece, addressable by element for masking
     unsigned short e[8];
 };
 
-#define VROW 40   // bytes of a staged value row: 16 keys = 32 bytes of data + 8 of padding
+// Lane i and lane i ^ 32 exchange a value without a trip through shared memory.
+__device__ __forceinline__ float max_of_both_halves(float v) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+}
+__device__ __forceinline__ float sum_of_both_halves(float v) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+}
+
+#define VROW 48   // bytes of a staged value row: 16 keys = 32 bytes of data + 16 of padding
 
 // Two waves per SIMD (at most 256 registers a lane), as two blocks of one group or one block of
 // two: while one wave waits for its next tile or at its barrier, the other computes.
@@ -169,9 +181,9 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
         }                                                                                           \
         _Pragma("unroll") for (int i = 0; i < VP; ++i) {                                            \
             const int id = tid + 256 * i;                                                           \
-            unsigned char* dst = vs_ + (id >> 1) * VROW + (id & 1) * 16;                            \
+            unsigned char* dst = vs_ + (id >> 1) * VROW + (id & 1) * 8;                             \
             *(uint2*)dst = vst[set_][i].u[0];                                                       \
-            *(uint2*)(dst + 8) = vst[set_][i].u[1];                                                 \
+            *(uint2*)(dst + 16) = vst[set_][i].u[1];                                                \
         }                                                                                           \
     }
 
@@ -199,7 +211,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
         __builtin_amdgcn_sched_barrier(0);                // keep the loads ahead of the computation
         if (wave_on && kk < k_stop && kk + 32 > k_start) { // some row of the wave sees some key of the tile (none beyond kmax)
             const unsigned char* ks_ = smem + buf * BUF + r * KROW + g * 16;
-            const unsigned char* vs_ = smem + buf * BUF + KBYTES + r * VROW + g * 8;
+            const unsigned char* vs_ = smem + buf * BUF + KBYTES + r * VROW + g * 16;
             // all key fragments are read before the first MFMA, all value fragments before the
             // softmax: shared-memory latency then passes under the arithmetic instead of before it
             bf16x8 kf[D / 16];
@@ -217,9 +229,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
             for (int db = 0; db < D / 32; ++db)
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    const unsigned char* vp = vs_ + (h * D + db * 32) * VROW;
-                    vf[db][h].u[0] = *(const uint2*)vp;
-                    vf[db][h].u[1] = *(const uint2*)(vp + 16);
+                    vf[db][h].v = *(const bf16x8*)(vs_ + (h * D + db * 32) * VROW);
                 }
 
             // (the scores stay unscaled: the scale is positive, so it is applied to the maximum, and
@@ -236,7 +246,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
                     tmax = fmaxf(tmax, s[e]);
                 }
             }
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            tmax = max_of_both_halves(tmax);
             const float mn = fmaxf(m, tmax * scale_log2);
             const float ref = (mn == -INFINITY) ? 0.f : mn;   // a column that has seen no key yet: all weights 0
             if (__any(mn > m)) {                              // some column's maximum moved: rescale
@@ -269,7 +279,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
 #undef STAGE_LOAD
 #undef STAGE_STORE
 #undef TILE_KEY
-    l += __shfl_xor(l, 32, 64);
+    l = sum_of_both_halves(l);
     if (NG == 2) {
         // group 1 hands its maxima, sums and accumulators to group 0, 16 values of every lane at a
         // time, through the staging memory (free after the loop's last barrier): [wave][value][lane]
