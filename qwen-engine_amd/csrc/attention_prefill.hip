@@ -13,7 +13,8 @@
 //       lane (g, r), g = lane / 32, r = lane % 32, takes K[key r][ks * 16 + g * 8 .. + 8]
 //       and ends up with 16 scores: keys 8 b + 4 g + j (b, j < 4) of column r
 //   online softmax per column in 32-bit, in the base-2 domain (scores are scaled by
-//       scale * log2 e once); the accumulator is rescaled only when a maximum moved
+//       scale * log2 e once); the accumulator is rescaled only when a score exceeds the column's
+//       reference by more than 8
 //   O^T[d, col] += V^T[d, key] . P^T[key, col]    v_mfma_f32_32x32x16_bf16, 2 * D / 32 of them;
 //       the 8 probabilities of a half tile that a lane holds are its B operand as they lie, and
 //       because value tiles are stored transposed ([D][P]) the A operand is the same 8 keys of
@@ -70,8 +71,10 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     constexpr int VP = 2 * D * 2 / 256;              // 16-byte value pieces per thread
     __shared__ __attribute__((aligned(16))) unsigned char smem_all[NG * 2 * BUF];
 
-    const int grp = threadIdx.x / 256;                     // which half of the key tiles (NG = 2)
-    const int tid = threadIdx.x % 256, lane = tid & 63, wave = tid >> 6;
+    // (group and wave are the same for all lanes of a wave: kept in scalar registers, so that what
+    // follows from them — tile keys, pages, addresses — is scalar arithmetic)
+    const int grp = __builtin_amdgcn_readfirstlane(threadIdx.x / 256);   // which half of the key tiles (NG = 2)
+    const int tid = threadIdx.x % 256, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     unsigned char* smem = smem_all + grp * 2 * BUF;
     const int g = lane >> 5, r = lane & 31;
     const int G = Hq / Hkv;
@@ -129,37 +132,44 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     // Two sets of staging registers in turn: the loads of a tile are issued two tiles ahead and
     // stored to shared memory one tile ahead, so a load has a whole tile's computation to arrive
     // (one tile of arithmetic is shorter than a trip to memory).
+    // The loads are buffer loads: the page's address and the offset of the 16 keys in it are
+    // scalar, and a thread adds bytes that are constant over the loop.  Which half of the tile a
+    // piece belongs to is the same for a whole wave (256 pieces are 2 D / 8 rows of 8 pieces).
     Piece kst[2][KP], vst[2][VP];
-    // what a thread adds to (page base + offset-in-page scaled) to reach its pieces: constant over the loop
-    long kconst[KP], vconst[VP];
+    int kconst[KP], vconst[VP];                           // bytes from the page's start, without the keys' offset
     bool khalf[KP], vhalf[VP];
 #pragma unroll
     for (int i = 0; i < KP; ++i) {
         const int id = tid + 256 * i;
         const int krow = id / (D / 8), col = id % (D / 8);
-        khalf[i] = krow >= 16;
-        kconst[i] = ((long)kvh * P + (krow & 15)) * D + col * 8;
+        khalf[i] = __builtin_amdgcn_readfirstlane(krow >= 16);
+        kconst[i] = ((kvh * P + (krow & 15)) * D + col * 8) * 2;
     }
 #pragma unroll
     for (int i = 0; i < VP; ++i) {
         const int id = tid + 256 * i;
         const int rem = id % (2 * D);
-        vhalf[i] = id >= 2 * D;
-        vconst[i] = ((long)(Hkv + kvh) * P) * D + (long)(rem >> 1) * P + (rem & 1) * 8;
+        vhalf[i] = __builtin_amdgcn_readfirstlane(id >= 2 * D);
+        vconst[i] = (((Hkv + kvh) * P) * D + (rem >> 1) * P + (rem & 1) * 8) * 2;
     }
     const int pmask = P - 1;
+    const int page_bytes = (int)page_stride * 2;
 #define STAGE_LOAD(set_, kk_)                                                                       \
     {                                                                                               \
         const bool first_ = (kk_) + 16 > kmin, second_ = (kk_) + 16 < kmax;                         \
         const int ka_ = first_ ? (kk_) : (kk_) + 16;                                                \
         const int kb_ = second_ ? (kk_) + 16 : (kk_);                                               \
-        const long pa_ = (long)bt[ka_ >> log2P] * page_stride, pb_ = (long)bt[kb_ >> log2P] * page_stride; \
-        const int oa_ = ka_ & pmask, ob_ = kb_ & pmask;                                             \
-        const long ka_base = pa_ + (long)oa_ * D, kb_base = pb_ + (long)ob_ * D;                    \
+        const __amdgpu_buffer_rsrc_t ra_ = __builtin_amdgcn_make_buffer_rsrc(                       \
+            (void*)(cache + (long)bt[ka_ >> log2P] * page_stride), 0, page_bytes, 0x00020000);      \
+        const __amdgpu_buffer_rsrc_t rb_ = __builtin_amdgcn_make_buffer_rsrc(                       \
+            (void*)(cache + (long)bt[kb_ >> log2P] * page_stride), 0, page_bytes, 0x00020000);      \
+        const int oa_ = (ka_ & pmask) * 2, ob_ = (kb_ & pmask) * 2;   /* bytes in a row of V^T */   \
         _Pragma("unroll") for (int i = 0; i < KP; ++i)                                              \
-            kst[set_][i].q = *(const uint4_t*)(cache + (khalf[i] ? kb_base : ka_base) + kconst[i]); \
+            kst[set_][i].q = __builtin_amdgcn_raw_buffer_load_b128(khalf[i] ? rb_ : ra_, kconst[i], \
+                                                                   (khalf[i] ? ob_ : oa_) * D, 0);  \
         _Pragma("unroll") for (int i = 0; i < VP; ++i)                                              \
-            vst[set_][i].q = *(const uint4_t*)(cache + (vhalf[i] ? pb_ + ob_ : pa_ + oa_) + vconst[i]); \
+            vst[set_][i].q = __builtin_amdgcn_raw_buffer_load_b128(vhalf[i] ? rb_ : ra_, vconst[i], \
+                                                                   vhalf[i] ? ob_ : oa_, 0);        \
     }
 #define STAGE_STORE(buf_, set_, kk_)                                                                \
     {                                                                                               \
@@ -246,16 +256,20 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
                     tmax = fmaxf(tmax, s[e]);
                 }
             }
-            tmax = max_of_both_halves(tmax);
-            const float mn = fmaxf(m, tmax * scale_log2);
-            const float ref = (mn == -INFINITY) ? 0.f : mn;   // a column that has seen no key yet: all weights 0
-            if (__any(mn > m)) {                              // some column's maximum moved: rescale
-                const float alpha = __builtin_amdgcn_exp2f(m - ref);
+            tmax = max_of_both_halves(tmax) * scale_log2;
+            // m is the reference the weights are taken against, not the exact maximum: a column moves
+            // it only when a score exceeds it by more than 8 (a weight above 2^8), which after the
+            // first tiles is rare, so that the accumulators are seldom rescaled.  The decision is the
+            // column's own: its sums do not depend on the other columns of the wave.
+            const bool moves = tmax > m + 8.f;                 // (never for a tile without a visible key)
+            if (__any(moves)) {
+                const float alpha = moves ? __builtin_amdgcn_exp2f(m - tmax) : 1.f;   // 0 from a column's first keys
+                m = moves ? tmax : m;
                 l *= alpha;
 #pragma unroll
                 for (int db = 0; db < D / 32; ++db) acc[db] *= alpha;
             }
-            m = mn;
+            const float ref = (m == -INFINITY) ? 0.f : m;      // a column that has seen no key yet: all weights 0
             PackV pb[2];
             float psum = 0.f;
 #pragma unroll
@@ -343,6 +357,7 @@ int qe_attention_prefill(const void* q, void* out, const void* cache, const int*
     int log2P = 0;
     while ((1 << log2P) < P) ++log2P;
     QE_REQUIRE(num_tiles % 4 == 0, "prefill attention: tiles come in groups of four");
+    QE_REQUIRE(4L * Hkv * P * D < (1L << 31), "prefill attention: a page of %ld bytes is too large", 4L * Hkv * P * D);
     if (num_tiles == 0) return 0;
     const int R = qe_attention_prefill_tile_rows(Hq, Hkv);
     const int waves_per_kv = (Hq / Hkv) / (32 / R);
