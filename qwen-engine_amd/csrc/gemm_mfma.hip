@@ -13,7 +13,9 @@
 // take; loads have to be in flight two steps ahead to arrive in time; and the result has to be
 // stored as whole rows.  128 x 128 tiles (four waves, two blocks a compute unit) are the default,
 // 64 x 128 where there would be too few blocks otherwise, 256 x 128 (eight waves) where even
-// those give every compute unit two blocks.
+// those give every compute unit two blocks, 256 x 256 (four waves, a wave's part 128 x 128) where
+// even that shape gives every compute unit two blocks in turn: it reads half the bytes per MFMA
+// from the L1 and from shared memory.
 //
 // Rows of x beyond M and rows of W beyond N are read as zero and never stored; K must be a
 // multiple of 8 (16-byte loads), a tail shorter than BK is filled with zeros.
@@ -27,6 +29,10 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
 // SILU: W holds gate and up rows interleaved in blocks of 32 (gate 0..31, up 0..31, gate 32..63,
 // ...), N counts all of them, and the result is silu(gate) * up, N / 2 wide: the two MFMA tiles a
 // lane holds side by side are the gate and the up of the same outputs.
+// BIG (256 x 256 by four waves, one wave a SIMD, a wave's part 128 x 128): the accumulators fill the
+// 256 AGPRs, so there is one set of staging registers, in VGPRs, loaded one step ahead (a step is
+// 2048 cycles of MFMAs, longer than a trip to the L2).  Per MFMA this shape reads half the bytes
+// from the L1 and from shared memory that 128 x 128 by four waves reads.
 template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU>
 __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
@@ -37,7 +43,10 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     constexpr int WM = BM / (NW / 2), WN = BN / 2;   // a wave's part: NW / 2 waves down, 2 across
     constexpr int MI = WM / 32, NJ = WN / 32;
     constexpr int LDA = BM / RPI, LD = (BM + BN) / RPI;   // pieces a thread stages per step: LDA of x, then of W
-    static_assert((LD == 12 || LD == 8 || LD == 6) && BM % RPI == 0 && BN % RPI == 0, "tile rows must be a multiple of the rows staged at once");
+    constexpr bool BIG = BM == 256 && BN == 256 && NW == 4;
+    constexpr int SETS = BIG ? 1 : 2;
+    static_assert((LD == 16 || LD == 12 || LD == 8 || LD == 6) && (LD == 16) == BIG && BM % RPI == 0 && BN % RPI == 0,
+                  "tile rows must be a multiple of the rows staged at once");
     constexpr int BUF = (BM + BN) * ROWB;   // bytes of one buffer: the x rows, then the W rows
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -68,7 +77,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const int nk = (klen + BK - 1) / BK;
     // Two sets of staging registers in turn: a step's loads are issued two steps ahead and go to
     // shared memory one step ahead, so a load has a whole step of MFMAs to arrive.
-    uint4_t stage[2][LD];
+    uint4_t stage[SETS][LD];
 
     // Piece i of a thread is row (tid / PPR) of the i-th group of RPI rows, 16 bytes at k = 8 (tid % PPR).
     // The loads are buffer loads: one descriptor for the tile's rows of x and one for its rows of W,
@@ -105,7 +114,14 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
         const int soff = (kt_) * BK * 2;                                                 \
         _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                 \
             const int vo = k_ok ? voff[i] : 0x7fffffff;                                  \
-            if (i < LDA)                                                                 \
+            if constexpr (BIG) {                                                         \
+                if (i < LDA)                                                             \
+                    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"              \
+                                 : "=&v"(stage[set_][i]) : "v"(vo), "s"(rsrc_a), "s"(soff) : "memory"); \
+                else                                                                     \
+                    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"              \
+                                 : "=&v"(stage[set_][i]) : "v"(vo), "s"(rsrc_b), "s"(soff) : "memory"); \
+            } else if (i < LDA)                                                          \
                 asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                  \
                              : "=&a"(stage[set_][i]) : "v"(vo), "s"(rsrc_a), "s"(soff) : "memory"); \
             else                                                                         \
@@ -115,7 +131,15 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     }
     // waits until at most `younger_` loads are in flight; the set's registers are valid afterwards
 #define WAIT_LOADS(set_, younger_)                                                       \
-    if constexpr (LD == 12)                                                              \
+    if constexpr (LD == 16)                                                              \
+        asm volatile("s_waitcnt vmcnt(%16)"                                              \
+                     : "+v"(stage[set_][0]), "+v"(stage[set_][1]), "+v"(stage[set_][2]), "+v"(stage[set_][3]), \
+                       "+v"(stage[set_][4]), "+v"(stage[set_][5]), "+v"(stage[set_][6 % LD]), "+v"(stage[set_][7 % LD]), \
+                       "+v"(stage[set_][8 % LD]), "+v"(stage[set_][9 % LD]), "+v"(stage[set_][10 % LD]),       \
+                       "+v"(stage[set_][11 % LD]), "+v"(stage[set_][12 % LD]), "+v"(stage[set_][13 % LD]),     \
+                       "+v"(stage[set_][14 % LD]), "+v"(stage[set_][15 % LD])                                  \
+                     : "n"(younger_) : "memory");                                        \
+    else if constexpr (LD == 12)                                                         \
         asm volatile("s_waitcnt vmcnt(%12)"                                              \
                      : "+a"(stage[set_][0]), "+a"(stage[set_][1]), "+a"(stage[set_][2]), "+a"(stage[set_][3]), \
                        "+a"(stage[set_][4]), "+a"(stage[set_][5]), "+a"(stage[set_][6]), "+a"(stage[set_][7]), \
@@ -134,7 +158,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
                      : "n"(younger_) : "memory");
 #define STORE_SHARED(buf_)                                                               \
     _Pragma("unroll") for (int i = 0; i < LD; ++i)                                       \
-        *(uint4_t*)(smem + (buf_) * BUF + dst + i * RPI * ROWB) = stage[buf_][i];
+        *(uint4_t*)(smem + (buf_) * BUF + dst + i * RPI * ROWB) = stage[(buf_) % SETS][i];
 
     floatx16 acc[MI][NJ];
 #pragma unroll
@@ -151,6 +175,8 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     // One step on buffer buf_ (a constant, so every shared-memory address is base + immediate).
     // The fragments of k step ks + 1 are read while the MFMAs of ks run, and the stores of the
     // next step's tile are issued before the last MFMAs, whose time then covers them.
+    // (Passing the barrier before those last MFMAs and reading the next step's first fragments
+    // under them was tried: 3 % faster with one wave a SIMD, 10 % slower with two.)
 #define READ_FRAGS(buf_, ks_, a_, b_)                                                    \
     _Pragma("unroll") for (int i = 0; i < MI; ++i)                                       \
         a_[i] = *(const bf16x8*)(a_frag + (buf_) * BUF + i * 32 * ROWB + (ks_) * 32);    \
@@ -164,7 +190,8 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     {                                                                                    \
         bf16x8 fa[2][MI], fb[2][NJ];                                                     \
         READ_FRAGS(buf_, 0, fa[0], fb[0])                                                \
-        LOAD_GLOBAL(buf_, (kt_) + 2)   /* this set went to shared memory a step ago */   \
+        if constexpr (SETS == 2) LOAD_GLOBAL(buf_, (kt_) + 2)   /* this set went to shared memory a step ago */ \
+        else LOAD_GLOBAL(0, (kt_) + 1)                                                   \
         __builtin_amdgcn_sched_barrier(0);                                               \
         _Pragma("unroll") for (int ks = 0; ks < BK / 16 - 1; ++ks) {                     \
             READ_FRAGS(buf_, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1])                 \
@@ -174,33 +201,82 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
         }                                                                                \
         /* the other buffer: its readers finished before the last barrier (after the last step  \
            this stores a step that does not exist, which nobody reads) */                    \
-        WAIT_LOADS((buf_) ^ 1, LD)   /* the LD loads just issued may stay in flight */   \
+        if constexpr (SETS == 2) { WAIT_LOADS((buf_) ^ 1, LD) }   /* the LD loads just issued may stay in flight */ \
+        else { WAIT_LOADS(0, 0) }                                                        \
         STORE_SHARED((buf_) ^ 1)                                                         \
         __builtin_amdgcn_sched_barrier(0);                                               \
         MFMAS(fa[(BK / 16 - 1) & 1], fb[(BK / 16 - 1) & 1])                              \
         __builtin_amdgcn_sched_barrier(0);                                               \
         __syncthreads();                                                                 \
     }
+    // The step of the BIG shape.  A wave is alone on its SIMD and issues in order, so whatever is
+    // not an MFMA is put between the MFMAs, one a time: the 16 loads of the next step among the 16
+    // MFMAs of the first k step, the 16 stores to shared memory among those of the last.
+#define LOAD_PIECE(kt_, i_)                                                              \
+    {                                                                                    \
+        const int vo = (kt_) * BK + pc * 8 < klen ? voff[i_] : 0x7fffffff;               \
+        const int soff = (kt_) * BK * 2;                                                 \
+        if ((i_) < LDA)                                                                  \
+            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                      \
+                         : "=&v"(stage[0][i_]) : "v"(vo), "s"(rsrc_a), "s"(soff) : "memory"); \
+        else                                                                             \
+            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                      \
+                         : "=&v"(stage[0][i_]) : "v"(vo), "s"(rsrc_b), "s"(soff) : "memory"); \
+    }
+#define K_STEP_BIG(buf_, kt_)                                                            \
+    {                                                                                    \
+        bf16x8 fa[2][MI], fb[2][NJ];                                                     \
+        READ_FRAGS(buf_, 0, fa[0], fb[0])                                                \
+        _Pragma("unroll") for (int ks = 0; ks < BK / 16; ++ks) {                         \
+            if (ks + 1 < BK / 16) { READ_FRAGS(buf_, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]) } \
+            if (ks == BK / 16 - 1) { WAIT_LOADS(0, 0) }                                  \
+            __builtin_amdgcn_sched_barrier(0);                                           \
+            _Pragma("unroll") for (int i = 0; i < MI; ++i)                               \
+                _Pragma("unroll") for (int j = 0; j < NJ; ++j) {                         \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks & 1][j], fa[ks & 1][i], acc[i][j], 0, 0, 0); \
+                    if (ks == 0) LOAD_PIECE((kt_) + 1, (i * NJ + j) % LD)                \
+                    if (ks == BK / 16 - 1)                                               \
+                        *(uint4_t*)(smem + ((buf_) ^ 1) * BUF + dst + ((i * NJ + j) % LD) * RPI * ROWB) = stage[0][(i * NJ + j) % LD]; \
+                    __builtin_amdgcn_sched_barrier(0);                                   \
+                }                                                                        \
+        }                                                                                \
+        __syncthreads();                                                                 \
+    }
 
     // step kt uses buffer and register set kt % 2
     LOAD_GLOBAL(0, 0)
-    LOAD_GLOBAL(1, 1)
-    WAIT_LOADS(0, LD)
+    if constexpr (SETS == 2) {
+        LOAD_GLOBAL(1, 1)
+        WAIT_LOADS(0, LD)
+    } else {
+        WAIT_LOADS(0, 0)
+    }
     STORE_SHARED(0)
     __syncthreads();
     // (two steps in a body without branches, and an odd last step after the loop)
     int kt = 0;
-    for (; kt + 1 < nk; kt += 2) {
-        K_STEP(0, kt)
-        K_STEP(1, kt + 1)
+    if constexpr (BIG) {
+        static_assert(!BIG || MI * NJ == LD, "one load and one store per MFMA of a k step");
+        for (; kt + 1 < nk; kt += 2) {
+            K_STEP_BIG(0, kt)
+            K_STEP_BIG(1, kt + 1)
+        }
+        if (kt < nk) K_STEP_BIG(0, kt)
+    } else {
+        for (; kt + 1 < nk; kt += 2) {
+            K_STEP(0, kt)
+            K_STEP(1, kt + 1)
+        }
+        if (kt < nk) K_STEP(0, kt)
     }
-    if (kt < nk) K_STEP(0, kt)
     // The loads past the end are still in flight and the compiler does not know of them: their
     // registers pass through a last wait, so that they stay reserved until the loads have landed
     // (a register whose value nobody uses would be handed out again at once).
     WAIT_LOADS(0, 0)
-    WAIT_LOADS(1, 0)
+    if constexpr (SETS == 2) { WAIT_LOADS(1, 0) }
 #undef K_STEP
+#undef K_STEP_BIG
+#undef LOAD_PIECE
 #undef READ_FRAGS
 #undef MFMAS
 #undef LOAD_GLOBAL
@@ -304,21 +380,25 @@ static int pick_mfma(const void* x, const void* w, const float* bias, void* out,
                      int tile, int splits, hipStream_t stream) {
     const long cus = 256;
     const long big = (long)qe_cdiv(M, 256) * qe_cdiv(N, 128) * splits, mid = (long)qe_cdiv(M, 128) * qe_cdiv(N, 128) * splits;
+    const long huge = (long)qe_cdiv(M, 256) * qe_cdiv(N, 256) * splits;
     // the largest tile that still gives every compute unit two blocks (one, for the middle size)
-    if (tile == 0) tile = (big >= 2 * cus && M > 128) ? 256 : ((mid >= cus && M > 64) ? 128 : 64);   // never taller than the rows need
+    if (tile == 0)
+        tile = (huge >= 2 * cus && M > 128) ? 512
+             : ((big >= 2 * cus && M > 128) ? 256 : ((mid >= cus && M > 64) ? 128 : 64));   // never taller than the rows need
+    if (tile == 512) return launch_mfma<TO, 256, 256, 64, 4, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 256) return launch_mfma<TO, 256, 128, 64, 8, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 128) return launch_mfma<TO, 128, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, splits, stream);
     return launch_mfma<TO, 64, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, splits, stream);
 }
 
-// tile: rows of the output tile (256, 128 or 64), 0 to choose by the shape.  silu: w is [N, K] with
+// tile: rows of the output tile (256, 128 or 64; 512 stands for 256 x 256), 0 to choose by the shape.  silu: w is [N, K] with
 // gate and up rows interleaved in blocks of 32, out is [M, N / 2] = silu(gate) * up.
 // splits > 1: out is float [splits, M, N], partial products along K (no silu then).
 int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
                  int tile, bool silu, int splits, hipStream_t stream) {
     QE_REQUIRE(splits >= 1 && (splits == 1 || (!silu && dt_o == QE_F32)), "mfma gemm: partial products are 32-bit and plain");
     QE_REQUIRE(K % 8 == 0 && K >= 64 && K < (1 << 22), "mfma gemm: K=%d is no multiple of 8 in [64, 2^22)", K);
-    QE_REQUIRE(tile == 0 || tile == 256 || tile == 128 || tile == 64, "mfma gemm: tile of %d rows", tile);
+    QE_REQUIRE(tile == 0 || tile == 512 || tile == 256 || tile == 128 || tile == 64, "mfma gemm: tile of %d rows", tile);
     if (silu) {
         QE_REQUIRE(!bias && N % 64 == 0, "mfma gemm: silu-mul takes no bias and gate|up rows in blocks of 32");
         if (dt_o == QE_BF16) return pick_mfma<bf16_t, true>(x, w, bias, out, M, N, K, tile, splits, stream);

@@ -563,7 +563,7 @@ def test_gemm_tiled_mfma(ops, M, N, K):
     want = P.linear(x.double(), w.double())
     got = ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_FAST)
     close(got, want, bf)
-    for rows in (64, 128, 256):                              # every tile shape on every size
+    for rows in (64, 128, 256, 512):                         # every tile shape on every size (512: 256 x 256)
         close(ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_TILE + rows), want, bf)
         close(ops.gemm(x.to(DEV), w.to(DEV), bias.to(DEV), out_dtype=torch.float32, algo=ops.ALGO_TILE + rows),
               want + bias.double(), torch.float32, scale=float(want.abs().max()))
@@ -699,7 +699,7 @@ def test_gemm_with_silu_mul_over_interleaved_rows(ops, M, I, K):
     if ops.gemm_silu_supported(x.to(DEV), w.to(DEV)):
         close(ops.gemm(x.to(DEV), w.to(DEV), epilogue=ops.EPI_SILU_MUL_IL), want, bf)
         if M > 64:
-            for rows in (64, 128, 256):
+            for rows in (64, 128, 256, 512):
                 close(ops.gemm(x.to(DEV), w.to(DEV), epilogue=ops.EPI_SILU_MUL_IL, algo=ops.ALGO_TILE + rows), want, bf)
     gu = ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_GENERIC)
     close(ops.silu_mul(gu, interleaved=True), want, bf)
