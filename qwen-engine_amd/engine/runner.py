@@ -117,7 +117,8 @@ class ModelRunner:
         self.table_width = [max(1, per_request if grp.window is not None else min(pool.num_pages, per_request))
                             for grp, pool in zip(self.cache.groups, self.cache.pools)]
         self.tables = [torch.full((max_requests, w), -1, dtype=torch.int32, device=dev) for w in self.table_width]
-        self.use_graphs = (dt == torch.bfloat16 and not has_state) if use_graphs is None else bool(use_graphs)
+        graph_safe = not has_state and getattr(model, "graph_safe", True)
+        self.use_graphs = (dt == torch.bfloat16 and graph_safe) if use_graphs is None else bool(use_graphs)
         self._graphs = {}
         self._stage: Optional[torch.Tensor] = None     # pinned host buffer of a step's integer arrays
         self._stage_np = None

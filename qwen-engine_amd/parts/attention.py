@@ -37,6 +37,10 @@ class PagedAttention:
         self.position = build_part(spec.position, hidden_size) if spec.position is not None else None
         self.w_qkv = self.b_qkv = self.w_o = self.q_norm = self.k_norm = None
 
+    @property
+    def graph_safe(self) -> bool:
+        return getattr(self.position, "graph_safe", True)
+
     # ---- what it needs ----------------------------------------------------------
     @staticmethod
     def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:

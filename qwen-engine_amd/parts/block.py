@@ -28,6 +28,11 @@ class PreNormBlock:
         self.ffn_norm = build_part(spec.ffn_norm, hidden_size)
         self.ffn = build_part(spec.ffn, hidden_size)
 
+    @property
+    def graph_safe(self) -> bool:
+        """False if any part of the block says that its forward cannot be recorded into a graph."""
+        return all(getattr(p, "graph_safe", True) for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
+
     @staticmethod
     def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
         out: Dict[str, TensorInfo] = {}

@@ -50,6 +50,13 @@ class DecoderModel:
         self.head: Optional[torch.Tensor] = None
         self.rt: Optional[Runtime] = None
 
+    @property
+    def graph_safe(self) -> bool:
+        """A part whose forward reads results back on the host, sizes tensors by their contents or
+        walks the requests of a step sets ``graph_safe = False``; the decode steps of a model with
+        such a part are run as they come instead of being recorded once and replayed."""
+        return all(getattr(p, "graph_safe", True) for p in (*self.blocks, self.final_norm))
+
     def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
         spec = self.spec
         self.rt = rt

@@ -4,7 +4,9 @@ A part class has
   * ``expected_tensors(spec, hidden_size) -> {relative name: TensorInfo}``
   * ``__init__(spec, hidden_size)`` (no GPU needed)
   * ``load(tensors, rt)`` with the tensors named above, as stored, on the CPU
-and, by role, the forward interface described in ``parts.base``.
+and, by role, the forward interface described in ``parts.base``.  A part whose forward
+cannot be recorded into a HIP graph (it reads results back on the host, or sizes tensors
+by their contents) says so with a class attribute ``graph_safe = False``.
 """
 from __future__ import annotations
 
