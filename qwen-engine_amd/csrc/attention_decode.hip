@@ -23,7 +23,7 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     const int lane = threadIdx.x, g = lane >> 4, n = lane & 15;
     const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
     const int G = Hq / Hkv;
-    const int t = dec_tokens[di];
+    const int t = dec_tokens ? dec_tokens[di] : di;       // (no list: every row, in order)
     const int p = positions[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int k_begin = max(split * SPLIT, lo);
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(64) void attention_decode_fused_split_kernel(
     const int lane = threadIdx.x, g = lane >> 4, n = lane & 15;
     const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
     const int G = Hq / Hkv;
-    const int t = dec_tokens[di];
+    const int t = dec_tokens ? dec_tokens[di] : di;       // (no list: every row, in order)
     const int p = positions[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const bool own = split == p / SPLIT;                   // this wave takes the token's own key and value
@@ -348,7 +348,7 @@ __global__ __launch_bounds__(256) void attention_decode_merge_kernel(
     __syncthreads();
     if (wave == 0) {
         const float inv = 1.f / (red_l[0] + red_l[1] + red_l[2] + red_l[3]);
-        bf16_t* orow = out + ((long)dec_tokens[di] * Hq + head) * D;
+        bf16_t* orow = out + ((long)(dec_tokens ? dec_tokens[di] : di) * Hq + head) * D;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             const int d = lane + i * 64;
@@ -366,7 +366,8 @@ size_t qe_attention_decode_workspace(int n_dec, int Hq, int D, int num_splits) {
     return (size_t)n_dec * Hq * num_splits * (D + 2) * sizeof(float);
 }
 
-// dec_tokens: the rows of q that are single new tokens of their requests.  max_position: the
+// dec_tokens: the rows of q that are single new tokens of their requests (null: the rows
+// 0 .. n_dec - 1, which saves every wave a dependent load).  max_position: the
 // largest of their positions (fixes the number of splits).  workspace: at least
 // qe_attention_decode_workspace(...) bytes.
 int qe_attention_decode(const void* q, void* out, const void* cache, const int* dec_tokens, int n_dec,

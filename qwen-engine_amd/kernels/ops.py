@@ -416,15 +416,16 @@ def attention_decode_fused_supported(qkv: torch.Tensor, cache: torch.Tensor, num
 
 def attention_decode_fused(qkv: torch.Tensor, num_heads: int, cache: torch.Tensor, positions: torch.Tensor,
                            tok_seq: torch.Tensor, block_table: torch.Tensor, scale: float, window: int,
-                           dec_tokens: torch.Tensor, max_dec_position: int,
+                           dec_tokens: Optional[torch.Tensor], max_dec_position: int,
                            q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                            table: Optional[torch.Tensor], slots: Optional[torch.Tensor],
                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of single new tokens with the step before it inside: per-head q/k RMSNorm
     (weights or None), half-split rotation from ``table`` (rows [cos | sin] of the head size, or
     None) and the write of each token's key and value to cache slot ``slots[t]`` (negative or no
-    slots: not written).  qkv [T, (Hq + 2 Hkv) D] bfloat16; the rows ``dec_tokens`` are computed
-    into out [T, Hq, D]; the cache holds each request's keys before the token's own position."""
+    slots: not written).  qkv [T, (Hq + 2 Hkv) D] bfloat16; the rows ``dec_tokens`` (None: all
+    rows) are computed into out [T, Hq, D]; the cache holds each request's keys before the
+    token's own position."""
     lib = load_library()
     _need(qkv, "qkv", torch.bfloat16, (None, None))
     T, dev = qkv.shape[0], qkv.device
@@ -438,7 +439,8 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, cache: torch.Tenso
     _need(positions, "positions", torch.int32, (T,), dev)
     _need(tok_seq, "tok_seq", torch.int32, (T,), dev)
     _need(block_table, "block_table", torch.int32, (None, None), dev)
-    _need(dec_tokens, "dec_tokens", torch.int32, (None,), dev)
+    if dec_tokens is not None:
+        _need(dec_tokens, "dec_tokens", torch.int32, (None,), dev)
     if q_weight is not None:
         _need(q_weight, "q_weight", torch.float32, (D,), dev)
     if k_weight is not None:
@@ -450,12 +452,12 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, cache: torch.Tenso
     if out is None:
         out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=dev)
     _need(out, "out", torch.bfloat16, (T, Hq, D), dev)
-    n_dec = dec_tokens.shape[0]
+    n_dec = dec_tokens.shape[0] if dec_tokens is not None else T
     if n_dec == 0:
         return out
     nbytes = lib.qe_attention_decode_workspace_bytes(n_dec, Hq, D, int(max_dec_position), DECODE_SPLIT_KEYS)
     ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
-    _check(lib.qe_attention_decode_fused_run(qkv.data_ptr(), out.data_ptr(), cache.data_ptr(), dec_tokens.data_ptr(),
+    _check(lib.qe_attention_decode_fused_run(qkv.data_ptr(), out.data_ptr(), cache.data_ptr(), _ptr(dec_tokens),
                                              n_dec, positions.data_ptr(), tok_seq.data_ptr(), block_table.data_ptr(),
                                              block_table.shape[1], _ptr(slots), _ptr(q_weight), _ptr(k_weight),
                                              float(eps), _ptr(table), Hq, Hkv, D, P, float(scale), int(window),

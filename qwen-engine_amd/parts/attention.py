@@ -108,7 +108,7 @@ class PagedAttention:
                 # every row is the one new token of its request: norm, rotation and cache write
                 # happen inside the attention kernel
                 o = ops.attention_decode_fused(qkv, self.hq, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g],
-                                               self.scale, self.window, ctx.dec_tokens, ctx.max_dec_position,
+                                               self.scale, self.window, None, ctx.max_dec_position,
                                                self.q_norm, self.k_norm, eps, table, slots)
                 return self._project_out(o.view(T, self.hq * self.d))
             q = ops.qk_rope_store(qkv, self.hq, self.hkv, self.d, ctx.positions, self.q_norm, self.k_norm,

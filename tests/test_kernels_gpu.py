@@ -534,6 +534,10 @@ def test_decode_attention_with_norm_rotation_and_cache_write_inside(ops, hq, hkv
                          dec_tokens=i32([b for b in range(B) if slots[b] >= 0]), max_dec_position=max(positions))
     rows = [b for b in range(B) if slots[b] >= 0]
     close(out[rows], out2[rows].float().cpu(), bf)
+    # without a list of rows every row is taken, in order: the same results to the bit
+    out3 = ops.attention_decode_fused(qkv.to(DEV), hq, cache.to(DEV), i32(positions), i32(list(range(B))), tab.to(DEV),
+                                      scale, window, None, max(positions), dev(qw), dev(kw), eps, dev(table), i32(slots))
+    assert torch.equal(out3, out)
 
 
 @pytest.mark.parametrize("key_pos", [0, 15, 16, 127, 128, 255, 256, 1000, 1023])
