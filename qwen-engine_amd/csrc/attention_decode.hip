@@ -168,7 +168,13 @@ struct NormRotate {
     }
 };
 
-template <int D, int SPLIT>
+// AHEAD: how many tiles the loads of a whole split run ahead of the computation.  A wave with one
+// tile in flight gets 8 KB per trip to memory (about 0.7 us); that is enough when the chip holds
+// two waves or more per SIMD, whose loads together keep the memory busy, and far too little for one
+// token's 256 waves.  With 3 the code of a whole split is straight-line (waits are then exact) and
+// takes 64 registers more, which with many waves costs more than it brings.  The order of the
+// arithmetic is the same either way.
+template <int D, int SPLIT, int AHEAD>
 __global__ __launch_bounds__(64) void attention_decode_fused_split_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* cache,
     const int* __restrict__ dec_tokens, const int* __restrict__ positions, const int* __restrict__ tok_seq,
@@ -176,6 +182,7 @@ __global__ __launch_bounds__(64) void attention_decode_fused_split_kernel(
     const float* __restrict__ q_w, const float* __restrict__ k_w, float eps, const float* __restrict__ table,
     float* __restrict__ part_acc, float* __restrict__ part_ml,
     int Hq, int Hkv, int P, float scale, int window, int num_splits) {
+    constexpr int TILES = SPLIT / 16;
     const int lane = threadIdx.x, g = lane >> 4, n = lane & 15;
     const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
     const int G = Hq / Hkv;
@@ -209,20 +216,34 @@ __global__ __launch_bounds__(64) void attention_decode_fused_split_kernel(
 #define LOAD(buf_, i_) load_tile<D>(buf_, cache, __builtin_amdgcn_readlane(my_page, (i_)), page_stride, kvh, Hkv, P, \
                                     (split * SPLIT + (i_) * 16) % P, g, n)
 #define STEP(buf_, i_) attn_tile_step<D>(st, buf_, qreg, scale, split * SPLIT + (i_) * 16, g, k_begin, k_end, k_begin, k_end)
-        KVTile<D> ta, tb;
-        int i = tile0;
         NormRotate<D> nq;
         nq.fetch(qkv + t * width + (long)head * D, head_ok, q_w, cs, g);
-        LOAD(ta, i);                                       // the first tiles travel while q is prepared
-        if (i + 1 < tile1) LOAD(tb, i + 1);
-        nq.finish(qreg, q_w != nullptr, eps, cs != nullptr);
-        while (true) {
-            STEP(ta, i);
-            if (++i >= tile1) break;
-            if (i + 1 < tile1) LOAD(ta, i + 1);
-            STEP(tb, i);
-            if (++i >= tile1) break;
+        if (AHEAD > 1 && tile0 == 0 && tile1 == TILES) {
+            KVTile<D> tl[AHEAD + 1];
+#pragma unroll
+            for (int j = 0; j < AHEAD; ++j) LOAD(tl[j], j);   // the first tiles travel while q is prepared
+            nq.finish(qreg, q_w != nullptr, eps, cs != nullptr);
+#pragma unroll
+            for (int j = 0; j < TILES; ++j) {
+                if (j + AHEAD < TILES) LOAD(tl[(j + AHEAD) % (AHEAD + 1)], j + AHEAD);
+                __builtin_amdgcn_sched_barrier(0);         // (the scheduler would move the loads down to their uses)
+                STEP(tl[j % (AHEAD + 1)], j);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            KVTile<D> ta, tb;
+            int i = tile0;
+            LOAD(ta, i);                                   // the first tiles travel while q is prepared
             if (i + 1 < tile1) LOAD(tb, i + 1);
+            nq.finish(qreg, q_w != nullptr, eps, cs != nullptr);
+            while (true) {
+                STEP(ta, i);
+                if (++i >= tile1) break;
+                if (i + 1 < tile1) LOAD(ta, i + 1);
+                STEP(tb, i);
+                if (++i >= tile1) break;
+                if (i + 1 < tile1) LOAD(tb, i + 1);
+            }
         }
 #undef LOAD
 #undef STEP
@@ -423,9 +444,15 @@ int qe_attention_decode_fused(const void* qkv, void* out, void* cache, const int
     float* part_ml = part_acc + (size_t)n_dec * Hq * num_splits * D;
     dim3 grid(num_splits, Hkv, n_dec);
     dim3 mgrid(n_dec, Hq);
+    const bool few = (long)num_splits * Hkv * n_dec <= 1024;   // at most a wave per SIMD: loads further ahead
 #define QE_DECODE_FUSED(D_, S_)                                                                         \
     do {                                                                                                \
-        attention_decode_fused_split_kernel<D_, S_><<<grid, 64, 0, stream>>>(                           \
+        if (few)                                                                                        \
+            attention_decode_fused_split_kernel<D_, S_, 3><<<grid, 64, 0, stream>>>(                    \
+                (const bf16_t*)qkv, (bf16_t*)cache, dec_tokens, positions, tok_seq, block_table, max_blocks, \
+                slots, q_w, k_w, eps, table, part_acc, part_ml, Hq, Hkv, P, scale, window, num_splits); \
+        else                                                                                            \
+        attention_decode_fused_split_kernel<D_, S_, 1><<<grid, 64, 0, stream>>>(                        \
             (const bf16_t*)qkv, (bf16_t*)cache, dec_tokens, positions, tok_seq, block_table, max_blocks, \
             slots, q_w, k_w, eps, table, part_acc, part_ml, Hq, Hkv, P, scale, window, num_splits);     \
         attention_decode_merge_kernel<D_><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, dec_tokens,     \
