@@ -115,6 +115,10 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks)
         qreg[ks] = *(const bf16x8*)(q + ((long)row * Hq + head) * D + ks * 16 + g * 8);
+    // Wait for q here, with an instruction the compiler sees: else it waits for these loads where q
+    // is first used, inside the loop, where its count of loads in flight includes the loop's own,
+    // and every round would end up waiting for the loads it has just issued.
+    __builtin_amdgcn_s_waitcnt(0x0f70);                    // vmcnt(0)
 
     float m = -INFINITY, l = 0.f;
     floatx16 acc[D / 32];
@@ -208,7 +212,12 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
         STAGE_LOAD(0, kk_first)
         STAGE_STORE(0, 0, kk_first)
     }
-    if (kk_second < kmax) STAGE_LOAD(1, kk_second)
+    // (From here on the loads are issued whether their tile exists or not, one that does not
+    // exist reads the first tile again and is never stored: with loads under a condition the
+    // compiler cannot count how many are in flight and waits for all of them before every store
+    // to shared memory, the ones just issued included.)
+#define EXISTING(kk_) ((kk_) < kmax ? (kk_) : kk0)
+    STAGE_LOAD(1, EXISTING(kk_second))
     __syncthreads();
     for (int i2 = 0; i2 < rounds; i2 += 2) {
 #pragma unroll
@@ -217,7 +226,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
         if (i >= rounds) break;                           // the same for all threads of the block
         const int kk = TILE_KEY(i);
         const int kk_1 = TILE_KEY(i + 1), kk_2 = TILE_KEY(i + 2);   // (values, not expressions in i: the macros have loops over i)
-        if (kk_2 < kmax) STAGE_LOAD(buf, kk_2)            // this set's tile went to shared memory a round ago
+        STAGE_LOAD(buf, EXISTING(kk_2))                   // this set's tile went to shared memory a round ago
         __builtin_amdgcn_sched_barrier(0);                // keep the loads ahead of the computation
         if (wave_on && kk < k_stop && kk + 32 > k_start) { // some row of the wave sees some key of the tile (none beyond kmax)
             const unsigned char* ks_ = smem + buf * BUF + r * KROW + g * 16;
@@ -291,6 +300,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
       }
     }
 #undef STAGE_LOAD
+#undef EXISTING
 #undef STAGE_STORE
 #undef TILE_KEY
     l = sum_of_both_halves(l);
