@@ -378,13 +378,22 @@ static int launch_mfma(const void* x, const void* w, const float* bias, void* ou
 template <typename TO, bool SILU>
 static int pick_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                      int tile, int splits, hipStream_t stream) {
-    const long cus = 256;
-    const long big = (long)qe_cdiv(M, 256) * qe_cdiv(N, 128) * splits, mid = (long)qe_cdiv(M, 128) * qe_cdiv(N, 128) * splits;
-    const long huge = (long)qe_cdiv(M, 256) * qe_cdiv(N, 256) * splits;
-    // the largest tile that still gives every compute unit two blocks (one, for the middle size)
-    if (tile == 0)
-        tile = (huge >= 2 * cus && M > 128) ? 512
-             : ((big >= 2 * cus && M > 128) ? 256 : ((mid >= cus && M > 64) ? 128 : 64));   // never taller than the rows need
+    // The shape is chosen by what the busiest compute unit gets: its number of tiles (they are dealt
+    // out in turn) times a tile's area, over how well the shape uses the unit (measured on large
+    // products: 256 x 256 reaches 1.05, 256 x 128 0.92, 128 x 128 0.85, 64 x 128 0.74 PFLOP/s).
+    // A shape is never taller than the rows need.
+    if (tile == 0) {
+        const long cus = 256;
+        struct Shape { int tile, bm, bn; float rate; };
+        const Shape shapes[4] = {{64, 64, 128, 0.74f}, {128, 128, 128, 0.85f}, {256, 256, 128, 0.92f}, {512, 256, 256, 1.05f}};
+        float best = 0.f;
+        for (const Shape& sh : shapes) {
+            if (sh.tile != 64 && M <= sh.bm / 2) continue;
+            const long blocks = (long)qe_cdiv(M, sh.bm) * qe_cdiv(N, sh.bn) * splits;
+            const float cost = (float)qe_cdiv(blocks, cus) * sh.bm * sh.bn / sh.rate;
+            if (tile == 0 || cost < best) { tile = sh.tile; best = cost; }
+        }
+    }
     if (tile == 512) return launch_mfma<TO, 256, 256, 64, 4, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 256) return launch_mfma<TO, 256, 128, 64, 8, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 128) return launch_mfma<TO, 128, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, splits, stream);
