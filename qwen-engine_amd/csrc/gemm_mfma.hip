@@ -36,7 +36,7 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
 template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU>
 __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n, int k_per_split) {
+    TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n, int k_per_split, int xcd_m, int xcd_n) {
     constexpr int ROWB = BK * 2 + 16;       // bytes of a staged row
     constexpr int PPR = BK / 8;             // 16-byte pieces per row
     constexpr int RPI = 64 * NW / PPR;      // rows the block stages with one piece per thread
@@ -51,21 +51,18 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // Consecutive blocks go to the eight XCDs in turn, and each XCD has an L2 of its own: the blocks
-    // of one XCD take a compact part of the tiles (an eighth of the tile columns, or of the tile
-    // rows), so that they share the rows of W and of x that they read through that L2.
+    // of one XCD take a compact part of the tiles, xcd_m parts down by xcd_n across (the host picks
+    // the cut that makes the XCDs read the fewest rows of x and W altogether; 0: no cut fits), so
+    // that they share what they read through that L2.
     int tile_m, tile_n;
-    {
+    if (xcd_m > 0) {
         const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
-        if (tiles_n % 8 == 0) {
-            tile_m = local % tiles_m;
-            tile_n = xcd * (tiles_n / 8) + local / tiles_m;
-        } else if (tiles_m % 8 == 0) {
-            tile_n = local % tiles_n;
-            tile_m = xcd * (tiles_m / 8) + local / tiles_n;
-        } else {
-            tile_m = blockIdx.x % tiles_m;
-            tile_n = blockIdx.x / tiles_m;
-        }
+        const int per_m = tiles_m / xcd_m, per_n = tiles_n / xcd_n;
+        tile_m = (xcd / xcd_n) * per_m + local % per_m;
+        tile_n = (xcd % xcd_n) * per_n + local / per_m;
+    } else {
+        tile_m = blockIdx.x % tiles_m;
+        tile_n = blockIdx.x / tiles_m;
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
@@ -369,8 +366,18 @@ static int launch_mfma(const void* x, const void* w, const float* bias, void* ou
     const int k_per_split = splits > 1 ? qe_cdiv(qe_cdiv(K, splits), BK) * BK : K;
     QE_REQUIRE(splits >= 1 && splits <= 65535 && (long)(splits - 1) * k_per_split < K,
                "mfma gemm: K=%d cannot be cut into %d parts", K, splits);
+    // the eight XCDs as a by b parts of the tiles (a b = 8): every XCD reads M / a rows of x and
+    // N / b rows of W, so all of them together b M + a N rows
+    int xcd_m = 0, xcd_n = 0;
+    long fewest = 0;
+    for (int a = 1; a <= 8; a *= 2) {
+        const int b = 8 / a;
+        if (tiles_m % a || tiles_n % b) continue;
+        const long rows = (long)b * M + (long)a * N;
+        if (xcd_m == 0 || rows < fewest) { xcd_m = a; xcd_n = b; fewest = rows; }
+    }
     gemm_mfma_kernel<TO, BM, BN, BK, NW, MINB, SILU><<<dim3((unsigned)blocks, (unsigned)splits), 64 * NW, shmem, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n, k_per_split);
+        (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n, k_per_split, xcd_m, xcd_n);
     QE_LAUNCH_CHECK();
     return 0;
 }
