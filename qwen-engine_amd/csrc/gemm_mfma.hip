@@ -58,8 +58,14 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     if (xcd_m > 0) {
         const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
         const int per_m = tiles_m / xcd_m, per_n = tiles_n / xcd_n;
-        tile_m = (xcd / xcd_n) * per_m + local % per_m;
-        tile_n = (xcd % xcd_n) * per_n + local / per_m;
+        // Inside the part the tiles go in bands of up to 8 tile rows, across the band column by
+        // column: the 32 or 64 blocks that an XCD runs at a time are then a patch of 8 by 4 or 8
+        // tiles, which reads 12 or 16 tiles' worth of rows where a column of 32 reads 33 (what
+        // the XCDs fetch through the fabric is what bounds a large product).
+        const int gm = per_m % 8 == 0 ? 8 : (per_m % 4 == 0 ? 4 : (per_m % 2 == 0 ? 2 : 1));
+        const int band = local / (gm * per_n), within = local % (gm * per_n);
+        tile_m = (xcd / xcd_n) * per_m + band * gm + within % gm;
+        tile_n = (xcd % xcd_n) * per_n + within / gm;
     } else {
         tile_m = blockIdx.x % tiles_m;
         tile_n = blockIdx.x / tiles_m;
