@@ -393,12 +393,12 @@ static int pick_mfma(const void* x, const void* w, const float* bias, void* out,
                      int tile, int splits, hipStream_t stream) {
     // The shape is chosen by what the busiest compute unit gets: its number of tiles (they are dealt
     // out in turn) times a tile's area, over how well the shape uses the unit (measured on large
-    // products: 256 x 256 reaches 1.05, 256 x 128 0.92, 128 x 128 0.85, 64 x 128 0.74 PFLOP/s).
+    // products: 256 x 256 reaches 1.13, 256 x 128 1.02, 128 x 128 0.96, 64 x 128 0.74 PFLOP/s).
     // A shape is never taller than the rows need.
     if (tile == 0) {
         const long cus = 256;
         struct Shape { int tile, bm, bn; float rate; };
-        const Shape shapes[4] = {{64, 64, 128, 0.74f}, {128, 128, 128, 0.85f}, {256, 256, 128, 0.92f}, {512, 256, 256, 1.05f}};
+        const Shape shapes[4] = {{64, 64, 128, 0.74f}, {128, 128, 128, 0.96f}, {256, 256, 128, 1.02f}, {512, 256, 256, 1.13f}};
         float best = 0.f;
         for (const Shape& sh : shapes) {
             if (sh.tile != 64 && M <= sh.bm / 2) continue;
