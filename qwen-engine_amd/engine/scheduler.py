@@ -126,26 +126,37 @@ class Scheduler:
     def plan(self) -> List[Planned]:
         """Decide the next step: decoded tokens of every running request that is ready, then
         portions of prompts, oldest first, within the token budget."""
+        groups = range(len(self.cache.groups))
         while True:
             planned: List[Planned] = []
-            wants: List[Tuple[Hashable, int]] = []
             budget = self.max_step_tokens
             blocked: Optional[Request] = None
+            # pages the entries planned so far need, per group: an entry fits if its own pages fit
+            # beside them (the same answer as cache.can_reserve on the whole list, without going
+            # through the list again for every candidate)
+            taken = [0 for _ in groups]
+
+            def fits(req_id, new_len) -> bool:
+                need = self.cache.pages_needed(req_id, new_len)
+                if any(taken[g] + need[g] > self.cache.available(g) for g in groups):
+                    return False
+                for g in groups:
+                    taken[g] += need[g]
+                return True
+
             for r in sorted(self.running, key=lambda r: r.admit_order):
                 remaining = r.num_known - r.num_computed
                 if remaining <= 0 or budget <= 0:
                     continue
                 n = 1 if remaining == 1 else min(remaining, self.prefill_chunk, budget)
-                want = (r.req_id, r.num_computed + n)
-                if not self.cache.can_reserve(wants + [want]):
-                    # fewer tokens may still fit (down to one)
-                    while n > 1 and not self.cache.can_reserve(wants + [(r.req_id, r.num_computed + n)]):
-                        n = n // 2
-                    want = (r.req_id, r.num_computed + n)
-                    if not self.cache.can_reserve(wants + [want]):
-                        blocked = blocked or r
-                        continue
-                wants.append(want)
+                while not fits(r.req_id, r.num_computed + n):
+                    if n == 1:
+                        n = 0
+                        break
+                    n = n // 2                                 # fewer tokens may still fit (down to one)
+                if n == 0:
+                    blocked = blocked or r
+                    continue
                 toks = r.known[r.num_computed:r.num_computed + n]
                 planned.append(Planned(r, toks, sample=(r.num_computed + n == r.num_known)))
                 budget -= n
@@ -170,8 +181,7 @@ class Scheduler:
                 start = self.cache.match_prefix(r.req_id, r.known)
                 remaining = r.num_known - start
                 n = min(remaining, self.prefill_chunk, budget)
-                want = (r.req_id, start + n)
-                if not self.cache.can_reserve(wants + [want]):
+                if not fits(r.req_id, start + n):
                     self.cache.free_request(r.req_id)
                     break
                 self.waiting.popleft()
@@ -181,7 +191,6 @@ class Scheduler:
                 self._admitted += 1
                 self.running.append(r)
                 self.stats["shared_prefix_tokens"] += start
-                wants.append(want)
                 planned.append(Planned(r, r.known[start:start + n], sample=(start + n == r.num_known)))
                 budget -= n
             if not planned and self.waiting and not self.running:
