@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16] [--layers L]
 
-The default run has the layer sizes of Qwen3-0.6B (BASELINE.json configs[2]) with
+The default run has the layer sizes of Qwen3-0.6B with
 random weights, a batch of 8 requests and a context of 4096 tokens: every request is
 first prefilled with random tokens through the engine's own step function, so that
 the K timed decode steps end at that context.  A "step" is one decode step (one new
@@ -17,7 +17,7 @@ line is printed:
 
 Other sizes and workloads (not what the default line reports):
 
-  --model 8b|32b            the layer sizes of Qwen3-8B / Qwen3-32B (BASELINE.json configs[3], [4]); with
+  --model 8b|32b            the layer sizes of Qwen3-8B / Qwen3-32B; with
                             --layers L fewer layers than the model has (the line names both numbers)
   --workload serving        N requests (--requests, default 64) with prompt lengths uniform in [128, 2048]
                             and 256 new tokens each through the scheduler: continuous batching, prompt

@@ -30,7 +30,7 @@ def prompts_for(cfg, lengths, seed):
 
 
 def test_greedy_generation_equals_the_plain_implementation(folders):
-    """BASELINE workload of the first tiny configuration: prompts of 5, 9 and 13 tokens, 8 greedy tokens."""
+    """The first tiny configuration's workload: prompts of 5, 9 and 13 tokens, 8 greedy tokens."""
     cfg, w = P.read_folder(folders["A"])
     prompts = prompts_for(cfg, (5, 9, 13), 1)
     want = [P.greedy_generate(cfg, w, p, 8) for p in prompts]
