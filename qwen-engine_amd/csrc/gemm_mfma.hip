@@ -30,9 +30,8 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
 // ...), N counts all of them, and the result is silu(gate) * up, N / 2 wide: the two MFMA tiles a
 // lane holds side by side are the gate and the up of the same outputs.
 // BIG (256 x 256 by four waves, one wave a SIMD, a wave's part 128 x 128): the accumulators fill the
-// 256 AGPRs, so there is one set of staging registers, in VGPRs, loaded one step ahead (a step is
-// 2048 cycles of MFMAs, longer than a trip to the L2).  Per MFMA this shape reads half the bytes
-// from the L1 and from shared memory that 128 x 128 by four waves reads.
+// 256 AGPRs, so the staging registers are VGPRs.  Per MFMA this shape reads half the bytes from
+// the L1 and from shared memory that 128 x 128 by four waves reads.
 template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU>
 __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
@@ -44,7 +43,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     constexpr int MI = WM / 32, NJ = WN / 32;
     constexpr int LDA = BM / RPI, LD = (BM + BN) / RPI;   // pieces a thread stages per step: LDA of x, then of W
     constexpr bool BIG = BM == 256 && BN == 256 && NW == 4;
-    constexpr int SETS = BIG ? 1 : 2;
+    constexpr int SETS = 2;
     static_assert((LD == 16 || LD == 12 || LD == 8 || LD == 6) && (LD == 16) == BIG && BM % RPI == 0 && BN % RPI == 0,
                   "tile rows must be a multiple of the rows staged at once");
     constexpr int BUF = (BM + BN) * ROWB;   // bytes of one buffer: the x rows, then the W rows
@@ -213,18 +212,22 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
         __syncthreads();                                                                 \
     }
     // The step of the BIG shape.  A wave is alone on its SIMD and issues in order, so whatever is
-    // not an MFMA is put between the MFMAs, one a time: the 16 loads of the next step among the 16
-    // MFMAs of the first k step, the 16 stores to shared memory among those of the last.
-#define LOAD_PIECE(kt_, i_)                                                              \
+    // not an MFMA is put between the MFMAs, one a time: the 16 loads of the next step after every
+    // third MFMA of the first three k steps (the compute unit's L1 takes 64 bytes a cycle, the four
+    // waves' 64 KB a step half of the step's time: issued in a row they hold up the MFMAs behind
+    // them, which cost a third of the step), the 16 stores to shared memory of what was loaded a step
+    // ago after every third MFMA of the
+    // last three k steps (the four waves' 64 KB a step are half a step of the LDS's time too).
+#define LOAD_PIECE(set_, kt_, i_)                                                        \
     {                                                                                    \
         const int vo = (kt_) * BK + pc * 8 < klen ? voff[i_] : 0x7fffffff;               \
         const int soff = (kt_) * BK * 2;                                                 \
         if ((i_) < LDA)                                                                  \
             asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                      \
-                         : "=&v"(stage[0][i_]) : "v"(vo), "s"(rsrc_a), "s"(soff) : "memory"); \
+                         : "=&v"(stage[set_][i_]) : "v"(vo), "s"(rsrc_a), "s"(soff) : "memory"); \
         else                                                                             \
             asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                      \
-                         : "=&v"(stage[0][i_]) : "v"(vo), "s"(rsrc_b), "s"(soff) : "memory"); \
+                         : "=&v"(stage[set_][i_]) : "v"(vo), "s"(rsrc_b), "s"(soff) : "memory"); \
     }
 #define K_STEP_BIG(buf_, kt_)                                                            \
     {                                                                                    \
@@ -232,14 +235,16 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
         READ_FRAGS(buf_, 0, fa[0], fb[0])                                                \
         _Pragma("unroll") for (int ks = 0; ks < BK / 16; ++ks) {                         \
             if (ks + 1 < BK / 16) { READ_FRAGS(buf_, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]) } \
-            if (ks == BK / 16 - 1) { WAIT_LOADS(0, 0) }                                  \
+            if (ks == 1) { WAIT_LOADS((buf_) ^ 1, (MI * NJ + BK / 16 - 2) / (BK / 16 - 1)) }   /* this step's own loads, those of k step 0, may stay in flight */ \
             __builtin_amdgcn_sched_barrier(0);                                           \
             _Pragma("unroll") for (int i = 0; i < MI; ++i)                               \
                 _Pragma("unroll") for (int j = 0; j < NJ; ++j) {                         \
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks & 1][j], fa[ks & 1][i], acc[i][j], 0, 0, 0); \
-                    if (ks == 0) LOAD_PIECE((kt_) + 1, (i * NJ + j) % LD)                \
-                    if (ks == BK / 16 - 1)                                               \
-                        *(uint4_t*)(smem + ((buf_) ^ 1) * BUF + dst + ((i * NJ + j) % LD) * RPI * ROWB) = stage[0][(i * NJ + j) % LD]; \
+                    if (ks < BK / 16 - 1 && (ks * MI * NJ + i * NJ + j) % (BK / 16 - 1) == 0) \
+                        LOAD_PIECE(buf_, (kt_) + 2, ((ks * MI * NJ + i * NJ + j) / (BK / 16 - 1)) % LD) \
+                    if (ks > 0 && ((ks - 1) * MI * NJ + i * NJ + j) % (BK / 16 - 1) == 0) \
+                        *(uint4_t*)(smem + ((buf_) ^ 1) * BUF + dst + ((((ks - 1) * MI * NJ + i * NJ + j) / (BK / 16 - 1)) % LD) * RPI * ROWB) = \
+                            stage[(buf_) ^ 1][(((ks - 1) * MI * NJ + i * NJ + j) / (BK / 16 - 1)) % LD]; \
                     __builtin_amdgcn_sched_barrier(0);                                   \
                 }                                                                        \
         }                                                                                \
