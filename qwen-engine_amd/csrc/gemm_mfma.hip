@@ -43,7 +43,6 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     constexpr int MI = WM / 32, NJ = WN / 32;
     constexpr int LDA = BM / RPI, LD = (BM + BN) / RPI;   // pieces a thread stages per step: LDA of x, then of W
     constexpr bool BIG = BM == 256 && BN == 256 && NW == 4;
-    constexpr int SETS = 2;
     static_assert((LD == 16 || LD == 12 || LD == 8 || LD == 6) && (LD == 16) == BIG && BM % RPI == 0 && BN % RPI == 0,
                   "tile rows must be a multiple of the rows staged at once");
     constexpr int BUF = (BM + BN) * ROWB;   // bytes of one buffer: the x rows, then the W rows
@@ -79,7 +78,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const int nk = (klen + BK - 1) / BK;
     // Two sets of staging registers in turn: a step's loads are issued two steps ahead and go to
     // shared memory one step ahead, so a load has a whole step of MFMAs to arrive.
-    uint4_t stage[SETS][LD];
+    uint4_t stage[2][LD];
 
     // Piece i of a thread is row (tid / PPR) of the i-th group of RPI rows, 16 bytes at k = 8 (tid % PPR).
     // The loads are buffer loads: one descriptor for the tile's rows of x and one for its rows of W,
@@ -160,7 +159,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
                      : "n"(younger_) : "memory");
 #define STORE_SHARED(buf_)                                                               \
     _Pragma("unroll") for (int i = 0; i < LD; ++i)                                       \
-        *(uint4_t*)(smem + (buf_) * BUF + dst + i * RPI * ROWB) = stage[(buf_) % SETS][i];
+        *(uint4_t*)(smem + (buf_) * BUF + dst + i * RPI * ROWB) = stage[buf_][i];
 
     floatx16 acc[MI][NJ];
 #pragma unroll
@@ -175,76 +174,70 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const unsigned char* a_frag = smem + (wm + fr) * ROWB + fk;
     const unsigned char* b_frag = smem + (BM + wn + fr) * ROWB + fk;
     // One step on buffer buf_ (a constant, so every shared-memory address is base + immediate).
-    // The fragments of k step ks + 1 are read while the MFMAs of ks run, and the stores of the
-    // next step's tile are issued before the last MFMAs, whose time then covers them.
-    // (Passing the barrier before those last MFMAs and reading the next step's first fragments
+    // A wave issues in order, so whatever is not an MFMA stands between the MFMAs: the fragments of
+    // k step ks + 1 are read before the MFMAs of ks; the loads of the step after the next go with
+    // the MFMAs of the first k steps, the stores to shared memory of the next step's tile, loaded
+    // a step ago, with those of the last.  Tiles of 128 rows or more spread the loads over all k
+    // steps but the last and the stores over all but the first (the compute unit's L1 takes 64
+    // bytes a cycle: the 64 KB a step of a 256 x 256 tile are half of the step's time, and as
+    // much for the LDS; issued in a row they hold up the MFMAs behind them, which cost that
+    // shape a third of the step).  The 64-row tile, whose steps are short, keeps the loads in
+    // the first k step and the stores in the last: a load then has the longest time to arrive
+    // (spread, its loads from HBM came late: 27 us against 24 for the o and down products of the
+    // small model, though it was the faster on operands that lie in the L2).
+    // (Passing the barrier before the last MFMAs and reading the next step's first fragments
     // under them was tried: 3 % faster with one wave a SIMD, 10 % slower with two.)
 #define READ_FRAGS(buf_, ks_, a_, b_)                                                    \
     _Pragma("unroll") for (int i = 0; i < MI; ++i)                                       \
         a_[i] = *(const bf16x8*)(a_frag + (buf_) * BUF + i * 32 * ROWB + (ks_) * 32);    \
     _Pragma("unroll") for (int j = 0; j < NJ; ++j)                                       \
         b_[j] = *(const bf16x8*)(b_frag + (buf_) * BUF + j * 32 * ROWB + (ks_) * 32);
-#define MFMAS(a_, b_)                                                                    \
-    _Pragma("unroll") for (int i = 0; i < MI; ++i)                                       \
-        _Pragma("unroll") for (int j = 0; j < NJ; ++j)                                   \
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_[j], a_[i], acc[i][j], 0, 0, 0);
-#define K_STEP(buf_, kt_)                                                                \
-    {                                                                                    \
-        bf16x8 fa[2][MI], fb[2][NJ];                                                     \
-        READ_FRAGS(buf_, 0, fa[0], fb[0])                                                \
-        if constexpr (SETS == 2) LOAD_GLOBAL(buf_, (kt_) + 2)   /* this set went to shared memory a step ago */ \
-        else LOAD_GLOBAL(0, (kt_) + 1)                                                   \
-        __builtin_amdgcn_sched_barrier(0);                                               \
-        _Pragma("unroll") for (int ks = 0; ks < BK / 16 - 1; ++ks) {                     \
-            READ_FRAGS(buf_, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1])                 \
-            __builtin_amdgcn_sched_barrier(0);   /* keep the reads ahead of the MFMAs */ \
-            MFMAS(fa[ks & 1], fb[ks & 1])                                                \
-            __builtin_amdgcn_sched_barrier(0);                                           \
-        }                                                                                \
-        /* the other buffer: its readers finished before the last barrier (after the last step  \
-           this stores a step that does not exist, which nobody reads) */                    \
-        if constexpr (SETS == 2) { WAIT_LOADS((buf_) ^ 1, LD) }   /* the LD loads just issued may stay in flight */ \
-        else { WAIT_LOADS(0, 0) }                                                        \
-        STORE_SHARED((buf_) ^ 1)                                                         \
-        __builtin_amdgcn_sched_barrier(0);                                               \
-        MFMAS(fa[(BK / 16 - 1) & 1], fb[(BK / 16 - 1) & 1])                              \
-        __builtin_amdgcn_sched_barrier(0);                                               \
-        __syncthreads();                                                                 \
-    }
-    // The step of the BIG shape.  A wave is alone on its SIMD and issues in order, so whatever is
-    // not an MFMA is put between the MFMAs, one a time: the 16 loads of the next step after every
-    // third MFMA of the first three k steps (the compute unit's L1 takes 64 bytes a cycle, the four
-    // waves' 64 KB a step half of the step's time: issued in a row they hold up the MFMAs behind
-    // them, which cost a third of the step), the 16 stores to shared memory of what was loaded a step
-    // ago after every third MFMA of the
-    // last three k steps (the four waves' 64 KB a step are half a step of the LDS's time too).
 #define LOAD_PIECE(set_, kt_, i_)                                                        \
     {                                                                                    \
         const int vo = (kt_) * BK + pc * 8 < klen ? voff[i_] : 0x7fffffff;               \
         const int soff = (kt_) * BK * 2;                                                 \
-        if ((i_) < LDA)                                                                  \
+        if constexpr (BIG) {                                                             \
+            if ((i_) < LDA)                                                              \
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                  \
+                             : "=&v"(stage[set_][i_]) : "v"(vo), "s"(rsrc_a), "s"(soff) : "memory"); \
+            else                                                                         \
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                  \
+                             : "=&v"(stage[set_][i_]) : "v"(vo), "s"(rsrc_b), "s"(soff) : "memory"); \
+        } else if ((i_) < LDA)                                                           \
             asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                      \
-                         : "=&v"(stage[set_][i_]) : "v"(vo), "s"(rsrc_a), "s"(soff) : "memory"); \
+                         : "=&a"(stage[set_][i_]) : "v"(vo), "s"(rsrc_a), "s"(soff) : "memory"); \
         else                                                                             \
             asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                      \
-                         : "=&v"(stage[set_][i_]) : "v"(vo), "s"(rsrc_b), "s"(soff) : "memory"); \
+                         : "=&a"(stage[set_][i_]) : "v"(vo), "s"(rsrc_b), "s"(soff) : "memory"); \
     }
-#define K_STEP_BIG(buf_, kt_)                                                            \
+    constexpr int NS = BK / 16, PER = MI * NJ;            // k steps; MFMAs of one
+    constexpr bool SPREAD = BM >= 128;
+    constexpr int LE = SPREAD ? NS - 1 : 1, SB = SPREAD ? 1 : NS - 1;   // loads go with the k steps [0, LE), stores with [SB, NS)
+    constexpr int LSLOTS = LE * PER, SSLOTS = (NS - SB) * PER;    // places (MFMAs) for a load, for a store
+    constexpr int EARLY = SB * PER * LD / LSLOTS < LD ? SB * PER * LD / LSLOTS : LD;   // this step's loads issued before k step SB
+    static_assert(NS >= 2, "a step has two k steps or more");
+    // the pieces that go with place s of n: [s LD / n, (s + 1) LD / n)
+#define K_STEP(buf_, kt_)                                                                \
     {                                                                                    \
         bf16x8 fa[2][MI], fb[2][NJ];                                                     \
         READ_FRAGS(buf_, 0, fa[0], fb[0])                                                \
-        _Pragma("unroll") for (int ks = 0; ks < BK / 16; ++ks) {                         \
-            if (ks + 1 < BK / 16) { READ_FRAGS(buf_, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]) } \
-            if (ks == 1) { WAIT_LOADS((buf_) ^ 1, (MI * NJ + BK / 16 - 2) / (BK / 16 - 1)) }   /* this step's own loads, those of k step 0, may stay in flight */ \
+        _Pragma("unroll") for (int ks = 0; ks < NS; ++ks) {                              \
+            if (ks + 1 < NS) { READ_FRAGS(buf_, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]) } \
+            /* the other set, loaded a step ago; this step's own loads, issued so far, may stay in flight */ \
+            if (ks == SB) { WAIT_LOADS((buf_) ^ 1, EARLY) }                              \
             __builtin_amdgcn_sched_barrier(0);                                           \
             _Pragma("unroll") for (int i = 0; i < MI; ++i)                               \
                 _Pragma("unroll") for (int j = 0; j < NJ; ++j) {                         \
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks & 1][j], fa[ks & 1][i], acc[i][j], 0, 0, 0); \
-                    if (ks < BK / 16 - 1 && (ks * MI * NJ + i * NJ + j) % (BK / 16 - 1) == 0) \
-                        LOAD_PIECE(buf_, (kt_) + 2, ((ks * MI * NJ + i * NJ + j) / (BK / 16 - 1)) % LD) \
-                    if (ks > 0 && ((ks - 1) * MI * NJ + i * NJ + j) % (BK / 16 - 1) == 0) \
-                        *(uint4_t*)(smem + ((buf_) ^ 1) * BUF + dst + ((((ks - 1) * MI * NJ + i * NJ + j) / (BK / 16 - 1)) % LD) * RPI * ROWB) = \
-                            stage[(buf_) ^ 1][(((ks - 1) * MI * NJ + i * NJ + j) / (BK / 16 - 1)) % LD]; \
+                    _Pragma("unroll") for (int p = 0; p < LD; ++p) {                     \
+                        const int sl = ks * PER + i * NJ + j, ss = sl - SB * PER;   /* place of a load, of a store */ \
+                        if (ks < LE && p >= sl * LD / LSLOTS && p < (sl + 1) * LD / LSLOTS) \
+                            LOAD_PIECE(buf_, (kt_) + 2, p)   /* this set went to shared memory a step ago */ \
+                        /* the other buffer: its readers finished before the last barrier (after the  \
+                           last step this stores a step that does not exist, which nobody reads) */ \
+                        if (ks >= SB && p >= ss * LD / SSLOTS && p < (ss + 1) * LD / SSLOTS) \
+                            *(uint4_t*)(smem + ((buf_) ^ 1) * BUF + dst + p * RPI * ROWB) = stage[(buf_) ^ 1][p]; \
+                    }                                                                    \
                     __builtin_amdgcn_sched_barrier(0);                                   \
                 }                                                                        \
         }                                                                                \
@@ -253,40 +246,25 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
 
     // step kt uses buffer and register set kt % 2
     LOAD_GLOBAL(0, 0)
-    if constexpr (SETS == 2) {
-        LOAD_GLOBAL(1, 1)
-        WAIT_LOADS(0, LD)
-    } else {
-        WAIT_LOADS(0, 0)
-    }
+    LOAD_GLOBAL(1, 1)
+    WAIT_LOADS(0, LD)
     STORE_SHARED(0)
     __syncthreads();
     // (two steps in a body without branches, and an odd last step after the loop)
     int kt = 0;
-    if constexpr (BIG) {
-        static_assert(!BIG || MI * NJ == LD, "one load and one store per MFMA of a k step");
-        for (; kt + 1 < nk; kt += 2) {
-            K_STEP_BIG(0, kt)
-            K_STEP_BIG(1, kt + 1)
-        }
-        if (kt < nk) K_STEP_BIG(0, kt)
-    } else {
-        for (; kt + 1 < nk; kt += 2) {
-            K_STEP(0, kt)
-            K_STEP(1, kt + 1)
-        }
-        if (kt < nk) K_STEP(0, kt)
+    for (; kt + 1 < nk; kt += 2) {
+        K_STEP(0, kt)
+        K_STEP(1, kt + 1)
     }
+    if (kt < nk) K_STEP(0, kt)
     // The loads past the end are still in flight and the compiler does not know of them: their
     // registers pass through a last wait, so that they stay reserved until the loads have landed
     // (a register whose value nobody uses would be handed out again at once).
     WAIT_LOADS(0, 0)
-    if constexpr (SETS == 2) { WAIT_LOADS(1, 0) }
+    WAIT_LOADS(1, 0)
 #undef K_STEP
-#undef K_STEP_BIG
 #undef LOAD_PIECE
 #undef READ_FRAGS
-#undef MFMAS
 #undef LOAD_GLOBAL
 #undef WAIT_LOADS
 #undef STORE_SHARED
@@ -398,12 +376,12 @@ static int pick_mfma(const void* x, const void* w, const float* bias, void* out,
                      int tile, int splits, hipStream_t stream) {
     // The shape is chosen by what the busiest compute unit gets: its number of tiles (they are dealt
     // out in turn) times a tile's area, over how well the shape uses the unit (measured on large
-    // products: 256 x 256 reaches 1.13, 256 x 128 1.02, 128 x 128 0.96, 64 x 128 0.74 PFLOP/s).
+    // products: 256 x 256 reaches 1.30, 256 x 128 1.16, 128 x 128 1.07, 64 x 128 0.80 PFLOP/s).
     // A shape is never taller than the rows need.
     if (tile == 0) {
         const long cus = 256;
         struct Shape { int tile, bm, bn; float rate; };
-        const Shape shapes[4] = {{64, 64, 128, 0.74f}, {128, 128, 128, 0.96f}, {256, 256, 128, 1.02f}, {512, 256, 256, 1.13f}};
+        const Shape shapes[4] = {{64, 64, 128, 0.80f}, {128, 128, 128, 1.07f}, {256, 256, 128, 1.16f}, {512, 256, 256, 1.30f}};
         float best = 0.f;
         for (const Shape& sh : shapes) {
             if (sh.tile != 64 && M <= sh.bm / 2) continue;
