@@ -16,6 +16,16 @@ struct bf16_t { uint16_t bits; };
 __device__ __forceinline__ float bf16_to_float(bf16_t v) {
     return __uint_as_float(((uint32_t)v.bits) << 16);
 }
+// One pair of a half-split rotation: (a, b) <- (c a - s b, s a + c b), with the roundings fixed (a
+// product, then one fused multiply-add), so that every kernel that rotates gives the same bits.
+__device__ __forceinline__ void rotate_pair(float c, float s, float& a, float& b) {
+#pragma clang fp contract(off)
+    const float x1 = a, x2 = b;
+    const float sx2 = s * x2, cx2 = c * x2;
+    a = __builtin_fmaf(c, x1, -sx2);
+    b = __builtin_fmaf(s, x1, cx2);
+}
+
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t bits16) {
     return __uint_as_float(bits16 << 16);
 }

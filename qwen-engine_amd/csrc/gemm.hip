@@ -11,6 +11,10 @@ bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w);
 int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
                  int tile, bool silu, int splits, hipStream_t stream);
 
+int qe_gemm_qkv(const void* x, const void* w, const float* bias, int M, int K, int Hq, int Hkv, int P,
+                const int* positions, const int* slots, const float* q_w, const float* k_w, float eps,
+                const float* table, void* q_out, void* cache, int tile, hipStream_t stream);
+
 enum { ALGO_AUTO = 0, ALGO_GENERIC = 1, ALGO_MFMA = 2, ALGO_TILE = 1000 };   // ALGO_TILE + rows: the tiled kernel with that tile
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3, EPI_SILU_MUL_IL = 4 };
 
@@ -84,4 +88,21 @@ extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* ou
         QE_REQUIRE(algo == ALGO_AUTO, "gemm: M=%d N=%d K=%d with these element types is not taken by an MFMA kernel", M, N, K);
     }
     return qe_gemm_generic(x, w, bias, out, M, N, K, dt_a, dt_w, dt_o, stream);
+}
+
+// 1 if qe_gemm_qkv_run takes these sizes: bfloat16 operands, heads of 128, more rows than the
+// kernel for few rows is made for (decode has the attention kernel that prepares its own inputs).
+extern "C" int qe_gemm_qkv_supported(int M, int K, int Hq, int Hkv, int D, int P, int dt_a, int dt_w) {
+    return (D == 128 && M > 64 && P >= 16 && (P & (P - 1)) == 0 &&
+            qe_gemm_mfma_ok(M, (Hq + 2 * Hkv) * D, K, dt_a, dt_w)) ? 1 : 0;
+}
+
+// The q|k|v product with per-head q/k norm, rotation and the cache write in its epilogue: q_out
+// [M, Hq, 128] bfloat16; k and v go to cache [pages, 2, Hkv, P, 128] at slots[m].  tile: 0 or the
+// tile to use (64, 128, 256; 512 for 256 x 256).
+extern "C" int qe_gemm_qkv_run(const void* x, const void* w, const float* bias, int M, int K, int Hq, int Hkv, int P,
+                               const int* positions, const int* slots, const float* q_w, const float* k_w, float eps,
+                               const float* table, void* q_out, void* cache, int tile, hipStream_t stream) {
+    if (M == 0) return 0;
+    return qe_gemm_qkv(x, w, bias, M, K, Hq, Hkv, P, positions, slots, q_w, k_w, eps, table, q_out, cache, tile, stream);
 }

@@ -25,17 +25,40 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float floatx16;
 typedef __attribute__((ext_vector_type(4))) unsigned int uint4_t;
+union Piece16 {   // 16 bytes, addressable by element
+    uint4_t q;
+    unsigned short e[8];
+};
 
 // SILU: W holds gate and up rows interleaved in blocks of 32 (gate 0..31, up 0..31, gate 32..63,
 // ...), N counts all of them, and the result is silu(gate) * up, N / 2 wide: the two MFMA tiles a
 // lane holds side by side are the gate and the up of the same outputs.
+// What the q|k|v product of an attention layer does with its result instead of storing it (QKV):
+// per-head RMSNorm of q and k (weights or null), half-split rotation from the table's row of the
+// token's position (or null), then q to q_out [M, Hq, 128], k and v into the cache at the token's
+// slot (negative: nowhere), exactly as the kernels of qk_rope_store.hip do on a stored product, in
+// the same arithmetic: the product is rounded to bfloat16 first.  Heads are 128 wide, so that a
+// tile's 128 columns are one head.
+struct QkvTail {
+    const int* positions;
+    const int* slots;
+    const float* q_w;
+    const float* k_w;
+    const float* table;
+    bf16_t* q_out;
+    bf16_t* cache;
+    float eps;
+    int Hq, Hkv, P;
+};
+
 // BIG (256 x 256 by four waves, one wave a SIMD, a wave's part 128 x 128): the accumulators fill the
 // 256 AGPRs, so the staging registers are VGPRs.  Per MFMA this shape reads half the bytes from
 // the L1 and from shared memory that 128 x 128 by four waves reads.
-template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU>
+template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU, bool QKV = false>
 __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n, int k_per_split, int xcd_m, int xcd_n) {
+    TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n, int k_per_split, int xcd_m, int xcd_n,
+    QkvTail tail) {
     constexpr int ROWB = BK * 2 + 16;       // bytes of a staged row
     constexpr int PPR = BK / 8;             // 16-byte pieces per row
     constexpr int RPI = 64 * NW / PPR;      // rows the block stages with one piece per thread
@@ -70,6 +93,15 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+    // (QKV: thread i fetches the position and the slot of the tile's row i now, for the end)
+    int my_pos = 0, my_slot = -1;
+    if constexpr (QKV) {
+        static_assert(!QKV || BM <= 64 * NW, "a thread for every row of the tile");
+        if (tid < BM && m0 + tid < M) {
+            if (tail.table) my_pos = tail.positions[m0 + tid];
+            if (tail.slots) my_slot = tail.slots[m0 + tid];
+        }
+    }
 
     // blockIdx.y cuts K: this block sums the k values [k0, k0 + klen) and writes the partial product
     // number blockIdx.y (out is then [splits][M][N]); without a cut k_per_split = K
@@ -276,6 +308,134 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     // in shared memory, a strip of 32 rows at a time (the staging buffers are free: every wave has
     // passed the loop's last barrier): it writes the strip as rows and reads it back 16 bytes a
     // lane, so that a store instruction covers whole rows of the strip.
+    if constexpr (QKV) {
+        // The whole tile goes to shared memory as bfloat16 rows (the staging buffers are free), then
+        // 16 lanes take a row of a head each, as in qk_rope_store_vec_kernel: lane j has the features
+        // 4 j .. 4 j + 3 and 64 + 4 j .. 64 + 4 j + 3, the two halves that rotate together.
+        constexpr int TROW = BN * 2 + 16;                  // bytes of a row of the tile
+        static_assert(BM * TROW <= 2 * BUF && BN % 128 == 0, "the tile must fit the staging buffers, in whole heads");
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int bq = 0; bq < 4; ++bq) {
+                    const int nl = wn + j * 32 + 8 * bq + 4 * (lane >> 5);
+                    float v[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] = acc[i][j][4 * bq + r];
+                    if (bias) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) v[r] += bias[n0 + nl + r < N ? n0 + nl + r : N - 1];
+                    }
+                    Vec4<bf16_t>::store((bf16_t*)(smem + (wm + i * 32 + (lane & 31)) * TROW) + nl, v);
+                }
+        // positions and slots of the tile's rows, once, into shared memory behind the tile
+        int* pos_sh = (int*)(smem + BM * TROW);
+        int* slot_sh = pos_sh + BM;
+        static_assert(BM * TROW + 2 * BM * 4 <= 2 * BUF, "the rows' positions and slots must fit too");
+        if (tid < BM) { pos_sh[tid] = my_pos; slot_sh[tid] = my_slot; }
+        __syncthreads();
+        const int D = 128, half = 64;
+        const int j16 = tid % 16;
+        const long page_stride = 2L * tail.Hkv * tail.P * D;
+        constexpr int GROUPS = 64 * NW / 16, ITEMS = BM * (BN / 128);
+        // (the only loads from memory in the loop are the table's rows: an item's row is fetched
+        // while the item before it is computed)
+        float c[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f};
+        {
+            const int idx = tid / 16;
+            if (tail.table && idx < ITEMS) {
+                const float* cs = tail.table + (long)pos_sh[idx % BM] * D;
+                Vec4<float>::load(cs + 4 * j16, c);
+                Vec4<float>::load(cs + half + 4 * j16, sn);
+            }
+        }
+        float wq_a[4], wq_b[4], wk_a[4], wk_b[4];
+        if (tail.q_w) {
+            Vec4<float>::load(tail.q_w + 4 * j16, wq_a);
+            Vec4<float>::load(tail.q_w + half + 4 * j16, wq_b);
+            Vec4<float>::load(tail.k_w + 4 * j16, wk_a);
+            Vec4<float>::load(tail.k_w + half + 4 * j16, wk_b);
+        }
+        for (int idx = tid / 16; idx < ITEMS; idx += GROUPS) {
+            const int hd = idx / BM, row = idx % BM;
+            const int m = m0 + row, head = n0 / 128 + hd;
+            float c_next[4] = {1.f, 1.f, 1.f, 1.f}, sn_next[4] = {0.f, 0.f, 0.f, 0.f};
+            if (tail.table && idx + GROUPS < ITEMS) {
+                const float* cs = tail.table + (long)pos_sh[(idx + GROUPS) % BM] * D;
+                Vec4<float>::load(cs + 4 * j16, c_next);
+                Vec4<float>::load(cs + half + 4 * j16, sn_next);
+            }
+            if (m < M && head < tail.Hq + tail.Hkv) {                   // (values: below, by tiles)
+                const bool is_q = head < tail.Hq;
+                const bf16_t* src = (const bf16_t*)(smem + row * TROW) + hd * 128;
+                float a[4], b[4];
+                Vec4<bf16_t>::load(src + 4 * j16, a);
+                Vec4<bf16_t>::load(src + half + 4 * j16, b);
+                if (tail.q_w) {
+                    float ss = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) ss += a[e] * a[e] + b[e] * b[e];
+                    for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+                    const float rstd = rsqrtf(ss / (float)D + tail.eps);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        a[e] = a[e] * rstd * (is_q ? wq_a[e] : wk_a[e]);
+                        b[e] = b[e] * rstd * (is_q ? wq_b[e] : wk_b[e]);
+                    }
+                }
+                if (tail.table) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) rotate_pair(c[e], sn[e], a[e], b[e]);
+                }
+                bf16_t* dst = nullptr;
+                if (is_q) {
+                    dst = tail.q_out + ((long)m * tail.Hq + head) * D;
+                } else {
+                    const int sl = slot_sh[row];
+                    if (sl >= 0) dst = tail.cache + (long)(sl / tail.P) * page_stride + ((long)(head - tail.Hq) * tail.P + sl % tail.P) * D;
+                }
+                if (dst) {
+                    Vec4<bf16_t>::store(dst + 4 * j16, a);
+                    Vec4<bf16_t>::store(dst + half + 4 * j16, b);
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { c[e] = c_next[e]; sn[e] = sn_next[e]; }
+        }
+        // values: 16 tokens of a head at a time; where their slots lie side by side in one page,
+        // 8 tokens of a feature are one 16-byte store into the transposed value tile [D][P]
+        for (int hd = 0; hd < BN / 128; ++hd) {
+            const int kh = n0 / 128 + hd - tail.Hq - tail.Hkv;
+            if (!tail.slots || kh < 0 || kh >= tail.Hkv) continue;      // the same for the whole block
+            for (int idx = tid; idx < (BM / 16) * D * 2; idx += 64 * NW) {   // 16 rows from r0, feature d, tokens 8 h .. 8 h + 7
+                const int r0 = idx / (D * 2) * 16, d = idx % (D * 2) / 2, h = idx % 2;
+                if (m0 + r0 >= M) continue;
+                const int s0 = slot_sh[r0];
+                bool run = m0 + r0 + 16 <= M && s0 >= 0 && s0 % tail.P + 16 <= tail.P && (s0 % tail.P) % 8 == 0;
+#pragma unroll
+                for (int i = 1; i < 16; ++i) run = run && slot_sh[r0 + i] == s0 + i;
+                if (run) {
+                    Piece16 pc8;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        pc8.e[e] = *(const unsigned short*)(smem + (r0 + 8 * h + e) * TROW + (hd * 128 + d) * 2);
+                    bf16_t* vt = tail.cache + (long)(s0 / tail.P) * page_stride + ((long)(tail.Hkv + kh) * tail.P) * D + s0 % tail.P;
+                    *(uint4_t*)(vt + (long)d * tail.P + 8 * h) = pc8.q;
+                } else {
+                    for (int e = 0; e < 8; ++e) {
+                        const int i = 8 * h + e;
+                        const int si = m0 + r0 + i < M ? slot_sh[r0 + i] : -1;
+                        if (si >= 0)
+                            tail.cache[(long)(si / tail.P) * page_stride + ((long)(tail.Hkv + kh) * tail.P) * D + (long)d * tail.P + si % tail.P] =
+                                *(const bf16_t*)(smem + (r0 + i) * TROW + (hd * 128 + d) * 2);
+                    }
+                }
+            }
+        }
+        return;
+    }
     const int NO = SILU ? N / 2 : N;                       // width of the output
     constexpr int WNO = SILU ? WN / 2 : WN;                // output columns of a wave's strip
     constexpr int ESZ = (int)sizeof(TO);
@@ -338,16 +498,16 @@ bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w) {
     return dt_a == QE_BF16 && dt_w == QE_BF16 && M > 16 && K % 8 == 0 && K >= 64;
 }
 
-template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU>
+template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU, bool QKV = false>
 static int launch_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                       int splits, hipStream_t stream) {
+                       int splits, hipStream_t stream, const QkvTail& tail = QkvTail{}) {
     const int tiles_m = qe_cdiv(M, BM), tiles_n = qe_cdiv(N, BN);
     const long blocks = (long)tiles_m * tiles_n;
     QE_REQUIRE(blocks <= 2147483647L, "mfma gemm: too many tiles");
     const size_t shmem = 2 * (BM + BN) * (BK * 2 + 16);
     static bool attr_set = false;   // one flag per instantiation
     if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)gemm_mfma_kernel<TO, BM, BN, BK, NW, MINB, SILU>,
+        (void)hipFuncSetAttribute((const void*)gemm_mfma_kernel<TO, BM, BN, BK, NW, MINB, SILU, QKV>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         attr_set = true;
     }
@@ -365,31 +525,36 @@ static int launch_mfma(const void* x, const void* w, const float* bias, void* ou
         const long rows = (long)b * M + (long)a * N;
         if (xcd_m == 0 || rows < fewest) { xcd_m = a; xcd_n = b; fewest = rows; }
     }
-    gemm_mfma_kernel<TO, BM, BN, BK, NW, MINB, SILU><<<dim3((unsigned)blocks, (unsigned)splits), 64 * NW, shmem, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n, k_per_split, xcd_m, xcd_n);
+    gemm_mfma_kernel<TO, BM, BN, BK, NW, MINB, SILU, QKV><<<dim3((unsigned)blocks, (unsigned)splits), 64 * NW, shmem, stream>>>(
+        (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n, k_per_split, xcd_m, xcd_n, tail);
     QE_LAUNCH_CHECK();
     return 0;
+}
+
+static int choose_tile(int M, int N, int splits, bool with_256x256 = true) {
+    // The shape is chosen by what the busiest compute unit gets: its number of tiles (they are dealt
+    // out in turn) times a tile's area, over how well the shape uses the unit (measured on large
+    // products: 256 x 256 reaches 1.30, 256 x 128 1.16, 128 x 128 1.07, 64 x 128 0.80 PFLOP/s).
+    // A shape is never taller than the rows need.
+    const long cus = 256;
+    struct Shape { int tile, bm, bn; float rate; };
+    const Shape shapes[4] = {{64, 64, 128, 0.80f}, {128, 128, 128, 1.07f}, {256, 256, 128, 1.16f}, {512, 256, 256, 1.30f}};
+    int tile = 0;
+    float best = 0.f;
+    for (const Shape& sh : shapes) {
+        if (sh.tile != 64 && M <= sh.bm / 2) continue;
+        if (sh.tile == 512 && !with_256x256) continue;
+        const long blocks = (long)qe_cdiv(M, sh.bm) * qe_cdiv(N, sh.bn) * splits;
+        const float cost = (float)qe_cdiv(blocks, cus) * sh.bm * sh.bn / sh.rate;
+        if (tile == 0 || cost < best) { tile = sh.tile; best = cost; }
+    }
+    return tile;
 }
 
 template <typename TO, bool SILU>
 static int pick_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                      int tile, int splits, hipStream_t stream) {
-    // The shape is chosen by what the busiest compute unit gets: its number of tiles (they are dealt
-    // out in turn) times a tile's area, over how well the shape uses the unit (measured on large
-    // products: 256 x 256 reaches 1.30, 256 x 128 1.16, 128 x 128 1.07, 64 x 128 0.80 PFLOP/s).
-    // A shape is never taller than the rows need.
-    if (tile == 0) {
-        const long cus = 256;
-        struct Shape { int tile, bm, bn; float rate; };
-        const Shape shapes[4] = {{64, 64, 128, 0.80f}, {128, 128, 128, 1.07f}, {256, 256, 128, 1.16f}, {512, 256, 256, 1.30f}};
-        float best = 0.f;
-        for (const Shape& sh : shapes) {
-            if (sh.tile != 64 && M <= sh.bm / 2) continue;
-            const long blocks = (long)qe_cdiv(M, sh.bm) * qe_cdiv(N, sh.bn) * splits;
-            const float cost = (float)qe_cdiv(blocks, cus) * sh.bm * sh.bn / sh.rate;
-            if (tile == 0 || cost < best) { tile = sh.tile; best = cost; }
-        }
-    }
+    if (tile == 0) tile = choose_tile(M, N, splits);
     if (tile == 512) return launch_mfma<TO, 256, 256, 64, 4, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 256) return launch_mfma<TO, 256, 128, 64, 8, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 128) return launch_mfma<TO, 128, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, splits, stream);
@@ -411,4 +576,25 @@ int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int
     }
     if (dt_o == QE_BF16) return pick_mfma<bf16_t, false>(x, w, bias, out, M, N, K, tile, splits, stream);
     return pick_mfma<float, false>(x, w, bias, out, M, N, K, tile, splits, stream);
+}
+
+// The q|k|v product of an attention layer with what follows it inside (see QkvTail): x [M, K] .
+// w [(Hq + 2 Hkv) 128, K]^T (+ bias), then q to q_out [M, Hq, 128] and k, v into the cache
+// [pages, 2, Hkv, P, 128] at slots[m] (negative or no slots: nowhere).  positions [M] index the
+// table's rows [cos | sin] of 128 floats; q_w, k_w, table may be null.
+int qe_gemm_qkv(const void* x, const void* w, const float* bias, int M, int K, int Hq, int Hkv, int P,
+                const int* positions, const int* slots, const float* q_w, const float* k_w, float eps,
+                const float* table, void* q_out, void* cache, int tile, hipStream_t stream) {
+    const int N = (Hq + 2 * Hkv) * 128;
+    QE_REQUIRE(K % 8 == 0 && K >= 64 && K < (1 << 22), "qkv gemm: K=%d is no multiple of 8 in [64, 2^22)", K);
+    QE_REQUIRE(M > 16 && Hq > 0 && Hkv > 0 && P >= 16 && (P & (P - 1)) == 0, "qkv gemm: sizes not taken");
+    QE_REQUIRE(tile == 0 || tile == 512 || tile == 256 || tile == 128 || tile == 64, "qkv gemm: tile of %d rows", tile);
+    QE_REQUIRE(!table || positions, "qkv gemm: a rotation needs positions");
+    QkvTail tail{positions, slots, q_w, k_w, table, (bf16_t*)q_out, (bf16_t*)cache, eps, Hq, Hkv, P};
+    // (the 256 x 256 shape has four waves for an epilogue over 65536 values: the others finish it sooner)
+    if (tile == 0) tile = choose_tile(M, N, 1, false);
+    if (tile == 512) return launch_mfma<bf16_t, 256, 256, 64, 4, 1, false, true>(x, w, bias, nullptr, M, N, K, 1, stream, tail);
+    if (tile == 256) return launch_mfma<bf16_t, 256, 128, 64, 8, 1, false, true>(x, w, bias, nullptr, M, N, K, 1, stream, tail);
+    if (tile == 128) return launch_mfma<bf16_t, 128, 128, 64, 4, 2, false, true>(x, w, bias, nullptr, M, N, K, 1, stream, tail);
+    return launch_mfma<bf16_t, 64, 128, 64, 4, 2, false, true>(x, w, bias, nullptr, M, N, K, 1, stream, tail);
 }

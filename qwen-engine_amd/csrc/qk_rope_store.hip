@@ -71,10 +71,10 @@ __global__ __launch_bounds__(64) void qk_rope_store_kernel(
         const int half = rotary_dim / 2;
         const float* cs = table + (long)positions[t] * rotary_dim;
         for (int i = lane; i < half; i += 64) {
-            const float c = cs[i], s = cs[half + i];
-            const float x1 = row[i], x2 = row[half + i];
-            Elem<TA>::store(dst + i, c * x1 - s * x2);
-            Elem<TA>::store(dst + half + i, s * x1 + c * x2);
+            float x1 = row[i], x2 = row[half + i];
+            rotate_pair(cs[i], cs[half + i], x1, x2);
+            Elem<TA>::store(dst + i, x1);
+            Elem<TA>::store(dst + half + i, x2);
         }
         for (int d = rotary_dim + lane; d < D; d += 64) Elem<TA>::store(dst + d, row[d]);
     } else {
@@ -155,11 +155,7 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
             Vec4<float>::load(cs + 4 * j, c);
             Vec4<float>::load(cs + half + 4 * j, sn);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float x1 = a[e], x2 = b[e];
-                a[e] = c[e] * x1 - sn[e] * x2;
-                b[e] = sn[e] * x1 + c[e] * x2;
-            }
+            for (int e = 0; e < 4; ++e) rotate_pair(c[e], sn[e], a[e], b[e]);
         }
         if (dst) {
             Vec4<TA>::store(dst + 4 * j, a);

@@ -50,6 +50,8 @@ def load_library():
         "qe_gemm_silu_supported": [i32, i32, i32, i32, i32],
         "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
         "qe_gemm_partial_splits": [i32, i32, i32],
+        "qe_gemm_qkv_supported": [i32, i32, i32, i32, i32, i32, i32, i32],
+        "qe_gemm_qkv_run": [vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, vp, f32, vp, vp, vp, i32, vp],
         "qe_gemm_fused_supported": [i32, i32, i32, i32, i32],
         "qe_attention_decode_supported": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_supported": [i32, i32, i32, i32, i32],
@@ -262,6 +264,61 @@ def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
     _check(lib.qe_gemm(x.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), M, N, K,
                        _DT[x.dtype], _DT[w.dtype], _DT[out_dtype], algo, epilogue, splits, _stream()), "gemm")
     return out
+
+
+def gemm_qkv_supported(x: torch.Tensor, w: torch.Tensor, cache: torch.Tensor, num_heads: int,
+                       table: Optional[torch.Tensor]) -> bool:
+    """True if gemm_qkv takes these operands: bfloat16, heads of 128, more than 64 rows, a rotation
+    (if any) over the whole head."""
+    lib = load_library()
+    if x.dtype not in _DT or w.dtype not in _DT or cache.dim() != 5 or cache.dtype != torch.bfloat16:
+        return False
+    Hkv, P, D = cache.shape[2], cache.shape[3], cache.shape[4]
+    if w.shape[0] != (int(num_heads) + 2 * Hkv) * D or (table is not None and table.shape[1] != D):
+        return False
+    return bool(lib.qe_gemm_qkv_supported(x.shape[0], x.shape[1], int(num_heads), Hkv, D, P, _DT[x.dtype], _DT[w.dtype]))
+
+
+def gemm_qkv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], num_heads: int, cache: torch.Tensor,
+             positions: Optional[torch.Tensor], q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+             eps: float, table: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+             q_out: Optional[torch.Tensor] = None, tile: int = 0) -> torch.Tensor:
+    """The q|k|v product x [T, K] . w [(Hq + 2 Hkv) D, K]^T (+ bias) with the step after it in its
+    epilogue: per-head q/k RMSNorm (weights or None), half-split rotation from ``table`` (rows
+    [cos | sin] per position, or None), q to the returned [T, Hq, D], k and v into ``cache``
+    [pages, 2, Hkv, P, D] at ``slots`` (negative or no slots: nowhere).  The same results as gemm
+    followed by qk_rope_store.  Needs gemm_qkv_supported."""
+    lib = load_library()
+    _need(x, "x", torch.bfloat16, (None, None))
+    T, K = x.shape
+    dev = x.device
+    _need(cache, "cache", torch.bfloat16, (None, 2, None, None, None), dev)
+    Hq, Hkv, P, D = int(num_heads), cache.shape[2], cache.shape[3], cache.shape[4]
+    _need(w, "w", torch.bfloat16, ((Hq + 2 * Hkv) * D, K), dev)
+    if not gemm_qkv_supported(x, w, cache, Hq, table):
+        raise KernelError("gemm_qkv: operands not taken")
+    if bias is not None:
+        _need(bias, "bias", torch.float32, ((Hq + 2 * Hkv) * D,), dev)
+    if positions is not None:
+        _need(positions, "positions", torch.int32, (T,), dev)
+    if table is not None:
+        if positions is None:
+            raise KernelError("gemm_qkv: a rotation needs positions")
+        _need(table, "table", torch.float32, (None, D), dev)
+    if (q_weight is None) != (k_weight is None):
+        raise KernelError("gemm_qkv: q and k norm weights come together")
+    if q_weight is not None:
+        _need(q_weight, "q_weight", torch.float32, (D,), dev)
+        _need(k_weight, "k_weight", torch.float32, (D,), dev)
+    if slots is not None:
+        _need(slots, "slots", torch.int32, (T,), dev)
+    if q_out is None:
+        q_out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=dev)
+    _need(q_out, "q_out", torch.bfloat16, (T, Hq, D), dev)
+    _check(lib.qe_gemm_qkv_run(x.data_ptr(), w.data_ptr(), _ptr(bias), T, K, Hq, Hkv, P, _ptr(positions), _ptr(slots),
+                               _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(table), q_out.data_ptr(),
+                               cache.data_ptr(), int(tile), _stream()), "gemm (q|k|v with norm, rotation, cache write)")
+    return q_out
 
 
 def qk_rope_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,

@@ -91,16 +91,23 @@ class PagedAttention:
             raise RuntimeError("attention was given no cache")
         T = x.shape[0]
         g = binding.group
-        qkv = ops.gemm(x, self.w_qkv, self.b_qkv)
         eps = self.qk_eps if self.qk_eps is not None else 0.0
         slots = ctx.slots[g] if binding.write else None
         cache = binding.kv
         pos = self.position
-        if pos is None or getattr(pos, "fused", False):
-            table = pos.table() if pos is not None else None
-            if table is not None and ctx.max_position >= table.shape[0]:
-                raise RuntimeError(f"position {ctx.max_position} is beyond the rotation table "
-                                   f"({table.shape[0]} positions)")
+        fused_position = pos is None or getattr(pos, "fused", False)
+        table = pos.table() if (pos is not None and fused_position) else None
+        if table is not None and ctx.max_position >= table.shape[0]:
+            raise RuntimeError(f"position {ctx.max_position} is beyond the rotation table "
+                               f"({table.shape[0]} positions)")
+        if fused_position and ops.gemm_qkv_supported(x, self.w_qkv, cache, self.hq, table):
+            # many rows (portions of prompts): norm, rotation and cache write are the epilogue of the
+            # q|k|v product, which never stores its result
+            q = ops.gemm_qkv(x, self.w_qkv, self.b_qkv, self.hq, cache, ctx.positions if table is not None else None,
+                             self.q_norm, self.k_norm, eps, table, slots)
+            return self._attend(q, ctx, cache, g, T)
+        qkv = ops.gemm(x, self.w_qkv, self.b_qkv)
+        if fused_position:
             only_new_tokens = (ctx.dec_tokens is not None and ctx.dec_tokens.shape[0] == T and
                                (ctx.other_tokens is None or ctx.other_tokens.shape[0] == 0))
             if (only_new_tokens and T <= FUSED_DECODE_MAX_TOKENS and binding.write and
@@ -121,6 +128,9 @@ class PagedAttention:
             pos.apply(packed, ctx.positions, self.hq, self.hkv)
             q = ops.qk_rope_store(packed.view(T, -1), self.hq, self.hkv, self.d, None, None, None, 0.0,
                                   None, slots, cache, ctx.page_size)
+        return self._attend(q, ctx, cache, g, T)
+
+    def _attend(self, q: torch.Tensor, ctx, cache: torch.Tensor, g: int, T: int) -> torch.Tensor:
         o = ops.attention(q, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g], self.scale, self.window,
                           dec_tokens=ctx.dec_tokens, max_dec_position=ctx.max_dec_position,
                           other_tokens=ctx.other_tokens,

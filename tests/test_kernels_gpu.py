@@ -291,6 +291,70 @@ def test_qk_norm_rope_store_of_many_tokens(ops, dtype, hq, hkv, d, page):
     assert torch.equal(cache[:, 1].float().cpu(), want[:, 1].to(dtype).float())      # values are copied exactly
 
 
+@pytest.mark.parametrize("hq,hkv,page,K", [(16, 8, 16, 1024), (3, 2, 32, 96), (5, 1, 16, 160)])
+@pytest.mark.parametrize("norm,rope,bias", [(True, True, False), (False, True, True), (True, False, False),
+                                            (False, False, False)])
+def test_qkv_product_with_norm_rotation_and_cache_write_inside(ops, hq, hkv, page, K, norm, rope, bias):
+    """The tiled product that norms, rotates and writes the cache from its own result, in every
+    tile shape, against the plain functions and against the product followed by the separate
+    kernel (the same arithmetic on the same rounded product: equal to the bit).  Tokens: a prompt
+    from a page's start (runs of 16 side by side), one from the middle of a page, scattered
+    slots, tokens without a slot; the number of tokens is no multiple of a tile."""
+    bf, d, eps = torch.bfloat16, 128, 1e-6
+    lens = [(0, 200), (page // 2 + 1, 100), (3, 16)]
+    T = sum(n for _, n in lens) + 24
+    width = (hq + 2 * hkv) * d
+    assert T * (hq + 2 * hkv) > 2048                                  # (the separate kernel is then the one with the same order of sums)
+    x = rand(T, K, seed=600, dtype=bf)
+    w = rand(width, K, seed=601, dtype=bf, scale=1.0 / math.sqrt(K))
+    b = rand(width, seed=602, scale=0.5) if bias else None
+    qw = 1 + rand(d, seed=603, scale=0.1) if norm else None
+    kw = 1 + rand(d, seed=604, scale=0.1) if norm else None
+    table = P.rope_table(10000.0, d, 256) if rope else None
+    pages = 40
+    perm = torch.randperm(pages, generator=torch.Generator().manual_seed(605)).tolist()
+    pos, slots = [], []
+    for first, n in lens:
+        mine = [perm.pop() for _ in range((first + n + page - 1) // page)]
+        for p_ in range(first, first + n):
+            pos.append(p_)
+            slots.append(mine[p_ // page] * page + p_ % page)
+    free = [pg * page + o for pg in perm[:4] for o in range(page)]
+    pick = torch.randperm(len(free), generator=torch.Generator().manual_seed(606))[:24].tolist()
+    for i in range(24):
+        pos.append(100 + i)
+        slots.append(-1 if i % 5 == 4 else free[pick[i]])
+    pos, slots = torch.tensor(pos, dtype=torch.int32), torch.tensor(slots, dtype=torch.int32)
+    dev = lambda t: None if t is None else t.to(DEV)
+    # the product and the separate kernel
+    cache2 = torch.zeros(pages, 2, hkv, page, d, dtype=bf, device=DEV)
+    qkv = ops.gemm(x.to(DEV), w.to(DEV), dev(b))
+    q2 = ops.qk_rope_store(qkv, hq, hkv, d, dev(pos) if rope else None, dev(qw), dev(kw), eps, dev(table),
+                           dev(slots), cache2, page)
+    # the plain functions on the rounded product
+    y = qkv.float().cpu()
+    qr = y[:, :hq * d].view(T, hq, d)
+    kr = y[:, hq * d:(hq + hkv) * d].view(T, hkv, d)
+    if norm:
+        qr, kr = P.rms_norm(qr, qw, eps), P.rms_norm(kr, kw, eps)
+    if rope:
+        qr, kr = P.apply_rope(table, pos, qr), P.apply_rope(table, pos, kr)
+    assert ops.gemm_qkv_supported(x.to(DEV), w.to(DEV), cache2, hq, dev(table))
+    for tile in (0, 64, 128, 256, 512):
+        cache = torch.zeros(pages, 2, hkv, page, d, dtype=bf, device=DEV)
+        q = ops.gemm_qkv(x.to(DEV), w.to(DEV), dev(b), hq, cache, dev(pos) if rope else None, dev(qw), dev(kw), eps,
+                         dev(table), dev(slots), tile=tile)
+        close(q, qr, bf)
+        assert torch.equal(q, q2), f"tile {tile}: q differs from the separate kernel's"
+        assert torch.equal(cache, cache2), f"tile {tile}: the cache differs from the separate kernel's"
+    # without slots nothing is written
+    cache = torch.zeros(pages, 2, hkv, page, d, dtype=bf, device=DEV)
+    q = ops.gemm_qkv(x.to(DEV), w.to(DEV), dev(b), hq, cache, dev(pos) if rope else None, dev(qw), dev(kw), eps,
+                     dev(table), None)
+    assert torch.equal(q, q2) and not bool(cache.any())
+    assert not ops.gemm_qkv_supported(x[:64].to(DEV), w.to(DEV), cache, hq, dev(table))      # few rows: not this kernel's
+
+
 def test_argmax_takes_the_lowest_index_on_ties(ops):
     logits = rand(5, 50000, seed=80)
     logits[0, 49999] = 9.0
