@@ -24,6 +24,9 @@ Other sizes and workloads (not what the default line reports):
                             portions of 512 tokens beside decoded tokens.  value = generated tokens a second
   --workload shared-prefix  N requests (default 32) that share a 1024-token prefix, each with 1024 tokens
                             of its own and 512 new tokens; the prefix's pages are shared
+  --warmup-passes N         both: untimed passes over the workload with other tokens before the timed
+                            one (default 1: the decode graphs are recorded there, as in a server that
+                            has run for a while; 0 times the recording too)
 """
 import argparse
 import json
@@ -69,6 +72,8 @@ def parse():
     ap.add_argument("--model", default="0.6b", choices=sorted(SIZES), help="whose layer sizes")
     ap.add_argument("--workload", default="decode", choices=["decode", "serving", "shared-prefix"])
     ap.add_argument("--requests", type=int, default=None, help="requests of the serving workloads")
+    ap.add_argument("--warmup-passes", type=int, default=1,
+                    help="serving workloads: untimed passes before the timed one (they record the decode graphs)")
     return ap.parse_args()
 
 
@@ -78,27 +83,38 @@ def serving_run(args, cfg, model, layers, full_layers) -> int:
     from qwen_engine_amd import EngineConfig
     from qwen_engine_amd.engine.llm_engine import LLMEngine
 
-    g = torch.Generator().manual_seed(args.seed + 2)
     V = cfg.vocab_size
     if args.workload == "serving":
         n = args.requests or 64
-        lens = torch.randint(128, 2049, (n,), generator=g).tolist()
-        prompts = [torch.randint(0, V, (k,), generator=g).tolist() for k in lens]
         new_tokens, sharing = 256, False
         what = f"{n} requests, prompts uniform in [128, 2048], {new_tokens} new tokens each, portions of 512"
     else:
         n = args.requests or 32
-        prefix = torch.randint(0, V, (1024,), generator=g).tolist()
-        prompts = [prefix + torch.randint(0, V, (1024,), generator=g).tolist() for _ in range(n)]
         new_tokens, sharing = 512, True
         what = f"{n} requests sharing a 1024-token prefix, 1024 tokens of their own, {new_tokens} new tokens each"
-    longest = max(len(p) for p in prompts) + new_tokens
+
+    def make_prompts(seed):
+        g = torch.Generator().manual_seed(seed)
+        if args.workload == "serving":
+            lens = torch.randint(128, 2049, (n,), generator=g).tolist()
+            return [torch.randint(0, V, (k,), generator=g).tolist() for k in lens]
+        prefix = torch.randint(0, V, (1024,), generator=g).tolist()
+        return [prefix + torch.randint(0, V, (1024,), generator=g).tolist() for _ in range(n)]
+
+    prompts = make_prompts(args.seed + 2)
+    longest = 2048 + new_tokens
     P = args.block_size
     pages = n * ((longest + P - 1) // P + 1)
     ecfg = EngineConfig(dtype="bfloat16" if args.dtype == "bf16" else "float32", block_size=P, num_blocks=pages,
                         max_num_seqs=n, max_model_len=longest, max_step_tokens=2048, prefill_chunk=512,
                         enable_prefix_sharing=sharing, seed=args.seed)
     engine = LLMEngine(model, None, ecfg)
+    # Untimed passes over the same workload with other tokens: a server records its decode graphs
+    # once and runs for long, so the timed pass should find them recorded.
+    for i in range(args.warmup_passes):
+        engine.submit(make_prompts(args.seed + 100 + i), max_new_tokens=new_tokens, ignore_eos=True)
+        engine.run()
+    before = engine.stats()
     engine.submit(prompts, max_new_tokens=new_tokens, ignore_eos=True)
     torch.cuda.synchronize()
     t = time.perf_counter()
@@ -119,7 +135,7 @@ def serving_run(args, cfg, model, layers, full_layers) -> int:
     prompt_tokens = sum(len(p) for p in prompts)
     line = {
         "metric": f"generated tok/s, {args.workload} workload (Qwen3-{args.model.upper()} sizes)",
-        "value": round(generated / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 0,
+        "value": round(generated / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup_passes,
         "ms_per_step": round(dt / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform-random token ids",
         "config": {"model": f"Qwen3-{args.model.upper()} sizes (random weights)", "layers": layers,
@@ -130,7 +146,8 @@ def serving_run(args, cfg, model, layers, full_layers) -> int:
                    "parallelism": "single GPU"},
         "seconds": round(dt, 3), "prompt_tokens": prompt_tokens, "generated_tokens": generated,
         "all_tokens_per_s": round((prompt_tokens + generated) / dt, 1),
-        "scheduler": {k: v for k, v in stats.items() if isinstance(v, (int, float))},
+        "warmup_unit": "passes over the workload with other tokens",
+        "scheduler": {k: v - before.get(k, 0) for k, v in stats.items() if isinstance(v, (int, float))},
     }
     print(json.dumps(line), flush=True)
     return 0

@@ -135,6 +135,8 @@ class LLMEngine:
         d.update(self.runner.cache.stats)
         d["free_pages"] = [p.num_free for p in self.runner.cache.pools]
         d["kept_pages"] = self.runner.cache.num_kept
+        d["graph_steps"] = self.runner.graph_steps
+        d["graphs_recorded"] = self.runner.graphs_recorded
         return d
 
 

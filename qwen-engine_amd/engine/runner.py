@@ -69,6 +69,7 @@ class ModelRunner:
     """
 
     SPLIT_BUCKET = 8      # decode graphs are recorded per this many splits of the keys
+    GRAPH_ROWS_EXACT, GRAPH_ROWS_STEP = 8, 8   # graphs are recorded for 1..8 rows, then for multiples of 8
     MAX_GRAPHS = 24       # recorded graphs kept (each holds its own activations); the least recently used goes first
 
     def __init__(self, model: DecoderModel, page_size: int, num_pages, max_requests: int,
@@ -125,6 +126,7 @@ class ModelRunner:
         self._stage_event = torch.cuda.Event()
         self.steps_run = 0
         self.graph_steps = 0
+        self.graphs_recorded = 0
 
     # ---- requests ------------------------------------------------------------------
     def add_request(self, req_id: Hashable):
@@ -325,8 +327,20 @@ class ModelRunner:
     # ---- decoding through a recorded graph ------------------------------------------------
     def _decode_step_with_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._single_token_layout(entries)
-        B, n_groups = len(seqs), len(self.cache.groups)
+        n_live, n_groups = len(seqs), len(self.cache.groups)
         i32 = np.int32
+        # Graphs are recorded for 1 to 8 rows and for multiples of 8: a batch in between is filled up
+        # with rows that stand at position 0 of the first request's table, write nowhere (cache slot
+        # -1) and whose logits are dropped, so that a batch that shrinks request by request does not
+        # record a graph for every size it passes.
+        B = n_live if n_live <= self.GRAPH_ROWS_EXACT else -(-n_live // self.GRAPH_ROWS_STEP) * self.GRAPH_ROWS_STEP
+        if B > n_live:
+            fill = B - n_live
+            token_ids = np.concatenate([token_ids, np.zeros(fill, dtype=i32)])
+            positions = np.concatenate([positions, np.zeros(fill, dtype=i32)])
+            tok_seq = np.concatenate([tok_seq, np.full(fill, tok_seq[0], dtype=i32)])
+            slots = [np.concatenate([x, np.full(fill, -1, dtype=i32)]) for x in slots]
+        state_slots = [s.state_slot for s in seqs] + [seqs[0].state_slot] * (B - n_live)
         cap = 2 * B                                    # table updates a decode step can bring per group
         splits = int(positions.max()) // ops.DECODE_SPLIT_KEYS + 1
         bucket = (splits + self.SPLIT_BUCKET - 1) // self.SPLIT_BUCKET * self.SPLIT_BUCKET
@@ -344,9 +358,10 @@ class ModelRunner:
             while len(self._graphs) >= self.MAX_GRAPHS:
                 self._graphs.pop(next(iter(self._graphs)))     # dicts keep insertion order: the oldest use
             rec = self._record_decode_graph(B, bucket, cap)
+            self.graphs_recorded += 1
         self._graphs[key] = rec                                # (re)inserted last = most recently used
         iota = np.arange(B, dtype=i32)
-        parts = [token_ids, positions, tok_seq, iota, np.asarray([s.state_slot for s in seqs], dtype=i32), iota]
+        parts = [token_ids, positions, tok_seq, iota, np.asarray(state_slots, dtype=i32), iota]
         for g in range(n_groups):
             pad = cap - len(upd_idx[g])
             parts += [slots[g], upd_idx[g], np.full(pad, -1, dtype=i32), upd_val[g], np.zeros(pad, dtype=i32)]
@@ -356,7 +371,7 @@ class ModelRunner:
         rec["event"].record()
         rec["graph"].replay()
         self.graph_steps += 1
-        return rec["logits"].clone()                   # the graph's own output is overwritten by the next replay
+        return rec["logits"][:n_live].clone()          # the graph's own output is overwritten by the next replay
 
     def _record_decode_graph(self, B: int, bucket: int, cap: int):
         """Static buffers for a decode step of B requests whose keys fit ``bucket`` splits, one

@@ -200,3 +200,37 @@ def test_command_line(folders, tmp_path):
     assert " ".join(map(str, [9, 10] + want[1])) in lines
     stats = json.loads(lines[-1])
     assert stats["decode_tokens"] == 8 and stats["prefill_tokens"] == 6
+
+
+def test_decode_batches_between_recorded_sizes_are_filled_up(folders):
+    """11 requests decode through the graph recorded for 16 rows, and after two of them have ended
+    the 9 that remain replay the same graph: the logits are those of a runner without graphs."""
+    from qwen_engine_amd.engine import ModelRunner, StepEntry, load_model
+    cfg, w = P.read_folder(folders["D"])
+    model = load_model(folders["D"], dtype="bfloat16")
+    prompts = prompts_for(cfg, tuple(range(5, 16)), 9)
+    runners = [ModelRunner(model, page_size=16, num_pages=40, max_requests=11, use_graphs=flag) for flag in (True, False)]
+    assert runners[0].GRAPH_ROWS_EXACT < 9 and runners[0].GRAPH_ROWS_STEP == 8
+    outs = []
+    for runner in runners:
+        got = []
+        for i, p in enumerate(prompts):
+            runner.add_request(i)
+            runner.step([StepEntry(i, p, [])])
+        live = list(range(11))
+        for step in range(4):
+            if step == 2:
+                for i in (3, 7):
+                    runner.free_request(i)
+                    live.remove(i)
+            got.append(runner.step([StepEntry(i, [(7 * i + step) % cfg["vocab_size"]], [0]) for i in live]))
+        outs.append(got)
+    assert runners[0].graph_steps == 4 and runners[0].graphs_recorded == 1 and runners[1].graph_steps == 0
+    for a, b in zip(*outs):
+        assert a.shape == b.shape and a.shape[0] in (11, 9)
+        assert float((a - b).abs().max()) <= 1e-3 * float(b.abs().max())
+    # and they are the plain implementation's logits for the first request's sequence
+    seq = prompts[0] + [(7 * 0 + s) % cfg["vocab_size"] for s in range(4)]
+    ref = P.forward_logits(cfg, w, seq, act_dtype=torch.bfloat16)
+    for s in range(4):
+        assert float((outs[0][s][0].cpu() - ref[len(prompts[0]) + s]).abs().max()) <= 2e-2 * float(ref.abs().max())
