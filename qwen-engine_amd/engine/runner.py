@@ -69,8 +69,7 @@ class ModelRunner:
     """
 
     SPLIT_BUCKET = 8      # decode graphs are recorded per this many splits of the keys
-    GRAPH_ROWS_EXACT, GRAPH_ROWS_STEP = 8, 8   # graphs are recorded for 1..8 rows, then for multiples of 8
-    MAX_GRAPHS = 24       # recorded graphs kept (each holds its own activations); the least recently used goes first
+    MAX_GRAPHS = 32       # recorded graphs kept (each holds its own activations); the least recently used goes first
 
     def __init__(self, model: DecoderModel, page_size: int, num_pages, max_requests: int,
                  prefix_sharing: bool = False, use_graphs: Optional[bool] = None,
@@ -127,6 +126,15 @@ class ModelRunner:
         self.steps_run = 0
         self.graph_steps = 0
         self.graphs_recorded = 0
+
+    @staticmethod
+    def graph_rows(n: int) -> int:
+        """The rows of the recorded decode graph that a batch of n single tokens replays: n itself up
+        to 8, the next multiple of 8 up to 64, of 32 beyond."""
+        if n <= 8:
+            return n
+        step = 8 if n <= 64 else 32
+        return -(-n // step) * step
 
     # ---- requests ------------------------------------------------------------------
     def add_request(self, req_id: Hashable):
@@ -329,11 +337,11 @@ class ModelRunner:
         seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._single_token_layout(entries)
         n_live, n_groups = len(seqs), len(self.cache.groups)
         i32 = np.int32
-        # Graphs are recorded for 1 to 8 rows and for multiples of 8: a batch in between is filled up
+        # Graphs are recorded for 1 to 8 rows, for multiples of 8 and, beyond 64, of 32: a batch in between is filled up
         # with rows that stand at position 0 of the first request's table, write nowhere (cache slot
         # -1) and whose logits are dropped, so that a batch that shrinks request by request does not
         # record a graph for every size it passes.
-        B = n_live if n_live <= self.GRAPH_ROWS_EXACT else -(-n_live // self.GRAPH_ROWS_STEP) * self.GRAPH_ROWS_STEP
+        B = self.graph_rows(n_live)
         if B > n_live:
             fill = B - n_live
             token_ids = np.concatenate([token_ids, np.zeros(fill, dtype=i32)])

@@ -210,7 +210,7 @@ def test_decode_batches_between_recorded_sizes_are_filled_up(folders):
     model = load_model(folders["D"], dtype="bfloat16")
     prompts = prompts_for(cfg, tuple(range(5, 16)), 9)
     runners = [ModelRunner(model, page_size=16, num_pages=40, max_requests=11, use_graphs=flag) for flag in (True, False)]
-    assert runners[0].GRAPH_ROWS_EXACT < 9 and runners[0].GRAPH_ROWS_STEP == 8
+    assert [ModelRunner.graph_rows(n) for n in (1, 8, 9, 11, 16, 57, 64, 65, 200)] == [1, 8, 16, 16, 16, 64, 64, 96, 224]
     outs = []
     for runner in runners:
         got = []
