@@ -234,3 +234,45 @@ def test_decode_batches_between_recorded_sizes_are_filled_up(folders):
     ref = P.forward_logits(cfg, w, seq, act_dtype=torch.bfloat16)
     for s in range(4):
         assert float((outs[0][s][0].cpu() - ref[len(prompts[0]) + s]).abs().max()) <= 2e-2 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_random_engine_sizes_and_prompt_sets(folders, which):
+    """Twenty draws of prompts (some sharing a prefix, one a prefix of another, one twice) and of
+    engine sizes (page size, pages from barely enough for one request to enough for all, live
+    requests, token budget, portion size, prefix sharing on or off): greedy float32 tokens equal
+    the plain implementation's, every request runs to its length, and every page comes back."""
+    import random
+    cfg, w = P.read_folder(folders[which])
+    base = prompts_for(cfg, (1, 7, 16, 30, 45, 3), 21)
+    plain = {}
+    preempted = shared = 0
+    for seed in range(20):
+        rng = random.Random(31 * ord(which) + seed)
+        prompts = list(base) + [base[3][:20] + base[2][:5], base[4][:32], list(base[4])]
+        rng.shuffle(prompts)
+        prompts = prompts[:rng.randint(2, len(prompts))]
+        new = rng.choice([1, 2, 6, 12])
+        page = rng.choice([1, 2, 4, 8, 16])
+        longest = max(len(p) for p in prompts) + new
+        per_request = -(-longest // page)
+        sizes = dict(dtype="float32", block_size=page, max_num_seqs=rng.randint(1, 5),
+                     num_blocks=rng.choice([per_request + 1, 2 * per_request, per_request * len(prompts) + 4]),
+                     max_model_len=longest + rng.choice([0, 3, 50]), max_step_tokens=rng.choice([3, 8, 20, 64, 2048]),
+                     prefill_chunk=rng.choice([2, 5, 16, 512]), enable_prefix_sharing=rng.random() < 0.7)
+        want = []
+        for p in prompts:
+            if (tuple(p), new) not in plain:
+                plain[tuple(p), new] = P.greedy_generate(cfg, w, p, new)
+            want.append(plain[tuple(p), new])
+        eng = LLMEngine.from_folder(folders[which], EngineConfig(**sizes))
+        eng.submit(prompts, max_new_tokens=new, ignore_eos=True)
+        res = eng.run()
+        assert [r.token_ids for r in res] == want, (seed, sizes)
+        assert all(r.finish_reason == "length" for r in res), (seed, sizes)
+        cache = eng.runner.cache
+        cache.check_invariants()
+        assert all(cache.available(g) == pool.num_pages for g, pool in enumerate(cache.pools)), (seed, sizes)
+        preempted += eng.stats()["preemptions"] > 0
+        shared += eng.stats()["shared_prefix_tokens"] > 0
+    assert preempted >= 2 and shared >= 5          # the draws reach both

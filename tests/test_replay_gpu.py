@@ -115,3 +115,25 @@ def test_a_step_without_wanted_logits_writes_no_file(cases, tmp_path):
     got = traces.collect(t, out_dir, cfg["vocab_size"])["x"]
     for pos in (10, 19):
         assert abs(got[pos] - ref["float32"]["r0"][pos].numpy()).max() < 1e-4 * float(ref["float32"]["r0"].abs().max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+def test_random_traces(cases, tmp_path, which, dtype):
+    """Six draws of the cutting: mixed traces with one to four live requests and 0 to 40 tokens
+    decoded one by one at the end, or portions of drawn sizes; page sizes other than the usual."""
+    import random
+    folder, cfg, reqs, ref = cases[which]
+    pages = {"A": [4, 1, 16], "B": [8, 2], "C": [16, 32], "D": [16, 32, 64]}[which]
+    for seed in range(6):
+        rng = random.Random(100 * ord(which) + seed)
+        if rng.random() < 0.75:
+            trace = traces.mixed(reqs, seed=seed, max_live=rng.randint(1, 4), tail=rng.choice([0, 1, 5, 12, 40]))
+        else:
+            trace = traces.portions(reqs, sizes=tuple(rng.choice([2, 3, 7, 16, 17, 33, 64, 65, 100, 129]) for _ in range(9)))
+        page = rng.choice(pages)
+        out_dir = str(tmp_path / f"out{seed}")
+        traces.run_in_process(trace, folder, dtype, out_dir, page)
+        got = traces.collect(trace, out_dir, cfg["vocab_size"])
+        bad, _ = traces.first_mismatch(got, ref[dtype], TOL[dtype])
+        assert bad is None, f"draw {seed}, page size {page}: first wrong logits at (request, position, relative error) {bad}"
