@@ -36,6 +36,11 @@ static bool tiled_for_few_rows(int M, int N, int K, int dt_a, int dt_w) {
     return M > 16 && (long)N * K >= (16L << 20) && qe_gemm_mfma_ok(M, N, K, dt_a, dt_w);
 }
 
+// 1 if a product of these sizes is quickest as partial products (epilogue 3) from the tiled kernel
+extern "C" int qe_gemm_partial_preferred(int M, int N, int K, int dt_a, int dt_w) {
+    return (M <= 64 && tiled_for_few_rows(M, N, K, dt_a, dt_w)) ? 1 : 0;
+}
+
 // number of partial products that epilogue 3 should be asked for
 extern "C" int qe_gemm_partial_splits(int M, int N, int K) {
     if (tiled_for_few_rows(M, N, K, QE_BF16, QE_BF16)) {

@@ -94,9 +94,63 @@ __global__ __launch_bounds__(64) void qk_rope_store_kernel(
 // elements that are neighbours in the tile.  That needs the 16 tokens to lie side by side in
 // one page (consecutive slots), which is how the tokens of a prompt lie; a block of tokens that
 // do not is written element by element.
+//
+// The projection can also come as 32-bit partial products [S][T][width] of a product that was cut
+// along K (few rows against a large matrix: the cut fills the chip): they are added here in the
+// order of S, with the bias if there is one, and rounded to the activation type first, as the
+// product itself would have stored them.
+template <typename TA>
+struct QkvSource {
+    const TA* qkv;          // [T][width], or null
+    const float* parts;     // [S][T][width]
+    const float* bias;      // [width] or null (with parts only)
+    int S;
+    long stride;            // T * width
+    // four neighbouring elements from element index idx = t * width + col
+    __device__ __forceinline__ void load4(long idx, int col, float (&v)[4]) const {
+        if (qkv) {
+            Vec4<TA>::load(qkv + idx, v);
+            return;
+        }
+        // (eight parts are asked for before the first is used: one trip to memory for them all)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = 0.f;
+        for (int s0 = 0; s0 < S; s0 += 8) {
+            float p[8][4];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int sk = s0 + k < S ? s0 + k : S - 1;
+                Vec4<float>::load(parts + sk * stride + idx, p[k]);
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (s0 + k < S) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += p[k][e];
+                }
+        }
+        if (bias) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += bias[col + e];
+        }
+        TA r[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { Elem<TA>::store(r + e, v[e]); v[e] = Elem<TA>::load(r + e); }
+    }
+    __device__ __forceinline__ float load1(long idx, int col) const {
+        if (qkv) return Elem<TA>::load(qkv + idx);
+        float v = parts[idx];
+        for (int s = 1; s < S; ++s) v += parts[s * stride + idx];
+        if (bias) v += bias[col];
+        TA r;
+        Elem<TA>::store(&r, v);
+        return Elem<TA>::load(&r);
+    }
+};
+
 template <typename TA>
 __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
-    const TA* __restrict__ qkv, const int* __restrict__ positions,
+    const QkvSource<TA> in, const int* __restrict__ positions,
     const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
     const float* __restrict__ table, const int* __restrict__ slot, TA* __restrict__ cache,
     TA* __restrict__ q_out, TA* __restrict__ packed_out, int Hq, int Hkv, int D, int P) {
@@ -110,13 +164,14 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
     const int s = slot ? slot[t] : -1;
     const float* cs = table ? table + (long)positions[t] * D : nullptr;
     const int nloop = packed_out ? nheads : Hq + Hkv;   // (values go to the cache by tiles, further down)
-    for (int head = threadIdx.x / lph; head < nloop; head += heads_per_pass) {
+    // (the blocks (t, 0 .. gridDim.y - 1) share the token's heads: more blocks where the tokens are few)
+    for (int head = threadIdx.x / lph + blockIdx.y * heads_per_pass; head < nloop; head += heads_per_pass * gridDim.y) {
         const bool is_q = head < Hq;
         const bool is_k = !is_q && head < Hq + Hkv;
-        const TA* src = qkv + t * width + (long)head * D;
+        const long src = t * width + (long)head * D;   // element index of the head's first feature
         float a[4], b[4];                      // features 4 j .. 4 j + 3 and half + 4 j .. half + 4 j + 3
-        Vec4<TA>::load(src + 4 * j, a);
-        Vec4<TA>::load(src + half + 4 * j, b);
+        in.load4(src + 4 * j, head * D + 4 * j, a);
+        in.load4(src + half + 4 * j, head * D + half + 4 * j, b);
         TA* dst = nullptr;
         if (packed_out) {
             dst = packed_out + t * width + (long)head * D;
@@ -162,7 +217,7 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
             Vec4<TA>::store(dst + half + 4 * j, b);
         }
     }
-    if (packed_out || !slot) return;
+    if (packed_out || !slot || blockIdx.y != 0) return;
 
     // ---- values of the 16 tokens t0 .. t0 + n - 1, key/value heads t - t0, t - t0 + n, ... ----
     extern __shared__ __attribute__((aligned(16))) unsigned char vsh[];   // [D][16] elements + 16 bytes a row
@@ -172,16 +227,31 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
     const int s0 = slot[t0];
     bool run = s0 >= 0 && s0 % P + n <= P;                 // side by side in one page?
     for (int i = 1; i < n; ++i) run = run && slot[t0 + i] == s0 + i;
+    if (!run) {
+        // not side by side (single new tokens of several requests): every block writes its own
+        // token's values, four neighbouring features a thread, element by element into the tiles
+        if (s < 0) return;
+        TA* page = cache + (long)(s / P) * (2L * Hkv * P * D) + (long)Hkv * P * D + s % P;
+        for (int idx = threadIdx.x; idx < Hkv * D / 4; idx += 256) {
+            const int col = 4 * idx;                       // feature col % D of key/value head col / D
+            float x[4];
+            in.load4(t * width + (long)(Hq + Hkv) * D + col, (Hq + Hkv) * D + col, x);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) Elem<TA>::store(page + (long)(col + e) * P, x[e]);
+        }
+        return;
+    }
     const int cpr = D / 8;                                 // 8-element chunks in a head
     for (int kh = (int)(t - t0); kh < Hkv; kh += n) {
-        const TA* src = qkv + t0 * width + (long)(Hq + Hkv + kh) * D;
-        if (run) {
+        const int col0 = (Hq + Hkv + kh) * D;
+        const long src = t0 * width + col0;
+        {
             __syncthreads();                               // the last head's readers are done
             for (int idx = threadIdx.x; idx < n * cpr; idx += 256) {
                 const int i = idx / cpr, c = idx % cpr;
                 float x[8];
-                Vec4<TA>::load(src + (long)i * width + 8 * c, *(float(*)[4])x);
-                Vec4<TA>::load(src + (long)i * width + 8 * c + 4, *(float(*)[4])(x + 4));
+                in.load4(src + (long)i * width + 8 * c, col0 + 8 * c, *(float(*)[4])x);
+                in.load4(src + (long)i * width + 8 * c + 4, col0 + 8 * c + 4, *(float(*)[4])(x + 4));
 #pragma unroll
                 for (int e = 0; e < 8; ++e) Elem<TA>::store((TA*)(vsh + (8 * c + e) * srow) + i, x[e]);
             }
@@ -199,14 +269,6 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
                 } else {
                     for (int e = 0; e < 4; ++e) if (4 * q4 + e < n) to[e] = from[e];
                 }
-            }
-        } else {
-            for (int idx = threadIdx.x; idx < n * D; idx += 256) {
-                const int i = idx / D, d = idx % D;
-                const int si = slot[t0 + i];
-                if (si >= 0)
-                    cache[(long)(si / P) * (2L * Hkv * P * D) + ((long)(Hkv + kh) * P) * D + (long)d * P + si % P] =
-                        src[(long)i * width + d];
             }
         }
     }
@@ -230,12 +292,12 @@ extern "C" int qe_qk_rope_store(const void* qkv, const int* positions, const flo
         (!table || rotary_dim == D)) {
         if (dt_a == QE_F32)
             qk_rope_store_vec_kernel<float><<<T, 256, (size_t)D * (16 * 4 + 16), stream>>>(
-                (const float*)qkv, positions, q_w, k_w, eps, table, slot, (float*)cache, (float*)q_out,
-                (float*)packed_out, Hq, Hkv, D, P);
+                QkvSource<float>{(const float*)qkv, nullptr, nullptr, 0, 0}, positions, q_w, k_w, eps, table, slot,
+                (float*)cache, (float*)q_out, (float*)packed_out, Hq, Hkv, D, P);
         else if (dt_a == QE_BF16)
             qk_rope_store_vec_kernel<bf16_t><<<T, 256, (size_t)D * (16 * 2 + 16), stream>>>(
-                (const bf16_t*)qkv, positions, q_w, k_w, eps, table, slot, (bf16_t*)cache, (bf16_t*)q_out,
-                (bf16_t*)packed_out, Hq, Hkv, D, P);
+                QkvSource<bf16_t>{(const bf16_t*)qkv, nullptr, nullptr, 0, 0}, positions, q_w, k_w, eps, table, slot,
+                (bf16_t*)cache, (bf16_t*)q_out, (bf16_t*)packed_out, Hq, Hkv, D, P);
         else
             QE_REQUIRE(false, "qk_rope_store: unknown dtype %d", dt_a);
         QE_LAUNCH_CHECK();
@@ -253,6 +315,36 @@ extern "C" int qe_qk_rope_store(const void* qkv, const int* positions, const flo
             (bf16_t*)q_out, (bf16_t*)packed_out, Hq, Hkv, D, P);
     else
         QE_REQUIRE(false, "qk_rope_store: unknown dtype %d", dt_a);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// 1 if qe_qk_rope_store_parts takes these sizes (the kernel with several lanes a head: a head size
+// 8 * 2^k up to 512 and a rotation, if any, over the whole head)
+extern "C" int qe_qk_rope_store_parts_supported(int D, int rotary_dim) {
+    const int lph = D / 8;
+    return (D % 8 == 0 && lph >= 1 && lph <= 64 && (lph & (lph - 1)) == 0 && (rotary_dim == 0 || rotary_dim == D)) ? 1 : 0;
+}
+
+// The same from 32-bit partial products parts [S, T, (Hq + 2 Hkv) D] (+ bias [width] or null) of
+// the projection; q_out and cache are bfloat16.
+extern "C" int qe_qk_rope_store_parts(const float* parts, int S, const float* bias, const int* positions,
+                                      const float* q_w, const float* k_w, float eps, const float* table,
+                                      int rotary_dim, const int* slot, void* cache, void* q_out, int T, int Hq,
+                                      int Hkv, int D, int P, hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && S >= 1 && Hq > 0 && Hkv > 0 && D > 0 && P > 0, "qk_rope_store: bad sizes");
+    QE_REQUIRE(qe_qk_rope_store_parts_supported(D, table ? rotary_dim : 0),
+               "qk_rope_store: partial products need a head size 8 * 2^k and a rotation over the whole head");
+    QE_REQUIRE(!table || positions, "qk_rope_store: a rotation needs positions");
+    QE_REQUIRE(!slot || cache, "qk_rope_store: slots without a cache");
+    QE_REQUIRE(q_out, "qk_rope_store: no output");
+    if (T == 0) return 0;
+    const long stride = (long)T * (Hq + 2 * Hkv) * D;
+    const int passes = qe_cdiv((Hq + Hkv) * (D / 8), 256);      // rounds of 256 lanes over the q and k heads of a token
+    const dim3 grid((unsigned)T, (unsigned)(passes < 4 ? passes : 4));
+    qk_rope_store_vec_kernel<bf16_t><<<grid, 256, (size_t)D * (16 * 2 + 16), stream>>>(
+        QkvSource<bf16_t>{nullptr, parts, bias, S, stride}, positions, q_w, k_w, eps, table, slot,
+        (bf16_t*)cache, (bf16_t*)q_out, nullptr, Hq, Hkv, D, P);
     QE_LAUNCH_CHECK();
     return 0;
 }

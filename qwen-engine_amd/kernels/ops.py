@@ -61,6 +61,9 @@ def load_library():
         "qe_attention_decode_fused_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, f32, vp,
                                           i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
         "qe_qk_rope_store": [vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
+        "qe_qk_rope_store_parts": [vp, i32, vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, vp],
+        "qe_qk_rope_store_parts_supported": [i32, i32],
+        "qe_gemm_partial_preferred": [i32, i32, i32, i32, i32],
         "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
         "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
         "qe_sample": [vp, vp, vp, vp, i32, i32, vp],
@@ -367,6 +370,60 @@ def qk_rope_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
                                 _ptr(q_out), _ptr(packed_out), T, num_heads, num_kv_heads, head_dim,
                                 page_size, _DT[qkv.dtype], _stream()), "qk_rope_store")
     return packed_out if packed else q_out
+
+
+def gemm_partial_preferred(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """True if the product of these operands is quickest cut along K into partial products
+    (EPI_PARTIAL): more than 16 and at most 64 rows against a matrix of 16 M elements or more."""
+    lib = load_library()
+    return bool(lib.qe_gemm_partial_preferred(x.shape[0], w.shape[0], x.shape[1], _DT[x.dtype], _DT[w.dtype]))
+
+
+def qk_rope_store_parts_supported(head_dim: int, table: Optional[torch.Tensor]) -> bool:
+    """True if qk_rope_store_parts takes this head size and rotation table."""
+    lib = load_library()
+    return bool(lib.qe_qk_rope_store_parts_supported(int(head_dim), 0 if table is None else table.shape[1]))
+
+
+def qk_rope_store_parts(parts: torch.Tensor, bias: Optional[torch.Tensor], num_heads: int, num_kv_heads: int,
+                        head_dim: int, positions: Optional[torch.Tensor], q_weight: Optional[torch.Tensor],
+                        k_weight: Optional[torch.Tensor], eps: float, table: Optional[torch.Tensor],
+                        slots: Optional[torch.Tensor], cache: Optional[torch.Tensor], page_size: int) -> torch.Tensor:
+    """qk_rope_store on a projection that comes as float32 partial products [S, T, (Hq + 2 Hkv) D]
+    (gemm with EPI_PARTIAL): they are added in the order of S, with ``bias`` [width] if given, and
+    rounded to bfloat16 before the norm, as the product would have stored them.  Returns q
+    [T, Hq, D] bfloat16; cache: one layer's bfloat16 pages."""
+    lib = load_library()
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _need(parts, "parts", torch.float32, (None, None, width))
+    S, T, dev = parts.shape[0], parts.shape[1], parts.device
+    if not qk_rope_store_parts_supported(head_dim, table):
+        raise KernelError("qk_rope_store_parts: head size or rotation not taken")
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (width,), dev)
+    if positions is not None:
+        _need(positions, "positions", torch.int32, (T,), dev)
+    if (q_weight is None) != (k_weight is None):
+        raise KernelError("qk_rope_store_parts: q and k norm weights come together")
+    if q_weight is not None:
+        _need(q_weight, "q_weight", torch.float32, (head_dim,), dev)
+        _need(k_weight, "k_weight", torch.float32, (head_dim,), dev)
+    rotary_dim = 0
+    if table is not None:
+        _need(table, "table", torch.float32, (None, head_dim), dev)
+        rotary_dim = head_dim
+        if positions is None:
+            raise KernelError("qk_rope_store_parts: a rotation needs positions")
+    if slots is not None:
+        _need(slots, "slots", torch.int32, (T,), dev)
+        if cache is None:
+            raise KernelError("qk_rope_store_parts: slots without a cache")
+        _need(cache, "cache", torch.bfloat16, (None, 2, num_kv_heads, page_size, head_dim), dev)
+    q_out = torch.empty((T, num_heads, head_dim), dtype=torch.bfloat16, device=dev)
+    _check(lib.qe_qk_rope_store_parts(parts.data_ptr(), S, _ptr(bias), _ptr(positions), _ptr(q_weight), _ptr(k_weight),
+                                      float(eps), _ptr(table), rotary_dim, _ptr(slots), _ptr(cache), q_out.data_ptr(),
+                                      T, num_heads, num_kv_heads, head_dim, page_size, _stream()), "qk_rope_store_parts")
+    return q_out
 
 
 def attention_decode_supported(q: torch.Tensor, cache: torch.Tensor) -> bool:

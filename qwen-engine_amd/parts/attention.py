@@ -106,6 +106,15 @@ class PagedAttention:
             q = ops.gemm_qkv(x, self.w_qkv, self.b_qkv, self.hq, cache, ctx.positions if table is not None else None,
                              self.q_norm, self.k_norm, eps, table, slots)
             return self._attend(q, ctx, cache, g, T)
+        if (fused_position and cache.dtype == torch.bfloat16 and ops.gemm_partial_preferred(x, self.w_qkv) and
+                ops.qk_rope_store_parts_supported(self.d, table)):
+            # 17 to 64 rows against a large matrix: the product is cut along K to fill the chip, and
+            # the kernel that norms, rotates and writes the cache adds the parts up as it reads them
+            parts = ops.gemm(x, self.w_qkv, epilogue=ops.EPI_PARTIAL)
+            q = ops.qk_rope_store_parts(parts, self.b_qkv, self.hq, self.hkv, self.d,
+                                        ctx.positions if table is not None else None, self.q_norm, self.k_norm,
+                                        eps, table, slots, cache, ctx.page_size)
+            return self._attend(q, ctx, cache, g, T)
         qkv = ops.gemm(x, self.w_qkv, self.b_qkv)
         if fused_position:
             only_new_tokens = (ctx.dec_tokens is not None and ctx.dec_tokens.shape[0] == T and

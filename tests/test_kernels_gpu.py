@@ -291,6 +291,45 @@ def test_qk_norm_rope_store_of_many_tokens(ops, dtype, hq, hkv, d, page):
     assert torch.equal(cache[:, 1].float().cpu(), want[:, 1].to(dtype).float())      # values are copied exactly
 
 
+@pytest.mark.parametrize("hq,hkv,d,page", [(6, 2, 128, 16), (5, 3, 64, 32), (4, 1, 16, 16)])
+@pytest.mark.parametrize("norm,rope,bias", [(True, True, False), (False, True, True), (True, False, True)])
+def test_norm_rotation_and_cache_write_from_partial_products(ops, hq, hkv, d, page, norm, rope, bias):
+    """The projection as three 32-bit partial products (+ bias): the kernel adds them in order, rounds
+    to bfloat16 and goes on as on a stored projection, to the bit.  Tokens in runs of 16 side by
+    side in a page (values written by tiles), a run across a page's edge, scattered slots, a token
+    without a slot."""
+    bf = torch.bfloat16
+    width, T, eps = (hq + 2 * hkv) * d, 260, 1e-6
+    parts = torch.stack([rand(T, width, seed=610 + i, scale=0.6) for i in range(3)])
+    b = rand(width, seed=613) if bias else None
+    summed = parts[0] + parts[1] + parts[2]
+    qkv = (summed + b if bias else summed).to(bf)
+    qw = 1 + rand(d, seed=614, scale=0.1) if norm else None
+    kw = 1 + rand(d, seed=615, scale=0.1) if norm else None
+    table = P.rope_table(10000.0, d, 600) if rope else None
+    pages = 40
+    g = torch.Generator().manual_seed(616)
+    second = (3 * page + 200 + page - 1) // page * page + page + page // 2
+    slots = list(range(3 * page, 3 * page + 200)) + [second + i for i in range(28)]   # 200 in a row, 28 from the middle of a page
+    free = [s_ for s_ in torch.randperm(pages * page, generator=g).tolist() if s_ not in set(slots)]
+    slots += free[:T - len(slots)]
+    slots[100] = -1
+    positions = torch.randint(0, 600, (T,), generator=g).to(torch.int32)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    dev = lambda t: None if t is None else t.to(DEV)
+    caches = [torch.full((pages, 2, hkv, page, d), 7.0, dtype=bf, device=DEV) for _ in range(2)]
+    assert ops.qk_rope_store_parts_supported(d, dev(table))
+    q1 = ops.qk_rope_store_parts(parts.to(DEV), dev(b), hq, hkv, d, positions.to(DEV) if rope else None, dev(qw), dev(kw),
+                                 eps, dev(table), i32(slots), caches[0], page)
+    q2 = ops.qk_rope_store(qkv.to(DEV), hq, hkv, d, positions.to(DEV) if rope else None, dev(qw), dev(kw), eps, dev(table),
+                           i32(slots), caches[1], page)
+    assert torch.equal(q1, q2) and torch.equal(caches[0], caches[1])
+    assert not torch.equal(caches[0], torch.full_like(caches[0], 7.0))
+    # a rotation over part of the head is not taken
+    if rope and d >= 32:
+        assert not ops.qk_rope_store_parts_supported(d, P.rope_table(10000.0, d // 2, 10))
+
+
 @pytest.mark.parametrize("hq,hkv,page,K", [(16, 8, 16, 1024), (3, 2, 32, 96), (5, 1, 16, 160)])
 @pytest.mark.parametrize("norm,rope,bias", [(True, True, False), (False, True, True), (True, False, False),
                                             (False, False, False)])
