@@ -92,8 +92,9 @@ __global__ __launch_bounds__(64) void qk_rope_store_kernel(
 // on those tokens' values: each takes some of the key/value heads, reads the 16 tokens' values
 // of that head, turns them round in shared memory and writes, per feature, the run of 16
 // elements that are neighbours in the tile.  That needs the 16 tokens to lie side by side in
-// one page (consecutive slots), which is how the tokens of a prompt lie; a block of tokens that
-// do not is written element by element.
+// one page (consecutive slots), which is how the tokens of a prompt lie; where they do not
+// (single new tokens of several requests), every block writes its own token's values element by
+// element.
 //
 // The projection can also come as 32-bit partial products [S][T][width] of a product that was cut
 // along K (few rows against a large matrix: the cut fills the chip): they are added here in the
