@@ -314,6 +314,40 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
         // 4 j .. 4 j + 3 and 64 + 4 j .. 64 + 4 j + 3, the two halves that rotate together.
         constexpr int TROW = BN * 2 + 16;                  // bytes of a row of the tile
         static_assert(BM * TROW <= 2 * BUF && BN % 128 == 0, "the tile must fit the staging buffers, in whole heads");
+        // positions and slots of the tile's rows, once, into shared memory behind the tile
+        int* pos_sh = (int*)(smem + BM * TROW);
+        int* slot_sh = pos_sh + BM;
+        static_assert(BM * TROW + 2 * BM * 4 <= 2 * BUF, "the rows' positions and slots must fit too");
+        if (tid < BM) { pos_sh[tid] = my_pos; slot_sh[tid] = my_slot; }
+        __syncthreads();
+        const int D = 128, half = 64;
+        const int j16 = tid % 16;
+        const long page_stride = 2L * tail.Hkv * tail.P * D;
+        constexpr int GROUPS = 64 * NW / 16, ITEMS = BM * (BN / 128);
+        constexpr int NIT = (ITEMS + GROUPS - 1) / GROUPS;         // items a group of 16 lanes takes, one after the other
+        constexpr int CHUNK = NIT < 8 ? NIT : 8;
+        // The only loads from memory in the items' loop are the table's rows, and an item is short
+        // beside a trip to memory: the rows of eight items are asked for at once, the first eight
+        // before the tile is written to shared memory.
+        float c[CHUNK][4], sn[CHUNK][4];
+#define LOAD_TABLE_ROWS(it0_)                                                            \
+        _Pragma("unroll") for (int k = 0; k < CHUNK; ++k) {                              \
+            const int idx = tid / 16 + ((it0_) + k) * GROUPS;                            \
+            _Pragma("unroll") for (int e = 0; e < 4; ++e) { c[k][e] = 1.f; sn[k][e] = 0.f; } \
+            if (tail.table && idx < ITEMS) {                                             \
+                const float* cs = tail.table + (long)pos_sh[idx % BM] * D;               \
+                Vec4<float>::load(cs + 4 * j16, c[k]);                                   \
+                Vec4<float>::load(cs + half + 4 * j16, sn[k]);                           \
+            }                                                                            \
+        }
+        LOAD_TABLE_ROWS(0)
+        float wq_a[4], wq_b[4], wk_a[4], wk_b[4];
+        if (tail.q_w) {
+            Vec4<float>::load(tail.q_w + 4 * j16, wq_a);
+            Vec4<float>::load(tail.q_w + half + 4 * j16, wq_b);
+            Vec4<float>::load(tail.k_w + 4 * j16, wk_a);
+            Vec4<float>::load(tail.k_w + half + 4 * j16, wk_b);
+        }
 #pragma unroll
         for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -330,80 +364,52 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
                     }
                     Vec4<bf16_t>::store((bf16_t*)(smem + (wm + i * 32 + (lane & 31)) * TROW) + nl, v);
                 }
-        // positions and slots of the tile's rows, once, into shared memory behind the tile
-        int* pos_sh = (int*)(smem + BM * TROW);
-        int* slot_sh = pos_sh + BM;
-        static_assert(BM * TROW + 2 * BM * 4 <= 2 * BUF, "the rows' positions and slots must fit too");
-        if (tid < BM) { pos_sh[tid] = my_pos; slot_sh[tid] = my_slot; }
         __syncthreads();
-        const int D = 128, half = 64;
-        const int j16 = tid % 16;
-        const long page_stride = 2L * tail.Hkv * tail.P * D;
-        constexpr int GROUPS = 64 * NW / 16, ITEMS = BM * (BN / 128);
-        // (the only loads from memory in the loop are the table's rows: an item's row is fetched
-        // while the item before it is computed)
-        float c[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f};
-        {
-            const int idx = tid / 16;
-            if (tail.table && idx < ITEMS) {
-                const float* cs = tail.table + (long)pos_sh[idx % BM] * D;
-                Vec4<float>::load(cs + 4 * j16, c);
-                Vec4<float>::load(cs + half + 4 * j16, sn);
-            }
-        }
-        float wq_a[4], wq_b[4], wk_a[4], wk_b[4];
-        if (tail.q_w) {
-            Vec4<float>::load(tail.q_w + 4 * j16, wq_a);
-            Vec4<float>::load(tail.q_w + half + 4 * j16, wq_b);
-            Vec4<float>::load(tail.k_w + 4 * j16, wk_a);
-            Vec4<float>::load(tail.k_w + half + 4 * j16, wk_b);
-        }
-        for (int idx = tid / 16; idx < ITEMS; idx += GROUPS) {
-            const int hd = idx / BM, row = idx % BM;
-            const int m = m0 + row, head = n0 / 128 + hd;
-            float c_next[4] = {1.f, 1.f, 1.f, 1.f}, sn_next[4] = {0.f, 0.f, 0.f, 0.f};
-            if (tail.table && idx + GROUPS < ITEMS) {
-                const float* cs = tail.table + (long)pos_sh[(idx + GROUPS) % BM] * D;
-                Vec4<float>::load(cs + 4 * j16, c_next);
-                Vec4<float>::load(cs + half + 4 * j16, sn_next);
-            }
-            if (m < M && head < tail.Hq + tail.Hkv) {                   // (values: below, by tiles)
-                const bool is_q = head < tail.Hq;
-                const bf16_t* src = (const bf16_t*)(smem + row * TROW) + hd * 128;
-                float a[4], b[4];
-                Vec4<bf16_t>::load(src + 4 * j16, a);
-                Vec4<bf16_t>::load(src + half + 4 * j16, b);
-                if (tail.q_w) {
-                    float ss = 0.f;
+        for (int it0 = 0; it0 < NIT; it0 += CHUNK) {
+            if (it0 > 0) { LOAD_TABLE_ROWS(it0) }
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) ss += a[e] * a[e] + b[e] * b[e];
-                    for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-                    const float rstd = rsqrtf(ss / (float)D + tail.eps);
+            for (int k = 0; k < CHUNK; ++k) {
+                const int idx = tid / 16 + (it0 + k) * GROUPS;
+                if (idx >= ITEMS) continue;
+                const int hd = idx / BM, row = idx % BM;
+                const int m = m0 + row, head = n0 / 128 + hd;
+                if (m < M && head < tail.Hq + tail.Hkv) {                   // (values: below, by tiles)
+                    const bool is_q = head < tail.Hq;
+                    const bf16_t* src = (const bf16_t*)(smem + row * TROW) + hd * 128;
+                    float a[4], b[4];
+                    Vec4<bf16_t>::load(src + 4 * j16, a);
+                    Vec4<bf16_t>::load(src + half + 4 * j16, b);
+                    if (tail.q_w) {
+                        float ss = 0.f;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        a[e] = a[e] * rstd * (is_q ? wq_a[e] : wk_a[e]);
-                        b[e] = b[e] * rstd * (is_q ? wq_b[e] : wk_b[e]);
+                        for (int e = 0; e < 4; ++e) ss += a[e] * a[e] + b[e] * b[e];
+                        for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+                        const float rstd = rsqrtf(ss / (float)D + tail.eps);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            a[e] = a[e] * rstd * (is_q ? wq_a[e] : wk_a[e]);
+                            b[e] = b[e] * rstd * (is_q ? wq_b[e] : wk_b[e]);
+                        }
+                    }
+                    if (tail.table) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) rotate_pair(c[k][e], sn[k][e], a[e], b[e]);
+                    }
+                    bf16_t* dst = nullptr;
+                    if (is_q) {
+                        dst = tail.q_out + ((long)m * tail.Hq + head) * D;
+                    } else {
+                        const int sl = slot_sh[row];
+                        if (sl >= 0) dst = tail.cache + (long)(sl / tail.P) * page_stride + ((long)(head - tail.Hq) * tail.P + sl % tail.P) * D;
+                    }
+                    if (dst) {
+                        Vec4<bf16_t>::store(dst + 4 * j16, a);
+                        Vec4<bf16_t>::store(dst + half + 4 * j16, b);
                     }
                 }
-                if (tail.table) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) rotate_pair(c[e], sn[e], a[e], b[e]);
-                }
-                bf16_t* dst = nullptr;
-                if (is_q) {
-                    dst = tail.q_out + ((long)m * tail.Hq + head) * D;
-                } else {
-                    const int sl = slot_sh[row];
-                    if (sl >= 0) dst = tail.cache + (long)(sl / tail.P) * page_stride + ((long)(head - tail.Hq) * tail.P + sl % tail.P) * D;
-                }
-                if (dst) {
-                    Vec4<bf16_t>::store(dst + 4 * j16, a);
-                    Vec4<bf16_t>::store(dst + half + 4 * j16, b);
-                }
             }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { c[e] = c_next[e]; sn[e] = sn_next[e]; }
         }
+#undef LOAD_TABLE_ROWS
         // values: 16 tokens of a head at a time; where their slots lie side by side in one page,
         // 8 tokens of a feature are one 16-byte store into the transposed value tile [D][P]
         for (int hd = 0; hd < BN / 128; ++hd) {
