@@ -49,6 +49,7 @@ struct QkvTail {
     bf16_t* cache;
     float eps;
     int Hq, Hkv, P;
+    int lp;   // log2 P: the page size is a power of two, and a division by a number known only at run time costs dozens of instructions an item
 };
 
 // BIG (256 x 256 by four waves, one wave a SIMD, a wave's part 128 x 128): the accumulators fill the
@@ -400,7 +401,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
                         dst = tail.q_out + ((long)m * tail.Hq + head) * D;
                     } else {
                         const int sl = slot_sh[row];
-                        if (sl >= 0) dst = tail.cache + (long)(sl / tail.P) * page_stride + ((long)(head - tail.Hq) * tail.P + sl % tail.P) * D;
+                        if (sl >= 0) dst = tail.cache + (long)(sl >> tail.lp) * page_stride + ((long)(head - tail.Hq) * tail.P + (sl & (tail.P - 1))) * D;
                     }
                     if (dst) {
                         Vec4<bf16_t>::store(dst + 4 * j16, a);
@@ -419,7 +420,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
                 const int r0 = idx / (D * 2) * 16, d = idx % (D * 2) / 2, h = idx % 2;
                 if (m0 + r0 >= M) continue;
                 const int s0 = slot_sh[r0];
-                bool run = m0 + r0 + 16 <= M && s0 >= 0 && s0 % tail.P + 16 <= tail.P && (s0 % tail.P) % 8 == 0;
+                bool run = m0 + r0 + 16 <= M && s0 >= 0 && (s0 & (tail.P - 1)) + 16 <= tail.P && (s0 & 7) == 0;
 #pragma unroll
                 for (int i = 1; i < 16; ++i) run = run && slot_sh[r0 + i] == s0 + i;
                 if (run) {
@@ -427,14 +428,14 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
                         pc8.e[e] = *(const unsigned short*)(smem + (r0 + 8 * h + e) * TROW + (hd * 128 + d) * 2);
-                    bf16_t* vt = tail.cache + (long)(s0 / tail.P) * page_stride + ((long)(tail.Hkv + kh) * tail.P) * D + s0 % tail.P;
+                    bf16_t* vt = tail.cache + (long)(s0 >> tail.lp) * page_stride + ((long)(tail.Hkv + kh) * tail.P) * D + (s0 & (tail.P - 1));
                     *(uint4_t*)(vt + (long)d * tail.P + 8 * h) = pc8.q;
                 } else {
                     for (int e = 0; e < 8; ++e) {
                         const int i = 8 * h + e;
                         const int si = m0 + r0 + i < M ? slot_sh[r0 + i] : -1;
                         if (si >= 0)
-                            tail.cache[(long)(si / tail.P) * page_stride + ((long)(tail.Hkv + kh) * tail.P) * D + (long)d * tail.P + si % tail.P] =
+                            tail.cache[(long)(si >> tail.lp) * page_stride + ((long)(tail.Hkv + kh) * tail.P) * D + (long)d * tail.P + (si & (tail.P - 1))] =
                                 *(const bf16_t*)(smem + (r0 + i) * TROW + (hd * 128 + d) * 2);
                     }
                 }
@@ -602,7 +603,9 @@ int qe_gemm_qkv(const void* x, const void* w, const float* bias, int M, int K, i
     QE_REQUIRE(M > 16 && Hq > 0 && Hkv > 0 && P >= 16 && (P & (P - 1)) == 0, "qkv gemm: sizes not taken");
     QE_REQUIRE(tile == 0 || tile == 512 || tile == 256 || tile == 128 || tile == 64, "qkv gemm: tile of %d rows", tile);
     QE_REQUIRE(!table || positions, "qkv gemm: a rotation needs positions");
-    QkvTail tail{positions, slots, q_w, k_w, table, (bf16_t*)q_out, (bf16_t*)cache, eps, Hq, Hkv, P};
+    int lp = 0;
+    while ((1 << lp) < P) ++lp;
+    QkvTail tail{positions, slots, q_w, k_w, table, (bf16_t*)q_out, (bf16_t*)cache, eps, Hq, Hkv, P, lp};
     // (the 256 x 256 shape has four waves for an epilogue over 65536 values: the others finish it sooner)
     if (tile == 0) tile = choose_tile(M, N, 1, false);
     if (tile == 512) return launch_mfma<bf16_t, 256, 256, 64, 4, 1, false, true>(x, w, bias, nullptr, M, N, K, 1, stream, tail);
