@@ -64,6 +64,7 @@ def load_library():
         "qe_qk_rope_store_parts": [vp, i32, vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, vp],
         "qe_qk_rope_store_parts_supported": [i32, i32],
         "qe_gemm_partial_preferred": [i32, i32, i32, i32, i32],
+        "qe_gemm_branch_splits": [i32, i32, i32, i32, i32],
         "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
         "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
         "qe_sample": [vp, vp, vp, vp, i32, i32, vp],
@@ -370,6 +371,16 @@ def qk_rope_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
                                 _ptr(q_out), _ptr(packed_out), T, num_heads, num_kv_heads, head_dim,
                                 page_size, _DT[qkv.dtype], _stream()), "qk_rope_store")
     return packed_out if packed else q_out
+
+
+def gemm_branch_splits(x: torch.Tensor, w: torch.Tensor) -> int:
+    """How a product whose result goes to a norm that adds it to the stream should be asked for:
+    0 = plain, S >= 1 = gemm(..., epilogue=EPI_PARTIAL, splits=S), the S partial products being
+    what that norm takes as ``delta`` (few rows; many rows against a narrow matrix with a long K)."""
+    lib = load_library()
+    if x.dtype not in _DT or w.dtype not in _DT:
+        return 0
+    return int(lib.qe_gemm_branch_splits(x.shape[0], w.shape[0], x.shape[1], _DT[x.dtype], _DT[w.dtype]))
 
 
 def gemm_partial_preferred(x: torch.Tensor, w: torch.Tensor) -> bool:

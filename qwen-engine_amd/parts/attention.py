@@ -147,9 +147,11 @@ class PagedAttention:
         return self._project_out(o.view(T, self.hq * self.d))
 
     def _project_out(self, o: torch.Tensor) -> torch.Tensor:
-        if ops.gemm_fused_supported(o, self.w_o):
-            # few rows: the product is cut along K to fill the chip; the norm that follows adds the parts
-            return ops.gemm(o, self.w_o, epilogue=ops.EPI_PARTIAL)
+        splits = ops.gemm_branch_splits(o, self.w_o)
+        if splits:
+            # the product is cut along K (few rows: to fill the chip; a narrow matrix: to give every
+            # compute unit blocks to overlap); the norm that follows adds the parts
+            return ops.gemm(o, self.w_o, epilogue=ops.EPI_PARTIAL, splits=splits)
         return ops.gemm(o, self.w_o)
 
 

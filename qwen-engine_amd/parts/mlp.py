@@ -47,8 +47,9 @@ class SwiGLU:
             a = ops.gemm(x, self.w_gu, epilogue=ops.EPI_SILU_MUL)
         else:
             a = ops.silu_mul(ops.gemm(x, self.w_gu), interleaved=self.interleaved)
-        if ops.gemm_fused_supported(a, self.w_down):
-            return ops.gemm(a, self.w_down, epilogue=ops.EPI_PARTIAL)
+        splits = ops.gemm_branch_splits(a, self.w_down)
+        if splits:   # partial products along K, added by the norm that follows
+            return ops.gemm(a, self.w_down, epilogue=ops.EPI_PARTIAL, splits=splits)
         return ops.gemm(a, self.w_down)
 
 
