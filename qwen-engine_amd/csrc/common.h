@@ -76,6 +76,19 @@ __device__ __forceinline__ float wave_sum(float v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
     return v;
 }
+// Sum over the 16 lanes of a row (lanes 16 r .. 16 r + 15), every lane getting it: the lane pairs and
+// the order are those of the butterfly `v += __shfl_xor(v, o)` for o = 8, 4, 2, 1 (a rotation by o
+// meets the same partner sums, which repeat with period 2 o), so the result is the same to the
+// bit, by four vector instructions instead of four trips through the LDS crossbar.
+__device__ __forceinline__ float row16_sum(float v) {
+#define QE_ROW_ROR(n_) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + (n_), 0xf, 0xf, false))
+    v += QE_ROW_ROR(8);
+    v += QE_ROW_ROR(4);
+    v += QE_ROW_ROR(2);
+    v += QE_ROW_ROR(1);
+#undef QE_ROW_ROR
+    return v;
+}
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));

@@ -335,7 +335,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
         _Pragma("unroll") for (int k = 0; k < CHUNK; ++k) {                              \
             const int idx = tid / 16 + ((it0_) + k) * GROUPS;                            \
             _Pragma("unroll") for (int e = 0; e < 4; ++e) { c[k][e] = 1.f; sn[k][e] = 0.f; } \
-            if (tail.table && idx < ITEMS) {                                             \
+            if (tail.table && idx < ITEMS && n0 / 128 + idx / BM < tail.Hq + tail.Hkv) {  \
                 const float* cs = tail.table + (long)pos_sh[idx % BM] * D;               \
                 Vec4<float>::load(cs + 4 * j16, c[k]);                                   \
                 Vec4<float>::load(cs + half + 4 * j16, sn[k]);                           \
@@ -384,7 +384,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
                         float ss = 0.f;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) ss += a[e] * a[e] + b[e] * b[e];
-                        for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+                        ss = row16_sum(ss);                                  // (the item's 16 lanes are a row)
                         const float rstd = rsqrtf(ss / (float)D + tail.eps);
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
@@ -412,31 +412,49 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
         }
 #undef LOAD_TABLE_ROWS
         // values: 16 tokens of a head at a time; where their slots lie side by side in one page,
-        // 8 tokens of a feature are one 16-byte store into the transposed value tile [D][P]
+        // 8 tokens of a feature are one 16-byte store into the transposed value tile [D][P].
+        // Whether 16 rows lie so is found once, by one thread a group of rows (0: no, 1: yes).
+        int* run_sh = slot_sh + BM;
+        static_assert(BM * TROW + 2 * BM * 4 + (BM / 16) * 4 <= 2 * BUF, "the groups' flags must fit too");
+        const bool has_values = tail.slots && n0 / 128 + BN / 128 > tail.Hq + tail.Hkv;   // the same for the whole block
+        if (has_values && tid < BM / 16) {
+            const int r0 = tid * 16, s0 = slot_sh[r0];
+            bool run = m0 + r0 + 16 <= M && s0 >= 0 && (s0 & (tail.P - 1)) + 16 <= tail.P && (s0 & 7) == 0;
+#pragma unroll
+            for (int i = 1; i < 16; ++i) run = run && slot_sh[r0 + i] == s0 + i;
+            run_sh[tid] = run ? 1 : 0;
+        }
+        if (has_values) __syncthreads();
         for (int hd = 0; hd < BN / 128; ++hd) {
             const int kh = n0 / 128 + hd - tail.Hq - tail.Hkv;
-            if (!tail.slots || kh < 0 || kh >= tail.Hkv) continue;      // the same for the whole block
-            for (int idx = tid; idx < (BM / 16) * D * 2; idx += 64 * NW) {   // 16 rows from r0, feature d, tokens 8 h .. 8 h + 7
-                const int r0 = idx / (D * 2) * 16, d = idx % (D * 2) / 2, h = idx % 2;
+            if (!has_values || kh < 0 || kh >= tail.Hkv) continue;      // the same for the whole block
+            // a thread: 16 rows from r0, the features d and d + 1, the tokens 8 h .. 8 h + 7 (two
+            // features at a time: half the reads from shared memory)
+            for (int idx = tid; idx < (BM / 16) * D; idx += 64 * NW) {
+                const int r0 = idx / D * 16, d = idx % D / 2 * 2, h = idx % 2;
                 if (m0 + r0 >= M) continue;
-                const int s0 = slot_sh[r0];
-                bool run = m0 + r0 + 16 <= M && s0 >= 0 && (s0 & (tail.P - 1)) + 16 <= tail.P && (s0 & 7) == 0;
+                if (run_sh[r0 / 16]) {
+                    const int s0 = slot_sh[r0];
+                    Piece16 lo, hi;
 #pragma unroll
-                for (int i = 1; i < 16; ++i) run = run && slot_sh[r0 + i] == s0 + i;
-                if (run) {
-                    Piece16 pc8;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        pc8.e[e] = *(const unsigned short*)(smem + (r0 + 8 * h + e) * TROW + (hd * 128 + d) * 2);
+                    for (int e = 0; e < 8; ++e) {
+                        const unsigned two = *(const unsigned*)(smem + (r0 + 8 * h + e) * TROW + (hd * 128 + d) * 2);
+                        lo.e[e] = (unsigned short)(two & 0xffffu);
+                        hi.e[e] = (unsigned short)(two >> 16);
+                    }
                     bf16_t* vt = tail.cache + (long)(s0 >> tail.lp) * page_stride + ((long)(tail.Hkv + kh) * tail.P) * D + (s0 & (tail.P - 1));
-                    *(uint4_t*)(vt + (long)d * tail.P + 8 * h) = pc8.q;
+                    *(uint4_t*)(vt + (long)d * tail.P + 8 * h) = lo.q;
+                    *(uint4_t*)(vt + (long)(d + 1) * tail.P + 8 * h) = hi.q;
                 } else {
                     for (int e = 0; e < 8; ++e) {
                         const int i = 8 * h + e;
                         const int si = m0 + r0 + i < M ? slot_sh[r0 + i] : -1;
-                        if (si >= 0)
-                            tail.cache[(long)(si >> tail.lp) * page_stride + ((long)(tail.Hkv + kh) * tail.P) * D + (long)d * tail.P + (si & (tail.P - 1))] =
-                                *(const bf16_t*)(smem + (r0 + i) * TROW + (hd * 128 + d) * 2);
+                        if (si >= 0) {
+                            bf16_t* to = tail.cache + (long)(si >> tail.lp) * page_stride + ((long)(tail.Hkv + kh) * tail.P) * D + (si & (tail.P - 1));
+                            const bf16_t* from = (const bf16_t*)(smem + (r0 + i) * TROW + (hd * 128 + d) * 2);
+                            to[(long)d * tail.P] = from[0];
+                            to[(long)(d + 1) * tail.P] = from[1];
+                        }
                     }
                 }
             }

@@ -198,7 +198,8 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
             float ss = 0.f;
 #pragma unroll
             for (int e = 0; e < 4; ++e) ss += a[e] * a[e] + b[e] * b[e];
-            for (int o = lph >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            if (lph == 16) ss = row16_sum(ss);             // (the same sum, without the LDS crossbar)
+            else for (int o = lph >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
             const float rstd = rsqrtf(ss / (float)D + eps);
             float wa[4], wb[4];
             Vec4<float>::load(w + 4 * j, wa);
