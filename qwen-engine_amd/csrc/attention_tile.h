@@ -38,6 +38,16 @@ __device__ __forceinline__ void load_tile(KVTile<D>& tile, const bf16_t* __restr
     for (int db = 0; db < D / 16; ++db) tile.v[db] = *(const short4_t*)(vbase + (long)db * 16 * P);
 }
 
+// The largest of the four lanes n, n + 16, n + 32, n + 48 (the four rows of 16 lanes), in all of them:
+// two swaps between vector registers (rows 1, 3 against rows 0, 2, then the halves of the wave)
+// where `__shfl_xor` would go twice through the LDS crossbar, once per tile of every wave.
+__device__ __forceinline__ float max_over_lane_rows(float v) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
 template <int D>
 struct AttnState {
     float m, l;              // running max and (this lane's share of the) running sum of column n
@@ -67,8 +77,7 @@ __device__ __forceinline__ void attn_tile_step(AttnState<D>& st, const KVTile<D>
         s[j] = ok[j] ? s[j] * scale : -INFINITY;
         tmax = fmaxf(tmax, s[j]);
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    tmax = max_over_lane_rows(tmax);
     const float mn = fmaxf(st.m, tmax);
     const float ref = (mn == -INFINITY) ? 0.f : mn;   // a column that has seen no key yet: all weights 0
     const float alpha = __expf(st.m - ref);
