@@ -47,12 +47,14 @@ union Piece {   // a staged 16-byte piece, addressable by element for masking
 
 // Lane i and lane i ^ 32 exchange a value without a trip through shared memory.
 __device__ __forceinline__ float max_of_both_halves(float v) {
-    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    float a, b;
+    pair_across_halves(v, a, b);
+    return fmaxf(a, b);
 }
 __device__ __forceinline__ float sum_of_both_halves(float v) {
-    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+    float a, b;
+    pair_across_halves(v, a, b);
+    return a + b;
 }
 
 #define VROW 48   // bytes of a staged value row: 16 keys = 32 bytes of data + 16 of padding

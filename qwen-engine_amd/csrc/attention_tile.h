@@ -42,10 +42,11 @@ __device__ __forceinline__ void load_tile(KVTile<D>& tile, const bf16_t* __restr
 // two swaps between vector registers (rows 1, 3 against rows 0, 2, then the halves of the wave)
 // where `__shfl_xor` would go twice through the LDS crossbar, once per tile of every wave.
 __device__ __forceinline__ float max_over_lane_rows(float v) {
-    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
-    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+    float a, b;
+    pair_across_rows(v, a, b);
+    v = fmaxf(a, b);
+    pair_across_halves(v, a, b);
+    return fmaxf(a, b);
 }
 
 template <int D>

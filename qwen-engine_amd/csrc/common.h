@@ -71,11 +71,25 @@ template <> struct Vec4<bf16_t> {
     }
 };
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+// v of this lane and of its partner across the wave's halves (lane ^ 32) or across odd and even
+// rows of 16 lanes (lane ^ 16), by a swap between two vector registers.  (The two results are
+// taken out of the returned pair into plain integers first: a bit cast applied to an element of
+// the pair gave the first element for both.)
+__device__ __forceinline__ void pair_across_halves(float v, float& mine, float& other) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const unsigned r0 = r[0], r1 = r[1];
+    mine = __uint_as_float(r0);
+    other = __uint_as_float(r1);
 }
+__device__ __forceinline__ void pair_across_rows(float v, float& mine, float& other) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const unsigned r0 = r[0], r1 = r[1];
+    mine = __uint_as_float(r0);
+    other = __uint_as_float(r1);
+}
+// (mine and other are this lane's and its partner's value in one order or the other, depending on
+// the lane's half or row: sums and maxima do not care)
+
 // Sum over the 16 lanes of a row (lanes 16 r .. 16 r + 15), every lane getting it: the lane pairs and
 // the order are those of the butterfly `v += __shfl_xor(v, o)` for o = 8, 4, 2, 1 (a rotation by o
 // meets the same partner sums, which repeat with period 2 o), so the result is the same to the
@@ -89,9 +103,32 @@ __device__ __forceinline__ float row16_sum(float v) {
 #undef QE_ROW_ROR
     return v;
 }
+// Sum and maximum over the 64 lanes of a wave, in every lane.  The partners and the order are those
+// of the butterfly `v += __shfl_xor(v, o)` for o = 32, 16, 8, 4, 2, 1, so the sum is the same to the
+// bit; but the halves of the wave and the odd and even rows of 16 lanes are exchanged by register
+// swaps and the lanes of a row by rotations, where each `__shfl_xor` is a trip through the LDS
+// crossbar of about 120 cycles that the next has to wait for.
+__device__ __forceinline__ float wave_sum(float v) {
+    float a, b;
+    pair_across_halves(v, a, b);
+    v = a + b;
+    pair_across_rows(v, a, b);
+    v = a + b;
+    return row16_sum(v);
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    float a, b;
+    pair_across_halves(v, a, b);
+    v = fmaxf(a, b);
+    pair_across_rows(v, a, b);
+    v = fmaxf(a, b);
+    // (a lane whose partner is switched off gets its own value back: neutral for a maximum, as the 0 above is for a sum)
+#define QE_ROW_ROR(n_) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x120 + (n_), 0xf, 0xf, false))
+    v = fmaxf(v, QE_ROW_ROR(8));
+    v = fmaxf(v, QE_ROW_ROR(4));
+    v = fmaxf(v, QE_ROW_ROR(2));
+    v = fmaxf(v, QE_ROW_ROR(1));
+#undef QE_ROW_ROR
     return v;
 }
 
