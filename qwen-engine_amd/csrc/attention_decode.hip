@@ -324,9 +324,11 @@ __global__ __launch_bounds__(256) void attention_decode_merge_kernel(
     const int di = blockIdx.x, head = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* pml = part_ml + ((long)di * Hq + head) * num_splits * 2;
     const float* pacc = part_acc + ((long)di * Hq + head) * num_splits * D;
+    // (the largest maximum is reduced only after the first eight splits' loads have been issued: its
+    // own loads were issued before them, so waiting for those does not wait for these)
     float M = -INFINITY;
     for (int s = lane; s < num_splits; s += 64) M = fmaxf(M, pml[2 * s]);
-    M = wave_max(M);
+    bool reduced = false;
     float denom = 0.f;
     float o[PER];
 #pragma unroll
@@ -347,10 +349,12 @@ __global__ __launch_bounds__(256) void attention_decode_merge_kernel(
 #pragma unroll
             for (int i = 0; i < PER; ++i) {
                 const int d = lane + i * 64;
-                // an empty split's accumulator was never written: not read
-                a[k][i] = (ms[k] != -INFINITY && d < D) ? pacc[(long)s * D + d] : 0.f;
+                // (asked for without waiting for the maxima: an empty split's accumulator was never
+                // written, and what is read of it is not used below; a split beyond the last reads the last)
+                a[k][i] = d < D ? pacc[(long)(s < num_splits ? s : num_splits - 1) * D + d] : 0.f;
             }
         }
+        if (!reduced) { M = wave_max(M); reduced = true; }
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             if (ms[k] == -INFINITY) continue;
