@@ -86,8 +86,29 @@ def library_file() -> str:
     return str(_build.library_path(verbose=False))
 
 
+_fixed_stream: Optional[int] = None
+
+
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    return _fixed_stream if _fixed_stream is not None else torch.cuda.current_stream().cuda_stream
+
+
+class one_stream:
+    """Within this scope every kernel goes to the stream that is current on entry: asking torch
+    for the current stream costs several microseconds a call, and a step of the model makes a
+    few hundred calls on one stream.  (Entered inside whatever stream or graph-capture context the
+    caller has set up; scopes nest.)"""
+
+    def __enter__(self):
+        global _fixed_stream
+        self._outer = _fixed_stream
+        _fixed_stream = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        global _fixed_stream
+        _fixed_stream = self._outer
+        return False
 
 
 def _check(rc: int, what: str) -> None:

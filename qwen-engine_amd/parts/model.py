@@ -95,12 +95,13 @@ class DecoderModel:
 
     def forward(self, ctx, bindings: List[CacheBinding]) -> torch.Tensor:
         """Runs the tokens of ctx through the schedule; returns float32 logits [R, V]."""
-        h = ops.embedding(ctx.token_ids, self.embed)
-        pending = None
-        for i, entry in enumerate(self.spec.schedule):
-            pending = self.blocks[entry.layer].forward(h, pending, ctx, bindings[i])
-        R = ctx.logit_rows.shape[0]
-        if R == 0:
-            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=h.device)
-        x = self.final_norm.forward(h, ctx.rt, delta=pending, rows=ctx.logit_rows)
-        return ops.gemm(x, self.head, out_dtype=torch.float32)
+        with ops.one_stream():           # (the whole step runs on the stream that is current now)
+            h = ops.embedding(ctx.token_ids, self.embed)
+            pending = None
+            for i, entry in enumerate(self.spec.schedule):
+                pending = self.blocks[entry.layer].forward(h, pending, ctx, bindings[i])
+            R = ctx.logit_rows.shape[0]
+            if R == 0:
+                return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=h.device)
+            x = self.final_norm.forward(h, ctx.rt, delta=pending, rows=ctx.logit_rows)
+            return ops.gemm(x, self.head, out_dtype=torch.float32)
