@@ -275,4 +275,13 @@ def test_random_engine_sizes_and_prompt_sets(folders, which):
         assert all(cache.available(g) == pool.num_pages for g, pool in enumerate(cache.pools)), (seed, sizes)
         preempted += eng.stats()["preemptions"] > 0
         shared += eng.stats()["shared_prefix_tokens"] > 0
+        if seed < 8:
+            # temperature sampling with a seed: the same tokens as an engine with room for everything
+            both = []
+            for cfg_sizes in (sizes, dict(dtype="float32", block_size=8, max_num_seqs=len(prompts), max_model_len=longest + 8)):
+                e2 = LLMEngine.from_folder(folders[which], EngineConfig(**cfg_sizes))
+                e2.submit(prompts, max_new_tokens=new, temperature=0.9, seed=5, ignore_eos=True)
+                both.append([r.token_ids for r in e2.run()])
+                e2.runner.cache.check_invariants()
+            assert both[0] == both[1], (seed, sizes)
     assert preempted >= 2 and shared >= 5          # the draws reach both
