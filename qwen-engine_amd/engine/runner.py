@@ -348,7 +348,6 @@ class ModelRunner:
             positions = np.concatenate([positions, np.zeros(fill, dtype=i32)])
             tok_seq = np.concatenate([tok_seq, np.full(fill, tok_seq[0], dtype=i32)])
             slots = [np.concatenate([x, np.full(fill, -1, dtype=i32)]) for x in slots]
-        state_slots = [s.state_slot for s in seqs] + [seqs[0].state_slot] * (B - n_live)
         cap = 2 * B                                    # table updates a decode step can bring per group
         splits = int(positions.max()) // ops.DECODE_SPLIT_KEYS + 1
         bucket = (splits + self.SPLIT_BUCKET - 1) // self.SPLIT_BUCKET * self.SPLIT_BUCKET
@@ -368,11 +367,12 @@ class ModelRunner:
             rec = self._record_decode_graph(B, bucket, cap)
             self.graphs_recorded += 1
         self._graphs[key] = rec                                # (re)inserted last = most recently used
-        iota = np.arange(B, dtype=i32)
-        parts = [token_ids, positions, tok_seq, iota, np.asarray(state_slots, dtype=i32), iota]
+        iota, none, zero = rec["iota"], rec["none"], rec["zero"]       # 0 .. B - 1; cap times -1; cap zeros
+        # (a row's table row is its request's state slot: tok_seq serves as both)
+        parts = [token_ids, positions, tok_seq, iota, tok_seq, iota]
         for g in range(n_groups):
             pad = cap - len(upd_idx[g])
-            parts += [slots[g], upd_idx[g], np.full(pad, -1, dtype=i32), upd_val[g], np.zeros(pad, dtype=i32)]
+            parts += [slots[g], upd_idx[g], none[:pad], upd_val[g], zero[:pad]]
         rec["event"].synchronize()                     # the last copy out of the host buffer is done
         np.concatenate(parts, out=rec["host_np"])
         rec["meta"].copy_(rec["host"], non_blocking=True)
@@ -439,4 +439,5 @@ class ModelRunner:
         event = torch.cuda.Event()
         event.record()
         return {"graph": graph, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits,
-                "event": event}
+                "event": event, "iota": np.arange(B, dtype=np.int32), "none": np.full(cap, -1, dtype=np.int32),
+                "zero": np.zeros(cap, dtype=np.int32)}
