@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 TOL = {"float32": 1e-4, "bfloat16": 2e-2}
 ACT = {"float32": None, "bfloat16": torch.bfloat16}
 LENGTHS = {"A": (70, 97, 133, 150, 41, 66), "B": (150, 65, 88, 129, 200, 77), "C": (100, 64, 131, 80, 45, 190),
-           "D": (300, 130, 257, 90, 411, 64)}
+           "D": (300, 130, 257, 90, 411, 64), "E": (350, 66, 257, 129, 480, 90)}
 
 
 def make_requests(cfg, which):
@@ -31,7 +31,7 @@ def cases(tmp_path_factory):
     """Per tiny configuration: the folder, the requests and the plain logits for both precisions."""
     tmp = tmp_path_factory.mktemp("models")
     out = {}
-    for which in "ABCD":
+    for which in "ABCDE":
         folder = make_folder(tmp, which, dtype=torch.bfloat16, std=0.05)
         cfg, w = P.read_folder(folder)
         reqs = make_requests(cfg, which)
@@ -53,25 +53,25 @@ def check(trace, case, dtype, tmp_path, which, program=False):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 def test_whole_requests(cases, tmp_path, which, dtype):
     check(traces.whole(cases[which][2]), cases[which], dtype, tmp_path, which)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 def test_last_32_tokens_one_by_one(cases, tmp_path, which, dtype):
     check(traces.tail_decoded(cases[which][2]), cases[which], dtype, tmp_path, which)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 def test_portions_of_changing_size(cases, tmp_path, which, dtype):
     check(traces.portions(cases[which][2]), cases[which], dtype, tmp_path, which)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 def test_mixed_with_pages_used_again(cases, tmp_path, which, dtype):
     trace = traces.mixed(cases[which][2], seed=7)
     assert max(len(s["entries"]) for s in trace.steps) >= 3
@@ -118,13 +118,13 @@ def test_a_step_without_wanted_logits_writes_no_file(cases, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 def test_random_traces(cases, tmp_path, which, dtype):
     """Six draws of the cutting: mixed traces with one to four live requests and 0 to 40 tokens
     decoded one by one at the end, or portions of drawn sizes; page sizes other than the usual."""
     import random
     folder, cfg, reqs, ref = cases[which]
-    pages = {"A": [4, 1, 16], "B": [8, 2], "C": [16, 32], "D": [16, 32, 64]}[which]
+    pages = {"A": [4, 1, 16], "B": [8, 2], "C": [16, 32], "D": [16, 32, 64], "E": [16, 32, 64]}[which]
     for seed in range(6):
         rng = random.Random(100 * ord(which) + seed)
         if rng.random() < 0.75:

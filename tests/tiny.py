@@ -34,7 +34,15 @@ TINY_D = dict(
     num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=2, head_dim=64,
     max_position_embeddings=1024, rms_norm_eps=1e-6, rope_theta=10000.0, tie_word_embeddings=False)
 
-TINY = {"A": (TINY_A, 0, 4), "B": (TINY_B, 1, 8), "C": (TINY_C, 2, 16), "D": (TINY_D, 3, 16)}   # config, seed, page size
+# E: head size 128, the size of the family's models: in bfloat16 the q|k|v product of a portion norms,
+# rotates and writes the cache in its epilogue, and decode steps run the kernels the large models run.
+TINY_E = dict(
+    architectures=["Qwen3ForCausalLM"], vocab_size=400, hidden_size=256, intermediate_size=320,
+    num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=128,
+    max_position_embeddings=1024, rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=False)
+
+TINY = {"A": (TINY_A, 0, 4), "B": (TINY_B, 1, 8), "C": (TINY_C, 2, 16), "D": (TINY_D, 3, 16),
+        "E": (TINY_E, 4, 16)}   # config, seed, page size
 
 
 def make_folder(tmp, which: str, dtype=torch.bfloat16, norm_std=0.01, std=0.02, scale_qk=None):
