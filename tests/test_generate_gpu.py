@@ -21,7 +21,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 @pytest.fixture(scope="module")
 def folders(tmp_path_factory):
     tmp = tmp_path_factory.mktemp("gen")
-    return {w: make_folder(tmp, w, dtype=torch.bfloat16, std=0.08) for w in "ABD"}
+    return {w: make_folder(tmp, w, dtype=torch.bfloat16, std=0.08) for w in "ABDE"}
 
 
 def prompts_for(cfg, lengths, seed):
@@ -80,17 +80,18 @@ def test_outputs_do_not_depend_on_the_engine_sizes(folders, sizes):
     assert together != want                                # and it is not greedy
 
 
+@pytest.mark.parametrize("which", ["D", "E"])
 @pytest.mark.parametrize("sizes", [dict(), dict(num_blocks=34, max_num_seqs=4), dict(max_step_tokens=48, prefill_chunk=32)])
-def test_bfloat16_generation_on_the_mfma_kernels(folders, sizes):
-    """The fourth tiny configuration (head size 64) in bfloat16: decode steps run as recorded
+def test_bfloat16_generation_on_the_mfma_kernels(folders, sizes, which):
+    """The tiny configurations with head sizes 64 and 128 in bfloat16: decode steps run as recorded
     graphs on the MFMA kernels, prompts in portions, and with few pages requests are preempted.
     Every token the engine chose must be the plain implementation's choice for the engine's own
     sequence, or within rounding of it (bfloat16 results depend on the cut in the last bits)."""
-    cfg, w = P.read_folder(folders["D"])
+    cfg, w = P.read_folder(folders[which])
     prompts = prompts_for(cfg, (150, 33, 70, 201, 16), 6)
     base = dict(dtype="bfloat16", block_size=16, max_num_seqs=3, max_model_len=320)
     base.update(sizes)
-    eng = LLMEngine.from_folder(folders["D"], EngineConfig(**base))
+    eng = LLMEngine.from_folder(folders[which], EngineConfig(**base))
     eng.submit(prompts, max_new_tokens=40, ignore_eos=True)
     res = eng.run()
     assert eng.runner.graph_steps > 0
