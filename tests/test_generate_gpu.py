@@ -124,16 +124,17 @@ def test_shared_prefix_pages_are_taken_over(folders):
     assert res[1].token_ids == P.greedy_generate(cfg, w, b, 4)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_long_decoding(folders, dtype):
+@pytest.mark.parametrize("dtype,which,page", [("float32", "A", 4), ("bfloat16", "A", 4), ("bfloat16", "E", 16), ("float32", "E", 16)])
+def test_long_decoding(folders, dtype, which, page):
     """300 tokens decoded one by one after a short prompt: logits at every decoded position equal
-    the plain implementation's on the whole sequence (pages fill and new ones are taken 75 times)."""
+    the plain implementation's on the whole sequence (pages fill and new ones are taken 75 times;
+    with heads of 128 the recorded decode step passes the ends of two splits of 128 keys)."""
     from qwen_engine_amd.engine import ModelRunner, StepEntry, load_model
-    cfg, w = P.read_folder(folders["A"])
+    cfg, w = P.read_folder(folders[which])
     toks = prompts_for(cfg, (305,), 4)[0]
     act = None if dtype == "float32" else torch.bfloat16
     ref = P.forward_logits(cfg, w, toks, act_dtype=act)
-    runner = ModelRunner(load_model(folders["A"], dtype=dtype), page_size=4, num_pages=80, max_requests=1)
+    runner = ModelRunner(load_model(folders[which], dtype=dtype), page_size=page, num_pages=80, max_requests=1)
     runner.add_request("r")
     rows = [runner.step([StepEntry("r", toks[:5], [4])])]
     for i in range(5, 305):
