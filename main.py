@@ -45,6 +45,8 @@ def parse_args(argv=None):
     ap.add_argument("--prefill-chunk", type=int, default=512, help="largest portion of a prompt in a step")
     ap.add_argument("--ignore-eos", action="store_true")
     ap.add_argument("--no-prefix-sharing", action="store_true")
+    ap.add_argument("--debug-poison", action="store_true",
+                    help="fill every cache page with NaN when it is handed out and when it goes back")
     ap.add_argument("--stats", action="store_true", help="print the engine's counters at the end")
     return ap.parse_args(argv)
 
@@ -66,7 +68,8 @@ def main(argv=None) -> int:
         dtype=args.model_dtype, block_size=args.block_size, num_blocks=args.num_blocks,
         max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len,
         max_step_tokens=args.max_step_tokens, prefill_chunk=args.prefill_chunk,
-        enable_prefix_sharing=not args.no_prefix_sharing, seed=args.seed)
+        enable_prefix_sharing=not args.no_prefix_sharing, seed=args.seed,
+        debug_poison=args.debug_poison)
     engine = LLMEngine.from_folder(args.model_name_or_path, engine_config)
 
     prompts = list(args.prompt) + [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]

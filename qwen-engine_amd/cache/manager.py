@@ -193,6 +193,10 @@ class CacheManager:
         self._kept: "OrderedDict[int, _SharedEntry]" = OrderedDict()
         self.stats = {"pages_allocated": 0, "pages_freed": 0, "shared_page_hits": 0, "kept_page_hits": 0,
                       "kept_pages_evicted": 0}
+        # with track_pages, every page that is handed out or goes back to a free list is noted as
+        # (group, page), for an owner of the storage that wants to overwrite such pages
+        self.track_pages = False
+        self._page_events: List[Tuple[int, int]] = []
 
     # ---- requests -------------------------------------------------------------
     def add_request(self, req_id: Hashable) -> RequestCache:
@@ -285,8 +289,20 @@ class CacheManager:
             for gg, page in enumerate(entry.pages):
                 self.pools[gg].give_back(page)
                 self.stats["pages_freed"] += 1
+                if self.track_pages:
+                    self._page_events.append((gg, page))
             self.stats["kept_pages_evicted"] += 1
-        return self.pools[g].allocate()
+        page = self.pools[g].allocate()
+        if self.track_pages:
+            self._page_events.append((g, page))
+        return page
+
+    def take_page_events(self) -> List[Tuple[int, int]]:
+        """(group, page) of every page handed out or given back to a free list since the last call
+        (only noted while ``track_pages`` is set).  Pages kept aside for a later request with the
+        same prefix are not among them: their contents are still wanted."""
+        out, self._page_events = self._page_events, []
+        return out
 
     def reserve(self, req_id: Hashable, new_len: int) -> None:
         """Give the request pages for every position it will hold up to new_len - 1.
@@ -337,6 +353,8 @@ class CacheManager:
     def _release(self, g: int, page: int) -> None:
         if self.pools[g].release(page):
             self.stats["pages_freed"] += 1
+            if self.track_pages:
+                self._page_events.append((g, page))
             if g == 0:
                 h = self._page_hash.pop(page, None)
                 if h is not None:
@@ -440,6 +458,8 @@ class CacheManager:
         for entry in self._kept.values():
             for g, page in enumerate(entry.pages):
                 self.pools[g].give_back(page)
+                if self.track_pages:
+                    self._page_events.append((g, page))
         self._kept.clear()
         self._shared.clear()
         self._page_hash.clear()

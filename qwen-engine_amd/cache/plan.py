@@ -50,6 +50,12 @@ def plan_cache(entry_needs: Sequence[Tuple[Optional[KVNeed], Optional[StateNeed]
                     (kv.num_kv_heads, kv.head_dim) != (src_kv.num_kv_heads, src_kv.head_dim):
                 raise ValueError(f"schedule entry {i} cannot read the cache of entry {cache_from}: "
                                  f"their key/value shapes differ")
+            if kv is not None and src_kv is not None and src_kv.window is not None and \
+                    (kv.window is None or kv.window > src_kv.window):
+                # the source's group gives pages back once its own window has passed them: a reader
+                # that looks further back would read pages that are no longer the request's
+                raise ValueError(f"schedule entry {i} (window {kv.window}) cannot read the cache of entry "
+                                 f"{cache_from}, which keeps only the last {src_kv.window} keys")
             entry_kv.append(None)
             entry_source.append(cache_from if src_kv is not None else None)
             entry_group.append(entry_group[cache_from])

@@ -19,6 +19,7 @@ class EngineConfig:
     enable_prefix_sharing: bool = True
     keep_freed_prefixes: bool = True   # shared pages of finished requests stay until their memory is needed
     seed: int = 0
+    debug_poison: bool = False       # NaN into every cache page when it is handed out and when it goes back
 
     def pages_per_group(self) -> int:
         if self.num_blocks is not None:

@@ -153,8 +153,9 @@ __global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ l
                 run += span_sum[i];
             }
         }
-        if (pick < 0) {  // target at or above the total after rounding: last token with weight
+        if (pick < 0) {  // target at or above the total after rounding: the last token with weight
             pick = V - 1;
+            while (pick > 0 && !(expf(row[pick] * inv_t - mx) > 0.f)) --pick;
         }
         chosen = pick;
     }

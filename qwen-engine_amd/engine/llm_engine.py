@@ -42,7 +42,7 @@ class LLMEngine:
         cfg = self.config
         self.runner = ModelRunner(model, page_size=cfg.block_size, num_pages=cfg.pages_per_group(),
                                   max_requests=cfg.max_num_seqs, prefix_sharing=cfg.enable_prefix_sharing,
-                                  keep_freed_prefixes=cfg.keep_freed_prefixes)
+                                  keep_freed_prefixes=cfg.keep_freed_prefixes, debug_poison=cfg.debug_poison)
         max_len = min(cfg.max_model_len, model.spec.max_positions)
         self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs, max_len, cfg.max_step_tokens,
                                    cfg.prefill_chunk, model.spec.eos_token_ids)

@@ -18,14 +18,15 @@ TOKEN_ROUNDING = 64   # a request's token count is rounded up to this for --max-
 
 
 def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[str],
-           out: IO[str] = sys.stdout, page_size: int = 16, device: str = "cuda:0") -> int:
+           out: IO[str] = sys.stdout, page_size: int = 16, device: str = "cuda:0",
+           debug_poison: bool = False) -> int:
     if TOKEN_ROUNDING % page_size:
         raise ValueError(f"page size {page_size} does not divide {TOKEN_ROUNDING}")
     os.makedirs(out_dir, exist_ok=True)
     model = load_model(model_dir, dtype=dtype, device=device)
     rounded = (max_tokens + TOKEN_ROUNDING - 1) // TOKEN_ROUNDING * TOKEN_ROUNDING
     num_pages = max(1, rounded // page_size)
-    runner = ModelRunner(model, page_size=page_size, num_pages=num_pages, max_requests=MAX_LIVE)
+    runner = ModelRunner(model, page_size=page_size, num_pages=num_pages, max_requests=MAX_LIVE, debug_poison=debug_poison)
     for line in lines:
         line = line.strip()
         if not line:

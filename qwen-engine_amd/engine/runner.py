@@ -73,7 +73,7 @@ class ModelRunner:
 
     def __init__(self, model: DecoderModel, page_size: int, num_pages, max_requests: int,
                  prefix_sharing: bool = False, use_graphs: Optional[bool] = None,
-                 keep_freed_prefixes: bool = False):
+                 keep_freed_prefixes: bool = False, debug_poison: bool = False):
         if model.rt is None:
             raise RuntimeError("the model has no weights yet")
         self.model = model
@@ -87,20 +87,27 @@ class ModelRunner:
                                   keep_freed_prefixes=keep_freed_prefixes) \
             if self.plan.groups else CacheManager([], [], page_size, max_requests)
         dev, dt = self.rt.device, self.rt.dtype
+        # debug_poison: the storage starts as NaN, and every page is filled with NaN again when it
+        # is handed out and when it goes back, so that a read of a key that was never written, or of
+        # a page that is no longer the request's, makes the logits NaN instead of slightly wrong
+        self.debug_poison = bool(debug_poison)
+        self.cache.track_pages = self.debug_poison
+        self.pages_poisoned = 0
         self.kv: List[Optional[torch.Tensor]] = []
         for i, need in enumerate(self.plan.entry_kv):
             if need is None:
                 self.kv.append(None)
                 continue
             pages = self.cache.pools[self.plan.entry_group[i]].num_pages
-            self.kv.append(torch.zeros((pages, 2, need.num_kv_heads, page_size, need.head_dim),
-                                       dtype=dt, device=dev))
+            self.kv.append(torch.full((pages, 2, need.num_kv_heads, page_size, need.head_dim),
+                                      float("nan") if self.debug_poison else 0.0, dtype=dt, device=dev))
         self.state: List[Optional[torch.Tensor]] = []
         for need in self.plan.entry_state:
             if need is None:
                 self.state.append(None)
             else:
-                self.state.append(torch.zeros((max_requests, *need.shape), dtype=torch_dtype(need.dtype), device=dev))
+                # (one slot more than requests: the spare one belongs to the rows that fill a graph up)
+                self.state.append(torch.zeros((max_requests + 1, *need.shape), dtype=torch_dtype(need.dtype), device=dev))
         self.bindings = []
         for i in range(len(model.spec.schedule)):
             src = self.plan.entry_source[i]
@@ -116,7 +123,14 @@ class ModelRunner:
         # bounded by its pool)
         self.table_width = [max(1, per_request if grp.window is not None else min(pool.num_pages, per_request))
                             for grp, pool in zip(self.cache.groups, self.cache.pools)]
-        self.tables = [torch.full((max_requests, w), -1, dtype=torch.int32, device=dev) for w in self.table_width]
+        # one row more than there are state slots: the spare row's first entry always names page 0
+        # of its pool.  It is the table row of the rows that fill a recorded decode graph up and of
+        # the stand-in batch while recording: they stand at position 0 and write nowhere, and what
+        # they read there lies inside the storage whatever the live requests hold.
+        self.tables = [torch.full((max_requests + 1, w), -1, dtype=torch.int32, device=dev) for w in self.table_width]
+        for t in self.tables:
+            t[max_requests, 0] = 0
+        self.spare_row = max_requests
         graph_safe = not has_state and getattr(model, "graph_safe", True)
         self.use_graphs = (dt == torch.bfloat16 and graph_safe) if use_graphs is None else bool(use_graphs)
         self._graphs = {}
@@ -142,6 +156,54 @@ class ModelRunner:
 
     def free_request(self, req_id: Hashable) -> None:
         self.cache.free_request(req_id)
+        self._poison_pages()
+
+    def _poison_pages(self) -> None:
+        """With debug_poison: NaN into every page that was handed out or went back since the last
+        call (plain fills on the current stream, outside any recorded graph)."""
+        if not self.debug_poison:
+            return
+        events = self.cache.take_page_events()
+        if not events:
+            return
+        by_group = {}
+        for g, page in events:
+            by_group.setdefault(g, set()).add(page)
+        for g, pages in by_group.items():
+            idx = torch.tensor(sorted(pages), dtype=torch.long, device=self.rt.device)
+            for i, kv in enumerate(self.kv):
+                if kv is not None and self.plan.entry_group[i] == g:
+                    kv.index_fill_(0, idx, float("nan"))
+            self.pages_poisoned += len(pages)
+
+    def _check_bounds(self, seqs: Sequence[SeqInfo], slots: List[np.ndarray], upd_idx: List[np.ndarray],
+                      upd_val: List[np.ndarray]) -> None:
+        """Host check of what a step sends to the device: every cache slot and every table entry
+        lies inside its pool and its table; with debug_poison also that each request holds a page
+        for every position its tokens can see."""
+        P = self.page_size
+        for g, pool in enumerate(self.cache.pools):
+            if len(slots[g]) and (int(slots[g].min()) < -1 or int(slots[g].max()) >= pool.num_pages * P):
+                raise RuntimeError(f"a cache slot of group {g} lies outside its {pool.num_pages} pages")
+            if len(upd_val[g]) and (int(upd_val[g].min()) < -1 or int(upd_val[g].max()) >= pool.num_pages):
+                raise RuntimeError(f"a table entry of group {g} names a page outside its {pool.num_pages} pages")
+            if len(upd_idx[g]) and (int(upd_idx[g].min()) < 0 or
+                                    int(upd_idx[g].max()) >= self.max_requests * self.table_width[g]):
+                raise RuntimeError(f"a table update of group {g} lies outside the requests' table rows")
+        if not self.debug_poison:
+            return
+        for s in seqs:
+            if s.req_id is None:
+                continue
+            rc = self.cache.get(s.req_id)
+            for g, grp in enumerate(self.cache.groups):
+                first_key = 0 if grp.window is None else max(0, s.kv_before - grp.window + 1)
+                last_key = s.kv_before + s.q_len - 1
+                table = rc.tables[g]
+                for i in range(first_key // P, last_key // P + 1):
+                    if i >= len(table) or table[i] < 0:
+                        raise RuntimeError(f"request {s.req_id!r} holds no page for position {i * P} of group {g}, "
+                                           f"which its tokens at {s.kv_before}..{last_key} can see")
 
     def cache_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.kv if t is not None)
@@ -291,6 +353,8 @@ class ModelRunner:
         device's block tables up to date (one copy to the device, one small kernel per group)."""
         tokens = self._check_and_reserve(entries)
         seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(entries, tokens)
+        self._check_bounds(seqs, slots, upd_idx, upd_val)
+        self._poison_pages()                       # (the pages just handed out, before anything is written)
         T, n_groups = len(token_ids), len(self.cache.groups)
         i32 = np.int32
         dec_rows = np.asarray([s.q_start for s in seqs if s.q_len == 1], dtype=i32)
@@ -329,16 +393,19 @@ class ModelRunner:
             logits = self.model.forward(ctx, self.bindings)
         for e in entries:
             self.cache.commit(e.req_id, e.tokens)
+        self._poison_pages()                       # (pages that a window has passed went back)
         self.steps_run += 1
         return logits
 
     # ---- decoding through a recorded graph ------------------------------------------------
     def _decode_step_with_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._single_token_layout(entries)
+        self._check_bounds(seqs, slots, upd_idx, upd_val)
+        self._poison_pages()                       # (the pages just handed out, before anything is written)
         n_live, n_groups = len(seqs), len(self.cache.groups)
         i32 = np.int32
         # Graphs are recorded for 1 to 8 rows, for multiples of 8 and, beyond 64, of 32: a batch in between is filled up
-        # with rows that stand at position 0 of the first request's table, write nowhere (cache slot
+        # with rows that stand at position 0 of the tables' spare row, write nowhere (cache slot
         # -1) and whose logits are dropped, so that a batch that shrinks request by request does not
         # record a graph for every size it passes.
         B = self.graph_rows(n_live)
@@ -346,7 +413,7 @@ class ModelRunner:
             fill = B - n_live
             token_ids = np.concatenate([token_ids, np.zeros(fill, dtype=i32)])
             positions = np.concatenate([positions, np.zeros(fill, dtype=i32)])
-            tok_seq = np.concatenate([tok_seq, np.full(fill, tok_seq[0], dtype=i32)])
+            tok_seq = np.concatenate([tok_seq, np.full(fill, self.spare_row, dtype=i32)])
             slots = [np.concatenate([x, np.full(fill, -1, dtype=i32)]) for x in slots]
         cap = 2 * B                                    # table updates a decode step can bring per group
         splits = int(positions.max()) // ops.DECODE_SPLIT_KEYS + 1
@@ -390,8 +457,8 @@ class ModelRunner:
         host = torch.zeros(n, dtype=torch.int32).pin_memory()
         meta = torch.zeros(n, dtype=torch.int32, device=dev)
         # a harmless stand-in batch for the runs that only record: every token at position 0 of
-        # slot 0, writing nowhere (cache slot -1), no table updates
-        stand_in = [0] * (3 * B) + list(range(B)) + [0] * B + list(range(B))
+        # the tables' spare row, writing nowhere (cache slot -1), no table updates
+        stand_in = [0] * (2 * B) + [self.spare_row] * B + list(range(B)) + [self.spare_row] * B + list(range(B))
         for g in range(n_groups):
             stand_in += [-1] * B + [-1] * cap + [0] * cap
         meta.copy_(torch.tensor(stand_in, dtype=torch.int32))
@@ -420,10 +487,6 @@ class ModelRunner:
                 ops.scatter_int(self.tables[g], d_upd[g][0], d_upd[g][1])
             return self.model.forward(ctx, self.bindings)
 
-        # slot 0's first table entry must name a real page while the stand-in batch runs
-        saved = [t[0, 0].item() for t in self.tables]
-        for t in self.tables:
-            t[0, 0] = 0
         torch.cuda.synchronize()
         stream = torch.cuda.Stream()
         stream.wait_stream(torch.cuda.current_stream())
@@ -434,8 +497,6 @@ class ModelRunner:
         with torch.cuda.graph(graph, stream=stream):
             logits = run()
         torch.cuda.synchronize()
-        for t, v in zip(self.tables, saved):
-            t[0, 0] = v
         event = torch.cuda.Event()
         event.record()
         return {"graph": graph, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits,

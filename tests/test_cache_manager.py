@@ -235,3 +235,45 @@ def test_plan_groups_entries_by_need_and_lets_an_entry_read_another():
     assert plan.bytes_per_token(2) == 3 * 2 * 2 * 16 * 2
     with pytest.raises(ValueError):
         plan_cache([(full, None, None), (KVNeed(1, 16, None), None, 0)])
+
+
+def test_an_entry_cannot_read_a_cache_that_keeps_fewer_keys_than_it_sees():
+    """The source's group gives pages back once its window has passed them: a reader over all keys,
+    or with a wider window, would follow table entries that are -1 by then."""
+    kv = lambda w: KVNeed(num_kv_heads=2, head_dim=16, window=w)
+    plan_cache([(kv(None), None, None), (kv(8), None, 0)])          # a window over a cache of all keys
+    plan_cache([(kv(16), None, None), (kv(16), None, 0), (kv(5), None, 0)])
+    with pytest.raises(ValueError):
+        plan_cache([(kv(16), None, None), (kv(None), None, 0)])
+    with pytest.raises(ValueError):
+        plan_cache([(kv(16), None, None), (kv(17), None, 0)])
+
+
+def test_pages_handed_out_and_given_back_are_noted_and_kept_pages_are_not():
+    """What the owner of the storage overwrites in its debug mode: every page that leaves or
+    reaches a free list, never a page that is kept for a later request with the same prefix."""
+    m = CacheManager([GroupSpec(), GroupSpec(window=6)], 6, page_size=4, max_requests=2,
+                     prefix_sharing=False)
+    m.track_pages = True
+    m.add_request("a")
+    m.reserve("a", 10)
+    assert sorted(m.take_page_events()) == [(0, 0), (0, 1), (0, 2), (1, 0), (1, 1), (1, 2)]
+    m.commit("a", list(range(10)))                       # the window of 6 has passed positions 0..3
+    assert m.take_page_events() == [(1, 0)]
+    m.free_request("a")
+    assert sorted(m.take_page_events()) == [(0, 0), (0, 1), (0, 2), (1, 1), (1, 2)]
+    assert m.take_page_events() == []
+    # kept prefixes: a finished request's registered pages stay, and are noted only when evicted
+    k = CacheManager([GroupSpec()], 3, page_size=4, max_requests=2, prefix_sharing=True, keep_freed_prefixes=True)
+    k.track_pages = True
+    k.add_request("a")
+    k.reserve("a", 9)
+    k.commit("a", list(range(9)))
+    k.take_page_events()
+    k.free_request("a")                                  # pages 0 and 1 are full and registered: kept
+    assert k.take_page_events() == [(0, 2)] and k.num_kept == 2
+    k.add_request("b")
+    k.reserve("b", 12)                                   # needs all three pages: the kept ones are given up
+    ev = k.take_page_events()
+    assert sorted(set(ev)) == [(0, 0), (0, 1), (0, 2)] and k.num_kept == 0
+    k.check_invariants()

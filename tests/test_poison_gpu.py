@@ -1,0 +1,83 @@
+"""Page poisoning and the tables' spare row.
+
+With ``debug_poison`` every cache page is NaN when it is handed out and when it goes back.  A
+table entry that names a wrong page in one cache group of one request then turns that request's
+logits into NaN also in bfloat16, where a stale page among hundreds of keys would otherwise
+move the logits by less than the rounding.  The other tests run their traces with the poison on;
+this file shows that it bites.  It also runs more decoding requests than a recorded graph has
+rows for, past the shortest window: the rows that fill the graph up must not follow a live
+request's table (whose first entries are -1 by then)."""
+import pytest
+import torch
+
+import qwen_engine_amd  # noqa: F401
+from qwen_engine_amd.engine import ModelRunner, StepEntry, load_model
+from plain import qwen3_plain as P
+from test_window_layers_gpu import PAGE, V, WINDOWS, plain_forward, toy  # noqa: F401  (toy is a fixture)
+
+pytestmark = pytest.mark.gpu
+
+
+def _tokens(n, seed):
+    return torch.randint(0, V, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("group", [0, 1, 2])
+def test_a_wrong_table_entry_in_one_group_gives_nan(toy, dtype, group):
+    """Three cache groups (windows of 40 and 17 keys, and all keys).  After a prompt of 100 tokens,
+    one entry of one group's table on the device is pointed at a page that the request does not
+    hold: the next token's logits are NaN; untouched, they are the plain implementation's."""
+    model = load_model(toy, dtype=dtype)
+    toks = _tokens(102, 5)
+    _, w = P.read_folder(toy)
+    ref = plain_forward(w, toks, None if dtype == "float32" else torch.bfloat16)
+    tol = (1e-4 if dtype == "float32" else 2e-2) * float(ref.abs().max())
+    for corrupt in (False, True):
+        runner = ModelRunner(model, page_size=PAGE, num_pages=24, max_requests=2, debug_poison=True)
+        runner.add_request("other")                      # another request came and went: its pages are poisoned
+        runner.step([StepEntry("other", _tokens(50, 6), [])])
+        runner.free_request("other")
+        runner.add_request("a")
+        runner.step([StepEntry("a", toks[:100], [])])
+        rc = runner.cache.get("a")
+        window = runner.cache.groups[group].window
+        first_key = 0 if window is None else 100 - window + 1
+        index = first_key // PAGE                        # a page that position 100 sees in this group
+        assert rc.tables[group][index] >= 0
+        if corrupt:
+            free_page = runner.cache.pools[group].free[0]
+            runner.tables[group][rc.state_slot, index] = free_page
+        logits = runner.step([StepEntry("a", toks[100:101], [0])]).cpu()
+        if corrupt:
+            assert torch.isnan(logits).any(), f"group {group}: a read of a page that is not the request's went unseen"
+        else:
+            assert float((logits[0] - ref[100]).abs().max()) <= tol
+        assert runner.pages_poisoned > 0
+
+
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_twenty_requests_decode_past_the_window(toy, use_graphs):
+    """20 live requests (a graph of 24 rows, four of them fill rows) decode in bfloat16 after prompts
+    longer than the windows, so that every live request's first table entries are -1."""
+    model = load_model(toy, dtype="bfloat16")
+    _, w = P.read_folder(toy)
+    lengths = [60 + 7 * i for i in range(20)]
+    reqs = [_tokens(n + 6, 100 + i) for i, n in enumerate(lengths)]
+    runner = ModelRunner(model, page_size=PAGE, num_pages=20 * 14, max_requests=20, use_graphs=use_graphs,
+                         debug_poison=True)
+    for i, (toks, n) in enumerate(zip(reqs, lengths)):
+        runner.add_request(i)
+        runner.step([StepEntry(i, toks[:n], [])])
+    for i in range(20):                                  # the windows have passed every request's first page
+        assert runner.cache.get(i).tables[0][0] == -1 or runner.cache.groups[0].window is None
+    outs = [runner.step([StepEntry(i, [reqs[i][lengths[i] + s]], [0]) for i in range(20)]).float().cpu()
+            for s in range(6)]
+    assert (runner.graph_steps == 6) == use_graphs
+    assert all(torch.isfinite(o).all() for o in outs)
+    for i in (0, 7, 19):
+        ref = plain_forward(w, reqs[i], torch.bfloat16)
+        for s in range(6):
+            err = float((outs[s][i] - ref[lengths[i] + s]).abs().max()) / float(ref.abs().max())
+            assert err <= 2e-2, f"request {i}, step {s}: error {err}"
+    runner.cache.check_invariants()

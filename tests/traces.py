@@ -110,18 +110,23 @@ def mixed(requests, seed=0, max_live=4, tail=12):
     return t
 
 
-def run_in_process(trace, folder, dtype, out_dir, page_size):
+def run_in_process(trace, folder, dtype, out_dir, page_size, debug_poison=True):
+    """(debug_poison: every page is NaN when it is handed out and when it goes back, so a read of a
+    key that was never written, or of a page that is another request's by now, shows as NaN)"""
     from qwen_engine_amd.engine.replay import replay
     sink = io.StringIO()
-    replay(folder, dtype, out_dir, trace.max_tokens, io.StringIO(trace.text()), sink, page_size=page_size)
+    replay(folder, dtype, out_dir, trace.max_tokens, io.StringIO(trace.text()), sink, page_size=page_size,
+           debug_poison=debug_poison)
     done = [ln for ln in sink.getvalue().splitlines() if ln.startswith("done ")]
     assert done == [f"done {i}" for i in range(len(trace.steps))]
 
 
-def run_program(trace, folder, dtype, out_dir, page_size, env=None):
+def run_program(trace, folder, dtype, out_dir, page_size, env=None, debug_poison=True):
     """Runs bin/trace_run as a user would: steps go in one at a time, each after 'done <step>'."""
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
            "--out", out_dir, "--max-tokens", str(trace.max_tokens), "--block-size", str(page_size)]
+    if debug_poison:
+        cmd.append("--debug-poison")
     proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, env=env)
     try:
         for i, rec in enumerate(trace.steps):
