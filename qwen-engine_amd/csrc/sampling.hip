@@ -1,6 +1,8 @@
 // Next-token choice on the device from 32-bit logits [R, V]: argmax (lowest index
 // on ties) and temperature sampling by inverse CDF with one uniform per row.
 #include "common.h"
+#include "no_alloc.h"
+#include <mutex>
 
 // One block of 256 threads per row.
 __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
@@ -106,6 +108,57 @@ extern "C" int qe_argmax(const float* logits, int* out, int R, int V, void* work
     }
     QE_LAUNCH_CHECK();
     return 0;
+}
+
+// ---- argmax for callers that cannot allocate ----------------------------------------------------
+// The two-stage argmax keeps each span's best (value, index) in device memory between its two
+// kernels.  qe_argmax takes that memory from the caller; qe_argmax_static keeps it in an array that
+// is part of the loaded library, one copy on every GPU, so the call allocates nothing.  In host code
+// the array's name is only a handle: the address the kernels get is asked for once per device
+// with hipGetSymbolAddress and kept.
+static __device__ __align__(256) unsigned char scratch[QE_ARGMAX_STATIC_BYTES];
+
+#define QE_MAX_DEVICES 64
+static void* g_scratch_ptr[QE_MAX_DEVICES];      // per device: the address of its copy of `scratch`
+static std::mutex g_scratch_mutex;
+
+// The current device's copy of the array (null and an error text if the runtime refuses).
+static void* static_scratch_of_current_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= QE_MAX_DEVICES) {
+        qe_set_error("argmax (static): no current device, or device %d beyond %d", dev, QE_MAX_DEVICES);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            qe_set_error("argmax (static): hipGetSymbolAddress: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+
+extern "C" long qe_argmax_static_max_bytes() { return QE_ARGMAX_STATIC_BYTES; }
+
+extern "C" int qe_argmax_static(const float* logits, int* out, int R, int V, hipStream_t stream) {
+    QE_REQUIRE(R >= 0 && V > 0, "argmax (static): bad sizes R=%d V=%d", R, V);
+    if (R == 0) return 0;
+    const long need = qe_argmax_workspace_bytes(R, V);
+    QE_REQUIRE(need <= (long)QE_ARGMAX_STATIC_BYTES,
+               "argmax (static): R=%d rows of V=%d need %ld bytes between the two stages, the static buffer has %ld "
+               "(use qe_argmax with a workspace)", R, V, need, (long)QE_ARGMAX_STATIC_BYTES);
+    void* ws = nullptr;
+    if (need > 0) {
+        ws = static_scratch_of_current_device();
+        if (!ws) return -1;
+    }
+    // (nothing has to start at zero: the first stage writes every entry that the second reads)
+    return qe_argmax(logits, out, R, V, ws, need, stream);
 }
 
 // Row r: temperature[r] <= 0 -> argmax.  Else with z_i = logits_i / temperature,
