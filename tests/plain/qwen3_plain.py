@@ -185,10 +185,11 @@ def rope_theta_of(cfg: dict) -> float:
 def forward_logits(cfg: dict, w: Dict[str, torch.Tensor], token_ids: List[int],
                    compute: torch.dtype = torch.float32,
                    act_dtype: Optional[torch.dtype] = None,
-                   position_offset: int = 0) -> torch.Tensor:
+                   position_offset: int = 0, rows: Optional[List[int]] = None) -> torch.Tensor:
     """Logits [T, V] of one whole sequence: embedding, the layers in order, final
     norm, head (src/models/qwen3/model.py:349-359,420-422); the head is the
-    embedding table when tie_word_embeddings (model.py:417-418)."""
+    embedding table when tie_word_embeddings (model.py:417-418).  With ``rows`` only those
+    rows of the logits are formed (the layers still run on the whole sequence)."""
     ids = torch.tensor(token_ids, dtype=torch.long)
     t = ids.numel()
     positions = torch.arange(t) + position_offset
@@ -196,6 +197,8 @@ def forward_logits(cfg: dict, w: Dict[str, torch.Tensor], token_ids: List[int],
     h = embedding(ids, w["model.embed_tokens.weight"]).to(compute)
     for i in range(cfg["num_hidden_layers"]):
         h = decoder_layer(h, positions, w, f"model.layers.{i}", cfg, table, act_dtype)
+    if rows is not None:
+        h = h[torch.tensor(list(rows), dtype=torch.long)]
     x = _round(rms_norm(h, w["model.norm.weight"].to(compute), cfg["rms_norm_eps"]), act_dtype)
     head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
     return linear(x, head.to(compute))

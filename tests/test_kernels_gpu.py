@@ -810,3 +810,54 @@ def test_gemm_with_silu_mul_over_interleaved_rows(ops, M, I, K):
                 close(ops.gemm(x.to(DEV), w.to(DEV), epilogue=ops.EPI_SILU_MUL_IL, algo=ops.ALGO_TILE + rows), want, bf)
     gu = ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_GENERIC)
     close(ops.silu_mul(gu, interleaved=True), want, bf)
+
+
+@pytest.mark.parametrize("L", [4096, 4097, 8300])
+def test_decode_kernel_with_more_than_32_splits(ops, L):
+    """A token at position L - 1 over 32, 33 and 65 splits of 128 keys: the merge kernel sums eight of a
+    wave's splits at a time and goes round again beyond 32 splits, and its first pass over the maxima
+    goes round again beyond 64.  In each of four head groups one key carries the result: the first
+    key, one in the middle, the last key of split 31, and the token's own."""
+    bf = torch.bfloat16
+    hq, hkv, d, page = 8, 4, 128, 16
+    k = rand(L, hkv, d, seed=510, dtype=bf, scale=0.1)
+    v = rand(L, hkv, d, seed=511, dtype=bf)
+    q = rand(1, hq, d, seed=512, dtype=bf)
+    far = [0, L // 2 + 5, 4095, L - 1]
+    for kvh, key_pos in enumerate(far):
+        k[key_pos, kvh] = (q[0, 2 * kvh].float() * 4).to(bf)
+    cache, ids = paged_cache(k, v, page, 513, bf)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    out = ops.attention(q.to(DEV), cache.to(DEV), i32([L - 1]), i32([0]), ids[None].to(DEV), 1 / math.sqrt(d),
+                        dec_tokens=i32([0]), max_dec_position=L - 1)
+    want = P.attention(q.float(), k.float(), v.float(), 1 / math.sqrt(d))
+    close(out, want, bf)
+    for kvh, key_pos in enumerate(far):
+        assert float((want[0, 2 * kvh] - v[key_pos, kvh].float()).abs().max()) < 0.05
+    # several rows whose graphs share the largest position: a shorter one leaves its last splits empty
+    positions = [L - 1, 130, 4000]
+    qs = rand(3, hq, d, seed=514, dtype=bf)
+    table = ids[None].repeat(3, 1)
+    out = ops.attention(qs.to(DEV), cache.to(DEV), i32(positions), i32([0, 1, 2]), table.to(DEV), 1 / math.sqrt(d),
+                        dec_tokens=i32([0, 1, 2]), max_dec_position=L - 1)
+    want = torch.cat([P.attention(qs[i:i + 1].float(), k[:p + 1].float(), v[:p + 1].float(), 1 / math.sqrt(d))
+                      for i, p in enumerate(positions)])
+    close(out, want, bf)
+
+
+@pytest.mark.parametrize("M", [1, 8, 64])
+def test_gemm_for_few_rows_against_the_whole_vocabulary(ops, M):
+    """The head's product at the family's vocabulary: [M, 1024] against [151936, 1024], 32-bit logits,
+    compared in 64-bit on the first and last columns and on 3000 drawn ones."""
+    bf = torch.bfloat16
+    N, K = 151936, 1024
+    x, w = rand(M, K, seed=520, dtype=bf), rand(N, K, seed=521, dtype=bf, scale=0.02)
+    got = ops.gemm(x.to(DEV), w.to(DEV), out_dtype=torch.float32).cpu()
+    assert got.shape == (M, N) and torch.isfinite(got).all()
+    cols = torch.cat([torch.arange(0, 80), torch.arange(N - 120, N),
+                      torch.randint(0, N, (3000,), generator=torch.Generator().manual_seed(522))])
+    want = x.double() @ w[cols].double().t()
+    close(got[:, cols], want, torch.float32, scale=float(want.abs().max()))
+    # the same through the generic 32-bit kernel, on 32-bit copies of the operands
+    got32 = ops.gemm(x.float().to(DEV), w.float().to(DEV), out_dtype=torch.float32, algo=ops.ALGO_GENERIC).cpu()
+    close(got32[:, cols], want, torch.float32, scale=float(want.abs().max()))
