@@ -75,6 +75,8 @@ class LayerSpec:
     ffn_norm: object
     ffn: object
     kind: str = "prenorm_block"
+    # checkpoint names of the four parts inside ``prefix``, in the order of the fields above
+    part_names: Tuple[str, str, str, str] = ("input_layernorm", "self_attn", "post_attention_layernorm", "mlp")
 
 
 @dataclass(frozen=True)
@@ -104,6 +106,9 @@ class ModelSpec:
     tie_head: bool
     max_positions: int
     eos_token_ids: Tuple[int, ...] = field(default_factory=tuple)
+    # optional parts around the layers: a spec with a ``kind`` (and a ``prefix`` for its tensors' names)
+    stream_prologue: Optional[object] = None   # changes the stream right after the embedding
+    logit_epilogue: Optional[object] = None    # changes the logits after the head
 
     def validate(self) -> None:
         if not self.layers:

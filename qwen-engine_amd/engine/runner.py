@@ -68,7 +68,6 @@ class ModelRunner:
     and replayed, so that their launch cost does not grow with the number of kernels.
     """
 
-    SPLIT_BUCKET = 8      # decode graphs are recorded per this many splits of the keys
     MAX_GRAPHS = 32       # recorded graphs kept (each holds its own activations); the least recently used goes first
 
     def __init__(self, model: DecoderModel, page_size: int, num_pages, max_requests: int,
@@ -131,8 +130,19 @@ class ModelRunner:
         for t in self.tables:
             t[max_requests, 0] = 0
         self.spare_row = max_requests
-        graph_safe = not has_state and getattr(model, "graph_safe", True)
+        # a part with per-request state is recorded into graphs only if it says that it can be
+        # (``graph_safe = True`` on the class); any other part unless it says that it cannot
+        stateful_ok = all(self.plan.entry_state[i] is None or
+                          getattr(model.blocks[e.layer].mixer, "graph_safe", False) is True
+                          for i, e in enumerate(model.spec.schedule))
+        graph_safe = stateful_ok and getattr(model, "graph_safe", True)
         self.use_graphs = (dt == torch.bfloat16 and graph_safe) if use_graphs is None else bool(use_graphs)
+        # the part classes that want something prepared for every step (parts.base: step_extras)
+        self._step_classes = []
+        for part in model.all_parts():
+            cls = type(part)
+            if hasattr(cls, "step_extras") and cls not in self._step_classes:
+                self._step_classes.append(cls)
         self._graphs = {}
         self._stage: Optional[torch.Tensor] = None     # pinned host buffer of a step's integer arrays
         self._stage_np = None
@@ -157,6 +167,14 @@ class ModelRunner:
     def free_request(self, req_id: Hashable) -> None:
         self.cache.free_request(req_id)
         self._poison_pages()
+
+    def _clear_state_of_new_requests(self, seqs: Sequence[SeqInfo]) -> None:
+        """The fixed-size state of a request that runs its first step begins at zero."""
+        for s in seqs:
+            if s.new_request:
+                for st in self.state:
+                    if st is not None:
+                        st[s.state_slot].zero_()
 
     def _poison_pages(self) -> None:
         """With debug_poison: NaN into every page that was handed out or went back since the last
@@ -357,26 +375,28 @@ class ModelRunner:
         self._poison_pages()                       # (the pages just handed out, before anything is written)
         T, n_groups = len(token_ids), len(self.cache.groups)
         i32 = np.int32
-        dec_rows = np.asarray([s.q_start for s in seqs if s.q_len == 1], dtype=i32)
-        other = [np.arange(s.q_start, s.q_start + s.q_len, dtype=i32) for s in seqs if s.q_len > 1]
-        other_rows = np.concatenate(other) if other else np.zeros(0, dtype=i32)
-        max_dec = max([s.kv_before for s in seqs if s.q_len == 1], default=0)
-        parts = [token_ids, positions, tok_seq, rows, np.asarray([s.state_slot for s in seqs], dtype=i32),
-                 dec_rows, other_rows]
+        parts = [token_ids, positions, tok_seq, rows, np.asarray([s.state_slot for s in seqs], dtype=i32)]
+        n_fixed = len(parts)
         for g in range(n_groups):
             parts += [slots[g], upd_idx[g], upd_val[g]]
+        # what single parts want prepared for the step: their arrays travel in the same copy
+        extras = {cls: dict(cls.step_extras(seqs)) for cls in self._step_classes}
+        wanted = [(cls, name) for cls, d in extras.items() for name, v in d.items() if isinstance(v, np.ndarray)]
+        parts += [extras[cls][name].astype(i32, copy=False) for cls, name in wanted]
         dev = self._to_device(parts)
-        d_tok, d_pos, d_seq, d_rows, d_state, d_dec, d_other = dev[:7]
+        d_tok, d_pos, d_seq, d_rows, d_state = dev[:n_fixed]
         d_slots = []
         for g in range(n_groups):
-            d_slot, d_idx, d_val = dev[7 + 3 * g:10 + 3 * g]
+            d_slot, d_idx, d_val = dev[n_fixed + 3 * g:n_fixed + 3 + 3 * g]
             d_slots.append(d_slot)
             if len(d_idx):
                 ops.scatter_int(self.tables[g], d_idx, d_val)
+        for (cls, name), t in zip(wanted, dev[n_fixed + 3 * n_groups:]):
+            extras[cls][name] = t
         return StepContext(rt=self.rt, page_size=self.page_size, num_tokens=T, seqs=seqs, token_ids=d_tok,
                            positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
                            logit_rows=d_rows, state_slots=d_state, max_position=int(positions.max()),
-                           dec_tokens=d_dec, other_tokens=d_other, max_dec_position=max_dec)
+                           extras=extras)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Runs the entries' tokens as one batch; returns float32 logits [wanted, vocab] on the
@@ -385,11 +405,7 @@ class ModelRunner:
             logits = self._decode_step_with_graph(entries)
         else:
             ctx = self.build_context(entries)
-            for s in ctx.seqs:          # fixed-size state of a starting request begins at zero
-                if s.new_request:
-                    for st in self.state:
-                        if st is not None:
-                            st[s.state_slot].zero_()
+            self._clear_state_of_new_requests(ctx.seqs)
             logits = self.model.forward(ctx, self.bindings)
         for e in entries:
             self.cache.commit(e.req_id, e.tokens)
@@ -402,6 +418,7 @@ class ModelRunner:
         seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._single_token_layout(entries)
         self._check_bounds(seqs, slots, upd_idx, upd_val)
         self._poison_pages()                       # (the pages just handed out, before anything is written)
+        self._clear_state_of_new_requests(seqs)
         n_live, n_groups = len(seqs), len(self.cache.groups)
         i32 = np.int32
         # Graphs are recorded for 1 to 8 rows, for multiples of 8 and, beyond 64, of 32: a batch in between is filled up
@@ -416,8 +433,9 @@ class ModelRunner:
             tok_seq = np.concatenate([tok_seq, np.full(fill, self.spare_row, dtype=i32)])
             slots = [np.concatenate([x, np.full(fill, -1, dtype=i32)]) for x in slots]
         cap = 2 * B                                    # table updates a decode step can bring per group
-        splits = int(positions.max()) // ops.DECODE_SPLIT_KEYS + 1
-        bucket = (splits + self.SPLIT_BUCKET - 1) // self.SPLIT_BUCKET * self.SPLIT_BUCKET
+        max_position = int(positions.max())
+        part_keys = tuple(cls.graph_key(max_position) if hasattr(cls, "graph_key") else None
+                          for cls in self._step_classes)
         if any(len(u) > cap for u in upd_idx):
             # more table changes than the recorded step takes (the first decode step after a
             # preemption, say): bring the tables up to date apart, then go on with none
@@ -426,17 +444,17 @@ class ModelRunner:
                     ops.scatter_int(self.tables[g], torch.from_numpy(upd_idx[g]).to(self.rt.device),
                                     torch.from_numpy(upd_val[g]).to(self.rt.device))
                 upd_idx[g] = upd_val[g] = np.zeros(0, dtype=i32)
-        key = (B, bucket)
+        key = (B, part_keys)
         rec = self._graphs.pop(key, None)
         if rec is None:
             while len(self._graphs) >= self.MAX_GRAPHS:
                 self._graphs.pop(next(iter(self._graphs)))     # dicts keep insertion order: the oldest use
-            rec = self._record_decode_graph(B, bucket, cap)
+            rec = self._record_decode_graph(B, part_keys, cap)
             self.graphs_recorded += 1
         self._graphs[key] = rec                                # (re)inserted last = most recently used
         iota, none, zero = rec["iota"], rec["none"], rec["zero"]       # 0 .. B - 1; cap times -1; cap zeros
         # (a row's table row is its request's state slot: tok_seq serves as both)
-        parts = [token_ids, positions, tok_seq, iota, tok_seq, iota]
+        parts = [token_ids, positions, tok_seq, iota, tok_seq]
         for g in range(n_groups):
             pad = cap - len(upd_idx[g])
             parts += [slots[g], upd_idx[g], none[:pad], upd_val[g], zero[:pad]]
@@ -448,17 +466,17 @@ class ModelRunner:
         self.graph_steps += 1
         return rec["logits"][:n_live].clone()          # the graph's own output is overwritten by the next replay
 
-    def _record_decode_graph(self, B: int, bucket: int, cap: int):
-        """Static buffers for a decode step of B requests whose keys fit ``bucket`` splits, one
-        run outside the graph (so that nothing is set up for the first time while recording),
-        then the recording."""
+    def _record_decode_graph(self, B: int, part_keys: tuple, cap: int):
+        """Static buffers for a decode step of B requests whose positions give the parts'
+        ``part_keys``, one run outside the graph (so that nothing is set up for the first time
+        while recording), then the recording."""
         dev, n_groups = self.rt.device, len(self.cache.groups)
-        n = 6 * B + n_groups * (B + 2 * cap)
+        n = 5 * B + n_groups * (B + 2 * cap)
         host = torch.zeros(n, dtype=torch.int32).pin_memory()
         meta = torch.zeros(n, dtype=torch.int32, device=dev)
         # a harmless stand-in batch for the runs that only record: every token at position 0 of
         # the tables' spare row, writing nowhere (cache slot -1), no table updates
-        stand_in = [0] * (2 * B) + [self.spare_row] * B + list(range(B)) + [self.spare_row] * B + list(range(B))
+        stand_in = [0] * (2 * B) + [self.spare_row] * B + list(range(B)) + [self.spare_row] * B
         for g in range(n_groups):
             stand_in += [-1] * B + [-1] * cap + [0] * cap
         meta.copy_(torch.tensor(stand_in, dtype=torch.int32))
@@ -470,7 +488,7 @@ class ModelRunner:
             off += k
             return t
 
-        d_tok, d_pos, d_seq, d_rows, d_state, d_dec = (take(B) for _ in range(6))
+        d_tok, d_pos, d_seq, d_rows, d_state = (take(B) for _ in range(5))
         d_slots, d_upd = [], []
         for g in range(n_groups):
             d_slots.append(take(B))
@@ -478,9 +496,9 @@ class ModelRunner:
         seqs = [SeqInfo(None, i, 1, 0, 0, False) for i in range(B)]
         ctx = StepContext(rt=self.rt, page_size=self.page_size, num_tokens=B, seqs=seqs, token_ids=d_tok,
                           positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
-                          logit_rows=d_rows, state_slots=d_state,
-                          max_position=0, dec_tokens=d_dec, other_tokens=None,
-                          max_dec_position=bucket * ops.DECODE_SPLIT_KEYS - 1)
+                          logit_rows=d_rows, state_slots=d_state, max_position=0,
+                          extras={cls: dict(cls.graph_extras(B, k, dev)) if hasattr(cls, "graph_extras") else {}
+                                  for cls, k in zip(self._step_classes, part_keys)})
 
         def run():
             for g in range(n_groups):
@@ -499,6 +517,8 @@ class ModelRunner:
         torch.cuda.synchronize()
         event = torch.cuda.Event()
         event.record()
-        return {"graph": graph, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits,
+        # (the context is kept with the graph: what the parts made for the recorded step, their
+        # graph_extras, is read by every replay)
+        return {"graph": graph, "ctx": ctx, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits,
                 "event": event, "iota": np.arange(B, dtype=np.int32), "none": np.full(cap, -1, dtype=np.int32),
                 "zero": np.zeros(cap, dtype=np.int32)}

@@ -16,6 +16,13 @@ at finish, and a rule for when pages run out:
     waiting queue, and it is recomputed from its prompt and the tokens it has already
     produced when it is admitted again (sampling does not depend on that);
   * a request that cannot fit even when it has the cache to itself fails with an error.
+
+Requests that arrive together and begin alike share their beginning too (the reference registers a
+prompt's pages when it allocates them, src/engine/kvcache.py:183-195, so the prompts of one batch
+find each other; here a page is registered only once it is computed): a waiting request whose
+first pages equal pages that a running request is still to compute is held back until they are
+computed, and then takes them over instead of computing them again.  Requests behind it in the
+queue may start meanwhile.
 """
 from __future__ import annotations
 
@@ -23,7 +30,7 @@ from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, Hashable, List, Optional, Sequence, Tuple
 
-from ..cache.manager import CacheManager
+from ..cache.manager import CacheManager, chain_hash
 from ..sampling.sampler import SamplingParams
 
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
@@ -42,6 +49,20 @@ class Request:
     admit_order: int = -1
     preemptions: int = 0
     prompt_text: Optional[str] = None
+    _page_hashes: Optional[Tuple[int, int, List[int]]] = None   # (page size, tokens hashed, chain hashes)
+
+    def page_hashes(self, page_size: int) -> List[int]:
+        """Chain hashes of the full pages of the known tokens (kept; extended when tokens were added)."""
+        known = self.known
+        full = len(known) // page_size
+        if self._page_hashes is None or self._page_hashes[0] != page_size:
+            self._page_hashes = (page_size, 0, [])
+        _, _, hashes = self._page_hashes
+        while len(hashes) < full:
+            i = len(hashes)
+            hashes.append(chain_hash(hashes[-1] if hashes else 0, known[i * page_size:(i + 1) * page_size]))
+        self._page_hashes = (page_size, full * page_size, hashes)
+        return hashes
 
     @property
     def known(self) -> List[int]:
@@ -73,7 +94,7 @@ class Scheduler:
         self.finished: List[Request] = []
         self._admitted = 0
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0,
-                      "shared_prefix_tokens": 0, "failed": 0}
+                      "shared_prefix_tokens": 0, "failed": 0, "held_back_for_prefix": 0}
 
     # ---- queue ----------------------------------------------------------------------
     def add(self, request: Request) -> None:
@@ -108,6 +129,25 @@ class Scheduler:
             if (span + P - 1) // P > pool.num_pages:
                 return False
         return True
+
+    def _pages_worth_waiting_for(self, r: Request, start: int) -> bool:
+        """True if a running request is still to compute pages that equal r's pages beyond its first
+        ``start`` tokens: r then does better to wait and take them over than to compute them itself."""
+        if not self.cache.prefix_sharing:
+            return False
+        P = self.cache.page_size
+        mine = r.page_hashes(P)[:(r.num_known - 1) // P]      # (one token is always left to compute)
+        have = start // P
+        if len(mine) <= have:
+            return False
+        for q in self.running:
+            theirs = q.page_hashes(P)
+            if len(theirs) <= have or theirs[have] != mine[have] or q.num_computed >= (have + 1) * P:
+                continue
+            # (equal chain hashes at index `have`: everything up to there is equal, up to collisions,
+            # which at worst make r wait until q has computed that page)
+            return True
+        return False
 
     def _preempt_last(self) -> bool:
         """Give back the pages of the running request that was admitted last."""
@@ -169,7 +209,8 @@ class Scheduler:
                     self.cache.free_request(blocked.req_id)
                     self._fail(blocked, "the cache is too small for this request")
                 continue
-            # admission, first in first out
+            # admission, first in first out (a request that waits for another's pages lets the next pass)
+            held: List[Request] = []
             while self.waiting and len(self.running) < self.max_num_seqs and budget > 0 \
                     and self.cache.slots.num_free > 0:
                 r = self.waiting[0]
@@ -179,6 +220,11 @@ class Scheduler:
                     continue
                 self.cache.add_request(r.req_id)
                 start = self.cache.match_prefix(r.req_id, r.known)
+                if self._pages_worth_waiting_for(r, start):
+                    self.cache.free_request(r.req_id)
+                    held.append(self.waiting.popleft())
+                    self.stats["held_back_for_prefix"] += 1
+                    continue
                 remaining = r.num_known - start
                 n = min(remaining, self.prefill_chunk, budget)
                 if not fits(r.req_id, start + n):
@@ -193,6 +239,7 @@ class Scheduler:
                 self.stats["shared_prefix_tokens"] += start
                 planned.append(Planned(r, r.known[start:start + n], sample=(start + n == r.num_known)))
                 budget -= n
+            self.waiting.extendleft(reversed(held))            # back to the front, in their order
             if not planned and self.waiting and not self.running:
                 # nothing runs and the first waiting request cannot start: it can never start
                 r = self.waiting.popleft()

@@ -8,8 +8,9 @@ Scores, mask and softmax follow src/layers/fused_ops/attn.py:236-267.
 """
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Dict, List, Optional
 
+import numpy as np
 import torch
 
 from ..cache.plan import KVNeed
@@ -24,7 +25,62 @@ from .registry import build_part, register_part
 FUSED_DECODE_MAX_TOKENS = 16
 
 
+def prefill_tiles(portions, rows_per_tile: int) -> List[int]:
+    """(first row, rows) pairs, flat, for portions given as (first row, number of rows): tiles of
+    at most rows_per_tile rows, in groups of four per portion, padded with (first row, 0): what the
+    prefill attention kernel takes."""
+    flat: List[int] = []
+    for start, n in portions:
+        tiles = [(start + r, min(rows_per_tile, n - r)) for r in range(0, n, rows_per_tile)]
+        while len(tiles) % 4:
+            tiles.append((start, 0))
+        for t in tiles:
+            flat.extend(t)
+    return flat
+
+
 class PagedAttention:
+    # ---- what the step function prepares for this part (parts.base) --------------------------
+    @staticmethod
+    def step_extras(seqs) -> dict:
+        """The rows that are the single new token of their request (they go to the decode kernel, the
+        largest of their positions fixing its number of key splits) and all other rows."""
+        dec = [s.q_start for s in seqs if s.q_len == 1]
+        other = [np.arange(s.q_start, s.q_start + s.q_len, dtype=np.int32) for s in seqs if s.q_len > 1]
+        return {"dec_tokens": np.asarray(dec, dtype=np.int32),
+                "other_tokens": np.concatenate(other) if other else np.zeros(0, dtype=np.int32),
+                "max_dec_position": max([s.kv_before for s in seqs if s.q_len == 1], default=0)}
+
+    GRAPH_SPLIT_BUCKET = 8      # a recorded decode step serves positions up to the next multiple of this many key splits
+
+    @staticmethod
+    def graph_key(max_position: int) -> int:
+        """The decode kernel's grid and workspace follow the number of key splits: recorded steps are
+        kept per bucket of splits."""
+        splits = int(max_position) // ops.DECODE_SPLIT_KEYS + 1
+        b = PagedAttention.GRAPH_SPLIT_BUCKET
+        return (splits + b - 1) // b * b
+
+    @staticmethod
+    def graph_extras(rows: int, key: int, device) -> dict:
+        return {"dec_tokens": torch.arange(rows, dtype=torch.int32, device=device), "other_tokens": None,
+                "max_dec_position": key * ops.DECODE_SPLIT_KEYS - 1}
+
+    def _extras(self, ctx) -> dict:
+        return ctx.extras.get(PagedAttention) or {"dec_tokens": None, "other_tokens": None, "max_dec_position": 0}
+
+    def _other_tiles(self, ctx) -> Optional[torch.Tensor]:
+        """The rows of requests that bring several tokens, cut into tiles for the prefill kernel: built
+        and sent to the device once per step and tile size, shared by the layers."""
+        rows_per_tile = ops.prefill_tile_rows(self.hq, self.hkv)
+        if rows_per_tile <= 0:
+            return None
+        key = ("paged_attention.tiles", rows_per_tile)
+        if key not in ctx.memo:
+            flat = prefill_tiles([(s.q_start, s.q_len) for s in ctx.seqs if s.q_len > 1], rows_per_tile)
+            ctx.memo[key] = torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(ctx.rt.device) if flat else None
+        return ctx.memo[key]
+
     def __init__(self, spec, hidden_size: int):
         self.spec = spec
         self.hidden = int(hidden_size)
@@ -117,14 +173,15 @@ class PagedAttention:
             return self._attend(q, ctx, cache, g, T)
         qkv = ops.gemm(x, self.w_qkv, self.b_qkv)
         if fused_position:
-            only_new_tokens = (ctx.dec_tokens is not None and ctx.dec_tokens.shape[0] == T and
-                               (ctx.other_tokens is None or ctx.other_tokens.shape[0] == 0))
+            ex = self._extras(ctx)
+            only_new_tokens = (ex["dec_tokens"] is not None and ex["dec_tokens"].shape[0] == T and
+                               (ex["other_tokens"] is None or ex["other_tokens"].shape[0] == 0))
             if (only_new_tokens and T <= FUSED_DECODE_MAX_TOKENS and binding.write and
                     ops.attention_decode_fused_supported(qkv, cache, self.hq, table)):
                 # every row is the one new token of its request: norm, rotation and cache write
                 # happen inside the attention kernel
                 o = ops.attention_decode_fused(qkv, self.hq, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g],
-                                               self.scale, self.window, None, ctx.max_dec_position,
+                                               self.scale, self.window, None, ex["max_dec_position"],
                                                self.q_norm, self.k_norm, eps, table, slots)
                 return self._project_out(o.view(T, self.hq * self.d))
             q = ops.qk_rope_store(qkv, self.hq, self.hkv, self.d, ctx.positions, self.q_norm, self.k_norm,
@@ -140,10 +197,11 @@ class PagedAttention:
         return self._attend(q, ctx, cache, g, T)
 
     def _attend(self, q: torch.Tensor, ctx, cache: torch.Tensor, g: int, T: int) -> torch.Tensor:
+        ex = self._extras(ctx)
         o = ops.attention(q, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g], self.scale, self.window,
-                          dec_tokens=ctx.dec_tokens, max_dec_position=ctx.max_dec_position,
-                          other_tokens=ctx.other_tokens,
-                          other_tiles=ctx.other_tiles(ops.prefill_tile_rows(self.hq, self.hkv)))
+                          dec_tokens=ex["dec_tokens"], max_dec_position=ex["max_dec_position"],
+                          other_tokens=ex["other_tokens"],
+                          other_tiles=self._other_tiles(ctx) if ex["other_tokens"] is not None else None)
         return self._project_out(o.view(T, self.hq * self.d))
 
     def _project_out(self, o: torch.Tensor) -> torch.Tensor:

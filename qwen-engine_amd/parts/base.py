@@ -12,6 +12,20 @@ FeedForward   forward(x, ctx) -> y
               partial products whose sum over S, taken in order, is the output (the norm adds them).
 Position      table() for the fused kernel, or apply(packed, positions, num_q, num_k) in place
               on a [T, Hq + 2 Hkv, D] tensor of q | k | v heads.
+Stream prologue   forward(h, ctx) -> None: changes the 32-bit stream in place right after the
+              embedding (a scale, an added table of positions).
+Logit epilogue    forward(logits, ctx) -> logits on the float32 logits [R, V] (a scale, a soft cap).
+
+What a part needs prepared per step beyond the flat batch, it asks for itself; the step function
+knows none of it.  A part class may define (all optional, all static):
+  step_extras(seqs) -> dict      from the step's SeqInfo list, on the host: int32 numpy arrays (sent
+                                 to the device with the batch, in the one copy) and plain numbers;
+                                 the part finds them as ctx.extras[its class]
+  graph_key(max_position)        what of a decode step's positions the part's launches depend on
+                                 (a recorded step is replayed only for the same key)
+  graph_extras(rows, key, device) -> dict   the same entries as step_extras for a recorded step of
+                                 ``rows`` single new tokens whose positions give ``key``, as
+                                 tensors that stay as they are for every replay
 """
 from __future__ import annotations
 

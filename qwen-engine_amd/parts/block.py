@@ -11,12 +11,9 @@ import torch
 from .base import CacheBinding, Runtime, TensorInfo
 from .registry import build_part, part_class, register_part
 
-# checkpoint names of the four parts inside a layer's prefix
-_NAMES = ("input_layernorm", "self_attn", "post_attention_layernorm", "mlp")
-
-
 def _names(spec):
-    return getattr(spec, "part_names", _NAMES)
+    """Checkpoint names of the four parts inside the layer's prefix (LayerSpec.part_names)."""
+    return spec.part_names
 
 
 class PreNormBlock:
@@ -32,6 +29,9 @@ class PreNormBlock:
     def graph_safe(self) -> bool:
         """False if any part of the block says that its forward cannot be recorded into a graph."""
         return all(getattr(p, "graph_safe", True) for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
+
+    def parts(self):
+        return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
 
     @staticmethod
     def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:

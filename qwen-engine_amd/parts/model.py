@@ -26,7 +26,15 @@ def expected_tensors(spec: ModelSpec) -> Dict[str, TensorInfo]:
         out[f"{base}.{rel}"] = info
     if not spec.tie_head:
         out[spec.head_name] = TensorInfo((spec.vocab_size, spec.hidden_size), "normal", "matrix")
+    for extra in (spec.stream_prologue, spec.logit_epilogue):
+        if extra is not None:
+            for rel, info in part_class(extra.kind).expected_tensors(extra, spec.hidden_size).items():
+                out[_join(getattr(extra, "prefix", ""), rel)] = info
     return out
+
+
+def _join(prefix: str, rel: str) -> str:
+    return f"{prefix}.{rel}" if prefix else rel
 
 
 def cache_plan(spec: ModelSpec) -> CachePlan:
@@ -46,6 +54,10 @@ class DecoderModel:
         self.spec = spec
         self.blocks = [build_part(layer, spec.hidden_size) for layer in spec.layers]
         self.final_norm = build_part(spec.final_norm, spec.hidden_size)
+        # optional parts around the layers: one that changes the stream right after the embedding
+        # (forward(h, ctx), in place), one that changes the logits after the head (forward(logits, ctx))
+        self.prologue = build_part(spec.stream_prologue, spec.hidden_size) if spec.stream_prologue is not None else None
+        self.epilogue = build_part(spec.logit_epilogue, spec.hidden_size) if spec.logit_epilogue is not None else None
         self.embed: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
         self.rt: Optional[Runtime] = None
@@ -55,7 +67,17 @@ class DecoderModel:
         """A part whose forward reads results back on the host, sizes tensors by their contents or
         walks the requests of a step sets ``graph_safe = False``; the decode steps of a model with
         such a part are run as they come instead of being recorded once and replayed."""
-        return all(getattr(p, "graph_safe", True) for p in (*self.blocks, self.final_norm))
+        return all(getattr(p, "graph_safe", True) for p in (*self.blocks, *self._around()))
+
+    def _around(self):
+        return [p for p in (self.final_norm, self.prologue, self.epilogue) if p is not None]
+
+    def all_parts(self):
+        """Every part of the model, the parts inside the blocks included."""
+        for b in self.blocks:
+            yield b
+            yield from (b.parts() if hasattr(b, "parts") else ())
+        yield from self._around()
 
     def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
         spec = self.spec
@@ -67,6 +89,12 @@ class DecoderModel:
         base = spec.final_norm_name[:-len(".weight")] if spec.final_norm_name.endswith(".weight") else spec.final_norm_name
         self.final_norm.load({k[len(base) + 1:]: v for k, v in tensors.items() if k.startswith(base + ".")}, rt)
         self.head = self.embed if spec.tie_head else rt.place_matrix(tensors[spec.head_name])
+        for part, part_spec in ((self.prologue, spec.stream_prologue), (self.epilogue, spec.logit_epilogue)):
+            if part is not None:
+                pre = getattr(part_spec, "prefix", "")
+                pre = pre + "." if pre else ""
+                names = part_class(part_spec.kind).expected_tensors(part_spec, spec.hidden_size)
+                part.load({rel: tensors[pre + rel] for rel in names}, rt)
 
     def weight_bytes_read_per_step(self) -> int:
         """Bytes of every weight a step uses once (the embedding table only where it is the head)."""
@@ -88,8 +116,9 @@ class DecoderModel:
                 for v in vars(part).values():
                     add(v)
             total += (n - 1) * (total - before)
-        for v in vars(self.final_norm).values():
-            add(v)
+        for part in self._around():
+            for v in vars(part).values():
+                add(v)
         add(self.head)
         return total
 
@@ -97,6 +126,8 @@ class DecoderModel:
         """Runs the tokens of ctx through the schedule; returns float32 logits [R, V]."""
         with ops.one_stream():           # (the whole step runs on the stream that is current now)
             h = ops.embedding(ctx.token_ids, self.embed)
+            if self.prologue is not None:
+                self.prologue.forward(h, ctx)
             pending = None
             for i, entry in enumerate(self.spec.schedule):
                 pending = self.blocks[entry.layer].forward(h, pending, ctx, bindings[i])
@@ -104,4 +135,7 @@ class DecoderModel:
             if R == 0:
                 return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=h.device)
             x = self.final_norm.forward(h, ctx.rt, delta=pending, rows=ctx.logit_rows)
-            return ops.gemm(x, self.head, out_dtype=torch.float32)
+            logits = ops.gemm(x, self.head, out_dtype=torch.float32)
+            if self.epilogue is not None:
+                logits = self.epilogue.forward(logits, ctx)
+            return logits

@@ -51,7 +51,7 @@ def test_outputs_do_not_depend_on_the_engine_sizes(folders, sizes):
     p = prompts_for(cfg, (1, 7, 16, 30), 2)
     p[3] = p[2] + p[3][16:]                               # the last two share a prefix of 16 tokens
     want = [P.greedy_generate(cfg, w, q, 10) for q in p]
-    base = dict(dtype="float32", block_size=8, max_num_seqs=4, max_model_len=48, prefill_chunk=6)
+    base = dict(dtype="float32", block_size=8, max_num_seqs=4, max_model_len=48, prefill_chunk=6, debug_poison=True)
     base.update(sizes)
     eng = LLMEngine.from_folder(folders["B"], EngineConfig(**base))
     eng.submit(p, max_new_tokens=10, ignore_eos=True)
@@ -89,7 +89,7 @@ def test_bfloat16_generation_on_the_mfma_kernels(folders, sizes, which):
     sequence, or within rounding of it (bfloat16 results depend on the cut in the last bits)."""
     cfg, w = P.read_folder(folders[which])
     prompts = prompts_for(cfg, (150, 33, 70, 201, 16), 6)
-    base = dict(dtype="bfloat16", block_size=16, max_num_seqs=3, max_model_len=320)
+    base = dict(dtype="bfloat16", block_size=16, max_num_seqs=3, max_model_len=320, debug_poison=True)
     base.update(sizes)
     eng = LLMEngine.from_folder(folders[which], EngineConfig(**base))
     eng.submit(prompts, max_new_tokens=40, ignore_eos=True)
@@ -122,6 +122,23 @@ def test_shared_prefix_pages_are_taken_over(folders):
     assert eng.stats()["shared_prefix_tokens"] == 32
     assert res[0].token_ids == P.greedy_generate(cfg, w, a, 4)
     assert res[1].token_ids == P.greedy_generate(cfg, w, b, 4)
+
+
+def test_requests_submitted_together_share_their_beginning(folders):
+    """Two prompts with 32 tokens in common and one that shares nothing, submitted in one call (the
+    reference's prompts 2 and 3 begin alike, main.py:64-68): the second of the pair waits for the
+    first one's pages instead of computing them again, and every output is the plain one."""
+    cfg, w = P.read_folder(folders["B"])
+    common = prompts_for(cfg, (32,), 3)[0]
+    a, b, c = common + [5, 6, 7], prompts_for(cfg, (11,), 8)[0], common + [9]
+    eng = LLMEngine.from_folder(folders["B"], EngineConfig(dtype="float32", block_size=8, max_num_seqs=3,
+                                                           max_model_len=64, prefill_chunk=16, debug_poison=True))
+    eng.submit([a, b, c], max_new_tokens=4, ignore_eos=True)
+    res = eng.run()
+    assert eng.stats()["shared_prefix_tokens"] == 32 and eng.stats()["held_back_for_prefix"] >= 1
+    assert eng.stats()["prefill_tokens"] == len(a) + len(b) + len(c) - 32
+    for r, prompt in zip(res, (a, b, c)):
+        assert r.token_ids == P.greedy_generate(cfg, w, prompt, 4)
 
 
 @pytest.mark.parametrize("dtype,which,page", [("float32", "A", 4), ("bfloat16", "A", 4), ("bfloat16", "E", 16), ("float32", "E", 16)])
@@ -258,7 +275,7 @@ def test_random_engine_sizes_and_prompt_sets(folders, which):
         page = rng.choice([1, 2, 4, 8, 16])
         longest = max(len(p) for p in prompts) + new
         per_request = -(-longest // page)
-        sizes = dict(dtype="float32", block_size=page, max_num_seqs=rng.randint(1, 5),
+        sizes = dict(dtype="float32", block_size=page, max_num_seqs=rng.randint(1, 5), debug_poison=True,
                      num_blocks=rng.choice([per_request + 1, 2 * per_request, per_request * len(prompts) + 4]),
                      max_model_len=longest + rng.choice([0, 3, 50]), max_step_tokens=rng.choice([3, 8, 20, 64, 2048]),
                      prefill_chunk=rng.choice([2, 5, 16, 512]), enable_prefix_sharing=rng.random() < 0.7)

@@ -750,7 +750,7 @@ def test_prefill_attention_kernel(ops, hq, hkv, d, page, window):
             other += list(range(row, row + n))
             portions.append((row, n))
         row += n
-    from qwen_engine_amd.engine.batch import prefill_tiles
+    from qwen_engine_amd.parts.attention import prefill_tiles
     tiles = torch.tensor(prefill_tiles(portions, R), dtype=torch.int32).view(-1, 2).tolist()
     width = max(len(t) for t in tables)
     table = torch.full((len(lens), width), -1, dtype=torch.int32)
@@ -779,7 +779,7 @@ def test_prefill_kernel_one_far_key_decides(ops, key_pos):
     cache, ids = paged_cache(k, v, page, 164, bf)
     n = L - first
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
-    from qwen_engine_amd.engine.batch import prefill_tiles
+    from qwen_engine_amd.parts.attention import prefill_tiles
     tiles = torch.tensor(prefill_tiles([(0, n)], ops.prefill_tile_rows(hq, hkv)), dtype=torch.int32).view(-1, 2).tolist()
     want = P.attention(q.float(), k.float(), v.float(), 1 / math.sqrt(d))
     for groups in (1, 2):

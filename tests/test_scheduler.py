@@ -199,3 +199,50 @@ def test_bad_requests_are_refused():
         sched.add(Request(1, [1], SamplingParams(max_new_tokens=0)))
     with pytest.raises(ValueError):
         sched.add(Request(2, [1], SamplingParams(temperature=-1.0)))
+
+
+def test_requests_that_arrive_together_share_their_beginning():
+    """The reference's prompt pair (main.py:64-68: the third prompt is the beginning of the second),
+    submitted in one batch: the second of the pair waits until the first has computed the pages
+    they have in common and takes them over, a request between them that shares nothing starts
+    at once, and the tokens are the same as without sharing."""
+    common = [50 + (7 * i) % 40 for i in range(22)]          # five full pages of four tokens and a half
+    prompts = [common + [91, 92, 93, 94, 95, 96], common[:20], [3, 1, 4, 1, 5, 9, 2, 6], common + [77]]
+    want = [expected_output(p, 6) for p in prompts]
+    for chunk in (8, 64):
+        sched, cache = make(sharing=True, chunk=chunk, budget=64)
+        reqs = [Request(i, p, SamplingParams(max_new_tokens=6)) for i, p in enumerate(prompts)]
+        for r in reqs:
+            sched.add(r)
+        log = []
+        drive(sched, cache, log)
+        assert [r.output for r in reqs] == want
+        first = [rid for rid, _, _ in log[0]]
+        assert first == [0, 2]                                # 1 and 3 wait for request 0's pages; 2 passes them
+        # request 1 (20 tokens = 5 pages, one token always left: 4 pages taken over), request 3 (5 pages)
+        assert sched.stats["shared_prefix_tokens"] == 16 + 20
+        assert sched.stats["held_back_for_prefix"] >= 2
+        n_prefill = sum(n for step in log for _, n, _ in step) - sched.stats["decode_tokens"]
+        assert n_prefill == sum(len(p) for p in prompts) - 36
+    # without sharing nothing waits
+    sched, cache = make(sharing=False)
+    for i, p in enumerate(prompts):
+        sched.add(Request(i, p, SamplingParams(max_new_tokens=6)))
+    log = []
+    drive(sched, cache, log)
+    assert [rid for rid, _, _ in log[0]] == [0, 1, 2, 3] and sched.stats["held_back_for_prefix"] == 0
+
+
+def test_a_request_held_back_for_a_prefix_goes_on_when_the_other_is_preempted_or_ends():
+    """The running request that the pages were expected from is preempted (too few pages) or ends
+    before it has computed them: the one that waited computes its prompt itself."""
+    common = list(range(30, 46))
+    a, b = common + [1, 2, 3], common + [4, 5]
+    sched, cache = make(num_pages=7, sharing=True, chunk=4, budget=8, max_num_seqs=2)
+    ra, rb = Request(0, a, SamplingParams(max_new_tokens=3)), Request(1, b, SamplingParams(max_new_tokens=3))
+    sched.add(ra)
+    sched.add(rb)
+    drive(sched, cache)
+    assert ra.output == expected_output(a, 3) and rb.output == expected_output(b, 3)
+    assert ra.finish_reason == rb.finish_reason == "length"
+    assert all(pool.num_free + cache.num_kept == pool.num_pages for pool in cache.pools)
