@@ -14,6 +14,7 @@ line is printed:
   roofline   the decode step's bytes (every weight once + the live requests' cache) / time / 8 TB/s
   points     decoded tokens a second at batch 1 and at batch 64
   measured_copy_gbs   what a plain copy of 1 GiB reaches on this device (read + write), for scale
+  measured_mfma_tflops   what register-resident bfloat16 MFMAs reach on this device, for scale
 
 Other sizes and workloads (not what the default line reports):
 
@@ -304,7 +305,11 @@ def main() -> int:
                      "unit": "GB/s", "frac": round(main_run["gbs"] / HBM_PEAK_GBS, 4)},
         "points": points,
         "measured_copy_gbs": round(copy_gbs(), 1),
+        "measured_mfma_tflops": round(ops.mfma_probe() / 1e12, 1),
     }
+    line["prefill"]["frac_of_measured"] = round(prefill["frac"] * PEAK_FLOPS[args.dtype] / (line["measured_mfma_tflops"] * 1e12), 4) \
+        if args.dtype == "bf16" else None
+    line["roofline"]["frac_of_measured_copy"] = round(main_run["gbs"] / line["measured_copy_gbs"], 4)
     print(json.dumps(line), flush=True)
     return 0
 

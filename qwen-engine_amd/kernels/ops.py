@@ -73,6 +73,8 @@ def load_library():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = ctypes.c_int
+    lib.qe_mfma_probe.argtypes = [vp, i32, i32, ctypes.POINTER(ctypes.c_double), vp]
+    lib.qe_mfma_probe.restype = ctypes.c_int
     lib.qe_argmax_workspace_bytes.argtypes = [i32, i32]
     lib.qe_argmax_workspace_bytes.restype = ctypes.c_long
     lib.qe_attention_decode_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]
@@ -641,3 +643,20 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tenso
     _check(lib.qe_sample(logits.data_ptr(), temperature.data_ptr(), uniform.data_ptr(), out.data_ptr(),
                          R, V, _stream()), "sample")
     return out
+
+
+def mfma_probe(blocks: int = 512, iters: int = 20000, device="cuda:0") -> float:
+    """Floating-point operations a second that register-resident bfloat16 MFMAs (32 x 32 x 16) reach
+    on this device, eight waves a compute unit with 512 blocks: a measured peak, for scale."""
+    lib = load_library()
+    out = torch.empty(blocks * 256, dtype=torch.float32, device=device)
+    flops = ctypes.c_double(0.0)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = 0.0
+    for rep in range(3):                                   # (the first repetition brings the clock up)
+        start.record()
+        _check(lib.qe_mfma_probe(out.data_ptr(), int(blocks), int(iters), ctypes.byref(flops), _stream()), "mfma probe")
+        end.record()
+        end.synchronize()
+        best = max(best, flops.value / (start.elapsed_time(end) * 1e-3))
+    return best

@@ -41,6 +41,14 @@ class TensorInfo(NamedTuple):
     role: str = "matrix"   # "matrix" keeps the stored element type in bfloat16 mode; "vector" is held in 32-bit
 
 
+def sub_tensors(tensors, prefix: str):
+    """The tensors whose names begin with ``prefix``, under their names without it.  A mapping
+    that reads tensors on demand (it has ``subset``) stays one: nothing is read here."""
+    if hasattr(tensors, "subset"):
+        return tensors.subset(prefix)
+    return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
+
+
 @dataclass
 class Runtime:
     """Where and in which element type the engine computes."""

@@ -8,7 +8,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import CacheBinding, Runtime, TensorInfo
+from .base import CacheBinding, Runtime, TensorInfo, sub_tensors
 from .registry import build_part, part_class, register_part
 
 def _names(spec):
@@ -43,8 +43,7 @@ class PreNormBlock:
 
     def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
         for name, part in zip(_names(self.spec), (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)):
-            pre = name + "."
-            part.load({k[len(pre):]: v for k, v in tensors.items() if k.startswith(pre)}, rt)
+            part.load(sub_tensors(tensors, name + "."), rt)
 
     def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], ctx, binding: CacheBinding) -> torch.Tensor:
         """h: 32-bit residual stream (updated in place).  pending: branch output not yet

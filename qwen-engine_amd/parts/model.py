@@ -10,7 +10,7 @@ import torch
 from ..cache.plan import CachePlan, plan_cache
 from ..config.spec import ModelSpec
 from ..kernels import ops
-from .base import CacheBinding, Runtime, TensorInfo
+from .base import CacheBinding, Runtime, TensorInfo, sub_tensors
 from .registry import build_part, part_class
 
 
@@ -84,10 +84,9 @@ class DecoderModel:
         self.rt = rt
         self.embed = rt.place_matrix(tensors[spec.embed_name])
         for layer, block in zip(spec.layers, self.blocks):
-            pre = layer.prefix + "."
-            block.load({k[len(pre):]: v for k, v in tensors.items() if k.startswith(pre)}, rt)
+            block.load(sub_tensors(tensors, layer.prefix + "."), rt)
         base = spec.final_norm_name[:-len(".weight")] if spec.final_norm_name.endswith(".weight") else spec.final_norm_name
-        self.final_norm.load({k[len(base) + 1:]: v for k, v in tensors.items() if k.startswith(base + ".")}, rt)
+        self.final_norm.load(sub_tensors(tensors, base + "."), rt)
         self.head = self.embed if spec.tie_head else rt.place_matrix(tensors[spec.head_name])
         for part, part_spec in ((self.prologue, spec.stream_prologue), (self.epilogue, spec.logit_epilogue)):
             if part is not None:

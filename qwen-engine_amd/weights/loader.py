@@ -9,7 +9,8 @@ wrong shapes are reported together in one error.
 from __future__ import annotations
 
 import os
-from typing import Dict, List, Tuple
+from collections.abc import Mapping
+from typing import Dict, Iterator, List, Tuple
 
 import torch
 
@@ -42,8 +43,37 @@ def safetensors_files(folder: str) -> List[str]:
     return [os.path.join(folder, f) for f in files]
 
 
-def read_checked(folder: str, expected: Dict[str, TensorInfo], tied_head_name: str = "") -> Dict[str, torch.Tensor]:
-    """All expected tensors of the folder, as stored, on the CPU.
+class LazyTensors(Mapping):
+    """The checked tensors of a model folder by name; a tensor is read from its file when it is
+    asked for, as stored, onto the CPU, and nothing of it is kept here.  The model asks part by
+    part, so that the host never holds more than one part's tensors (the reference reads every
+    tensor of the checkpoint into one dict first, src/models/qwen3/utils.py:77-82)."""
+
+    def __init__(self, handles, where: Dict[str, int], names: Dict[str, str]):
+        self._handles, self._where, self._names = handles, where, names   # names: name here -> name in the files
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        real = self._names[name]
+        return self._handles[self._where[real]].get_tensor(real)
+
+    def __iter__(self) -> Iterator[str]:
+        return iter(self._names)
+
+    def __contains__(self, name) -> bool:       # (asking whether a tensor is there reads nothing)
+        return name in self._names
+
+    def __len__(self) -> int:
+        return len(self._names)
+
+    def subset(self, prefix: str) -> "LazyTensors":
+        """The tensors whose names begin with ``prefix``, under their names without it."""
+        return LazyTensors(self._handles, self._where,
+                           {k[len(prefix):]: real for k, real in self._names.items() if k.startswith(prefix)})
+
+
+def read_checked(folder: str, expected: Dict[str, TensorInfo], tied_head_name: str = "") -> LazyTensors:
+    """Checks the folder's safetensors headers against the expected tensors and returns them as a
+    mapping that reads each tensor when it is asked for (as stored, on the CPU).
 
     ``tied_head_name``: a tensor of this name is tolerated though not expected (a
     checkpoint with tied embeddings may store the head again); it is not read.
@@ -65,4 +95,4 @@ def read_checked(folder: str, expected: Dict[str, TensorInfo], tied_head_name: s
                    if n in where and shapes[n] != tuple(expected[n].shape))
     if missing or unexpected or wrong:
         raise WeightError(folder, missing, unexpected, wrong)
-    return {name: handles[where[name]].get_tensor(name) for name in expected}
+    return LazyTensors(handles, where, {name: name for name in expected})

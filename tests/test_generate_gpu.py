@@ -221,6 +221,42 @@ def test_command_line(folders, tmp_path):
     assert stats["decode_tokens"] == 8 and stats["prefill_tokens"] == 6
 
 
+def test_text_prompts_through_the_command_line(folders, tmp_path):
+    """Raw text goes through the folder's tokenizer.json without a template, and what is printed is
+    the decoded prompt + output without special tokens (src/engine/llm_engine.py:52-55,67-73).  The
+    tokenizer is a word-level one written here, with a vocabulary as large as the model's."""
+    import shutil
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import Whitespace
+    folder = str(tmp_path / "model_with_tokenizer")
+    shutil.copytree(folders["A"], folder)
+    cfg, w = P.read_folder(folder)
+    words = ["[UNK]", "[EOS]"] + [f"w{i}" for i in range(cfg["vocab_size"] - 2)]
+    tok = Tokenizer(WordLevel({word: i for i, word in enumerate(words)}, unk_token="[UNK]"))
+    tok.pre_tokenizer = Whitespace()
+    tok.add_special_tokens(["[UNK]", "[EOS]"])
+    tok.save(os.path.join(folder, "tokenizer.json"))
+    texts = ["w5 w17 w3 w200", "w9 w9 w31 never_seen w4 w77 w12"]
+    ids = [tok.encode(t).ids for t in texts]
+    assert ids[0] == [7, 19, 5, 202] and ids[1][3] == 0                  # the unknown word
+    cmd = [sys.executable, os.path.join(ROOT, "main.py"), "--model", folder, "--prompt", texts[0], "--prompt", texts[1],
+           "--max-new-tokens", "6", "--max-num-seqs", "2", "--max-model-len", "32", "--block-size", "4",
+           "--model-dtype", "float32", "--ignore-eos"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = r.stdout.splitlines()
+    for t, p in zip(texts, ids):
+        out = P.greedy_generate(cfg, w, p, 6)
+        assert f"Prompt: {tok.decode(p, skip_special_tokens=True)}" in lines
+        assert tok.decode(p + out, skip_special_tokens=True) in lines        # specials ([UNK], [EOS]) are left out
+    # the Python entry point with text, and a request that stops at the end-of-sequence token
+    res = generate(folder, [texts[0]], SamplingParams(max_new_tokens=6, ignore_eos=True),
+                   EngineConfig(dtype="float32", block_size=4, max_model_len=32))
+    assert res[0].prompt_token_ids == ids[0]
+    assert res[0].text == tok.decode(ids[0] + res[0].token_ids, skip_special_tokens=True)
+
+
 def test_decode_batches_between_recorded_sizes_are_filled_up(folders):
     """11 requests decode through the graph recorded for 16 rows, and after two of them have ended
     the 9 that remain replay the same graph: the logits are those of a runner without graphs."""

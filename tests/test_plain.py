@@ -188,5 +188,53 @@ def test_norm_comes_before_rotation_and_only_without_bias(tmp_path):
     assert not torch.allclose(a, b, rtol=1e-3, atol=1e-5)
 
 
+def test_the_per_head_norm_runs_before_the_rotation(tmp_path):
+    """model.py:204-208: q and k are normed per head, then rotated.  With norm weights that are zero on
+    the first half of the head, the normed head is [0 | x2], and its rotation [-sin x2 | cos x2]: the
+    score of a query at i and a key at j is sum_d cos((i - j) f_d) x2q_d x2k_d, a function of the
+    distance only.  Had the rotation come first, the weights would have cut the rotated head to
+    [0 | sin x1 + cos x2] and the scores would be others.  The expected output is formed here from
+    that closed form, without the functions that rotate."""
+    folder = make_folder(tmp_path, "B", dtype=torch.float32, std=0.3)
+    cfg, w = P.read_folder(folder)
+    w = dict(w)
+    hq, hkv, d, eps = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["rms_norm_eps"]
+    half = d // 2
+    mask = torch.cat([torch.zeros(half), torch.ones(half)])
+    pre = "model.layers.0.self_attn"
+    w[f"{pre}.q_norm.weight"] = mask * (1.0 + 0.1 * rand(d, seed=41))
+    w[f"{pre}.k_norm.weight"] = mask * (1.0 + 0.1 * rand(d, seed=42))
+    T = 9
+    x = rand(T, cfg["hidden_size"], seed=40)
+    pos = torch.arange(T) + 3                               # no token at position 0, where a rotation does nothing
+    theta = P.rope_theta_of(cfg)
+    table = P.rope_table(theta, d, 64)
+    got = P.attention_block(x, pos, w, "model.layers.0", cfg, table)
+
+    q = (x @ w[f"{pre}.q_proj.weight"].t()).view(T, hq, d).double()
+    k = (x @ w[f"{pre}.k_proj.weight"].t()).view(T, hkv, d).double()
+    v = (x @ w[f"{pre}.v_proj.weight"].t()).view(T, hkv, d).double()
+    x2q = (q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * w[f"{pre}.q_norm.weight"].double())[..., half:]
+    x2k = (k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * w[f"{pre}.k_norm.weight"].double())[..., half:]
+    f = theta ** (-torch.arange(half, dtype=torch.float64) / half)
+    dist = (pos[:, None] - pos[None, :]).double()
+    cosd = torch.cos(dist[:, :, None] * f)                  # [i, j, d]
+    out = torch.zeros(T, hq, d, dtype=torch.float64)
+    for h in range(hq):
+        kv = h // (hq // hkv)
+        s = torch.einsum("id,jd,ijd->ij", x2q[:, h], x2k[:, kv], cosd) / (d ** 0.5)
+        s = s.masked_fill(dist < 0, float("-inf"))
+        out[:, h] = torch.softmax(s, dim=-1) @ v[:, kv]
+    want = out.reshape(T, hq * d) @ w[f"{pre}.o_proj.weight"].double().t()
+    torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=1e-5)
+    # and the closed form is not blind to the order: with the rotation first the result is another
+    qr = P.apply_rope(table, pos, (x @ w[f"{pre}.q_proj.weight"].t()).view(T, hq, d))
+    kr = P.apply_rope(table, pos, (x @ w[f"{pre}.k_proj.weight"].t()).view(T, hkv, d))
+    qn = P.rms_norm(qr, w[f"{pre}.q_norm.weight"], eps)
+    kn = P.rms_norm(kr, w[f"{pre}.k_norm.weight"], eps)
+    other = P.attention(qn, kn, v.float(), 1.0 / d ** 0.5, pos, pos).reshape(T, hq * d) @ w[f"{pre}.o_proj.weight"].t()
+    assert float((other.double() - want).abs().max()) > 100 * float((got.double() - want).abs().max()) + 1e-3
+
+
 def test_greedy_takes_the_lowest_index_on_ties():
     assert P.greedy(torch.tensor([[1.0, 3.0, 3.0, 2.0], [0.0, 0.0, 0.0, 0.0]])) == [1, 0]

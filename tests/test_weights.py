@@ -118,3 +118,28 @@ def test_placement_keeps_stored_precision():
     assert torch.equal(f32.place_matrix(m16), m16.float())      # exact
     assert bf.place_matrix(table).dtype == torch.int32
     assert bf.place_vector(m16[0]).dtype == torch.float32
+
+
+def test_tensors_are_read_part_by_part(tmp_path, monkeypatch):
+    """read_checked opens the files and checks names and shapes, but reads no tensor; the model then
+    asks for each tensor once, part by part (the reference holds the whole checkpoint on the host
+    first, utils.py:77-82), and the parts see their tensors under their own names."""
+    from qwen_engine_amd.parts import DecoderModel
+    from qwen_engine_amd.weights.loader import LazyTensors
+    cfg = Qwen3Config.from_dict(TINY_B)
+    folder = write_model_folder(str(tmp_path / "m"), cfg, 3)
+    spec = cfg.to_model_spec()
+    read = []
+    real = LazyTensors.__getitem__
+    monkeypatch.setattr(LazyTensors, "__getitem__", lambda self, name: (read.append(self._names[name]), real(self, name))[1])
+    got = read_checked(folder, expected_tensors(spec))
+    assert read == [] and len(got) == len(expected_tensors(spec))
+    layer0 = got.subset("model.layers.0.")
+    assert "self_attn.q_proj.weight" in layer0 and "mlp.down_proj.weight" in layer0 and read == []
+    assert all(not k.startswith("model.") for k in layer0)
+    model = DecoderModel(spec)
+    model.load(got, Runtime(torch.device("cpu"), torch.float32))
+    assert sorted(read) == sorted(expected_tensors(spec))          # every tensor exactly once
+    assert read[0] == "model.embed_tokens.weight" and read[-1] == "lm_head.weight"
+    t = random_tensors(cfg, 3)
+    assert torch.equal(model.blocks[2].mixer.w_o, t["model.layers.2.self_attn.o_proj.weight"].float())
