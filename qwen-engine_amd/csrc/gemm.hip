@@ -5,7 +5,9 @@ int qe_gemm_generic(const void* x, const void* w, const float* bias, void* out, 
                     int dt_a, int dt_w, int dt_o, hipStream_t stream);
 bool qe_gemm_skinny_ok(int M, int N, int K, int dt_a, int dt_w);
 int qe_gemm_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                   int dt_o, int epilogue, int splits, hipStream_t stream);
+                   int dt_o, int epilogue, int splits, const float* norm_w, float norm_eps,
+                   const float* delta, int n_delta, float* h_out, hipStream_t stream);
+bool qe_gemm_skinny_norm_ok(int M, int N, int K);
 int qe_gemm_skinny_splits(int N, int K);
 bool qe_gemm_mfma_ok(int M, int N, int K, int dt_a, int dt_w);
 int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
@@ -21,6 +23,13 @@ enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3, EPI_S
 // 1 if the fused epilogues (add into the 32-bit residual stream; silu(gate) * up) can be used
 extern "C" int qe_gemm_fused_supported(int M, int N, int K, int dt_a, int dt_w) {
     return qe_gemm_skinny_ok(M, N, K, dt_a, dt_w) ? 1 : 0;
+}
+
+// 1 if the product can take the RMSNorm before it as its prologue (qe_gemm's norm_w): x is then the
+// 32-bit stream; few rows, bfloat16 weights (N counts the weight rows)
+extern "C" int qe_gemm_norm_supported(int M, int N, int K, int dt_w) {
+    return (dt_w == QE_BF16 && qe_gemm_skinny_ok(M, N, K, QE_BF16, dt_w) && qe_gemm_skinny_norm_ok(M, N, K) &&
+            !((long)N * K >= (16L << 20) && M > 16)) ? 1 : 0;
 }
 
 // 1 if epilogue 4 (silu-mul over interleaved gate|up rows) can be used: N counts the outputs
@@ -77,13 +86,29 @@ extern "C" int qe_gemm_branch_splits(int M, int N, int K, int dt_a, int dt_w) {
 // 3: out is float [splits, M, N], partial products along K to be summed over the first index.
 // 4: as 2 with the gate and up rows of w interleaved in blocks of 32 (gate 0..31, up 0..31, ...);
 //    taken by the kernel for few rows and by the tiled one.
+// norm_w (or null): the weight of an RMSNorm (eps norm_eps) that stands before the product: x is then the
+// 32-bit stream [M, K]; needs qe_gemm_norm_supported and epilogue 0, 2 or 4.  With it, delta (or null):
+// n_delta float tensors [M, K] one after the other that are added to the stream's rows, in order, before
+// the norm (the partial products of the branch before); the sums are written to h_out [M, K] (not x).
 // algo: 0 = choose, 1 = the generic 32-bit kernel, 2 = an MFMA kernel (the one for few rows up to
 // 64 rows, except against a very wide matrix from 17 rows on; else the tiled one) or an error if
 // neither takes the operands.
 extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                       int dt_a, int dt_w, int dt_o, int algo, int epilogue, int splits, hipStream_t stream) {
+                       int dt_a, int dt_w, int dt_o, int algo, int epilogue, int splits,
+                       const float* norm_w, float norm_eps, const float* delta, int n_delta, float* h_out,
+                       hipStream_t stream) {
     QE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     if (M == 0) return 0;
+    QE_REQUIRE(norm_w || (!delta && !h_out), "gemm: partial products to add go with the norm prologue");
+    if (norm_w) {
+        // x is the 32-bit stream; the kernel for few rows norms it itself
+        const int n_rows = (epilogue == EPI_SILU_MUL || epilogue == EPI_SILU_MUL_IL) ? 2 * N : N;
+        QE_REQUIRE(dt_a == QE_F32 && qe_gemm_norm_supported(M, n_rows, K, dt_w),
+                   "gemm: M=%d N=%d K=%d is not taken with the norm as prologue", M, N, K);
+        QE_REQUIRE(epilogue == EPI_STORE || epilogue == EPI_SILU_MUL || epilogue == EPI_SILU_MUL_IL,
+                   "gemm: the norm prologue goes with the store and silu-mul epilogues");
+        return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, epilogue, 1, norm_w, norm_eps, delta, n_delta, h_out, stream);
+    }
     const bool skinny = qe_gemm_skinny_ok(M, N, K, dt_a, dt_w);
     const bool tiled = qe_gemm_mfma_ok(M, N, K, dt_a, dt_w);
     if (epilogue == EPI_SILU_MUL_IL && (!skinny || tiled_for_few_rows(M, 2 * N, K, dt_a, dt_w))) {
@@ -97,7 +122,7 @@ extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* ou
     }
     if (epilogue != EPI_STORE) {
         QE_REQUIRE(skinny, "gemm: M=%d N=%d K=%d with these element types is not taken by the kernel for few rows", M, N, K);
-        return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, epilogue, splits, stream);
+        return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, epilogue, splits, nullptr, 0.f, nullptr, 0, nullptr, stream);
     }
     QE_REQUIRE(algo == ALGO_AUTO || algo == ALGO_GENERIC || algo == ALGO_MFMA || algo > ALGO_TILE, "gemm: unknown algo %d", algo);
     if (algo > ALGO_TILE) {
@@ -106,7 +131,7 @@ extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* ou
     }
     if (algo != ALGO_GENERIC) {
         if (skinny && !tiled_for_few_rows(M, N, K, dt_a, dt_w))
-            return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, EPI_STORE, 1, stream);
+            return qe_gemm_skinny(x, w, bias, out, M, N, K, dt_o, EPI_STORE, 1, nullptr, 0.f, nullptr, 0, nullptr, stream);
         if (tiled) return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, 0, false, 1, stream);
         QE_REQUIRE(algo == ALGO_AUTO, "gemm: M=%d N=%d K=%d with these element types is not taken by an MFMA kernel", M, N, K);
     }

@@ -12,6 +12,18 @@
 // Epilogues: store (+ bias); add into a 32-bit residual stream; silu(gate) * up, where W holds
 // the gate rows followed by the up rows and a block owns 16 of each; 32-bit partial products
 // of a product cut along K over several blocks (for matrices with few rows, to fill the chip).
+//
+// Prologue (up to 16 rows): the RMSNorm that stands before the product.  x is then the 32-bit
+// residual stream; every block norms the rows itself (sum of squares, rsqrt, weight: the same
+// arithmetic in the same order as the norm kernel, so the same bits), leaves them as bfloat16 in
+// shared memory and takes its operands from there.  A decode step is a chain of short dependent
+// kernels, each of which costs a few microseconds whatever it does: the norm as a kernel of
+// its own costs as much as the product behind it.
+//
+// WAVES: waves of a block, which split K between them: 4, or 8 for gate|up with up to 16 rows
+// (a block then has all of its share of the weights in flight at once).  (A product that adds
+// into the stream itself with 16 waves a block, instead of partial products over 256 blocks, was
+// tried for o and down: its 64 blocks take 6.7 us where the partial products take 4.3.)
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -19,26 +31,170 @@ typedef __attribute__((ext_vector_type(4))) float floatx4;
 
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SILU_MUL = 2, EPI_PARTIAL = 3, EPI_SILU_MUL_IL = 4 };
 
+// The prologue of a product of few rows (M <= 16): the rows of the 32-bit stream hs [M][K], with the
+// n_delta partial products delta[s][M][K] of the branch before added in the order of s (the residual
+// sum), normed as rmsnorm_regs_kernel norms them and left as bfloat16 in xs [M][K + 8].  That kernel's
+// block has tn = min(256, K / 4 rounded up to whole waves) threads, thread t owns the elements
+// (t + i tn) 4 .. + 3, the sum of squares runs over i, then over the lanes of a wave, then over the
+// waves in order; the same here (threads beyond tn add zeros), so the bits are the same.  If
+// h_out is given, this block also writes the summed rows there (one block of the grid does).
+//
+// Rows of up to 1024 elements (one group of four a thread), MB >= M rows: everything is asked for in
+// as few trips to memory as the registers allow (the rows and the first partial products
+// together, then SB partial products of all rows at a time), with addresses that are always valid
+// (a row or a partial product beyond the last reads the last again and is not used), so that no
+// branch stands between the loads.  The rows stay in registers between the two passes.
+template <int WAVES, int MB>
+__device__ __forceinline__ void norm_short_rows(const float* __restrict__ hs, const float* __restrict__ delta,
+                                                int n_delta, float* __restrict__ h_out, const float* __restrict__ norm_w,
+                                                float norm_eps, bf16_t* xs, int M, int K, int KP, float (*ss_red)[16],
+                                                bool mine) {
+    constexpr int SB = MB <= 4 ? 8 : (MB <= 8 ? 4 : 2);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = (int)threadIdx.x * 4;
+    const bool have = mine && c < K;                         // (threads beyond K / 4 have nothing)
+    const int cc = have ? c : 0;
+    const long dstride = (long)M * K;
+    float v[MB][4];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) Vec4<float>::load(hs + (long)min(m, M - 1) * K + cc, v[m]);
+    float wv[4];
+    Vec4<float>::load(norm_w + cc, wv);
+    for (int s0 = 0; s0 < n_delta; s0 += SB) {
+        float d[SB][MB][4];
+#pragma unroll
+        for (int j = 0; j < SB; ++j)
+#pragma unroll
+            for (int m = 0; m < MB; ++m)
+                Vec4<float>::load(delta + min(s0 + j, n_delta - 1) * dstride + (long)min(m, M - 1) * K + cc, d[j][m]);
+#pragma unroll
+        for (int j = 0; j < SB; ++j)
+            if (s0 + j < n_delta) {
+#pragma unroll
+                for (int m = 0; m < MB; ++m)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[m][e] += d[j][m][e];
+            }
+    }
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ss += v[m][e] * v[m][e];
+        const float t = wave_sum(have ? ss : 0.f);
+        if (lane == 0) ss_red[wave][m] = t;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        if (m < M && have) {
+            float tot = 0.f;
+            for (int i = 0; i < WAVES; ++i) tot += ss_red[i][m];
+            const float rstd = rsqrtf(tot / (float)K + norm_eps);
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = v[m][e] * rstd * wv[e];
+            Vec4<bf16_t>::store(xs + (long)m * KP + c, o);
+            if (h_out) Vec4<float>::store(h_out + (long)m * K + c, v[m]);
+        }
+    }
+}
+
+template <int WAVES>
+__device__ __forceinline__ void norm_rows_into_lds(const float* __restrict__ hs, const float* __restrict__ delta,
+                                                   int n_delta, float* __restrict__ h_out, const float* __restrict__ norm_w,
+                                                   float norm_eps, bf16_t* xs, int M, int K, int KP) {
+    __shared__ float ss_red[WAVES][16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int tn = ((K / 4 + 63) / 64) * 64;
+    if (tn > 256) tn = 256;
+    const int nv = (K / 4 + tn - 1) / tn;
+    const bool mine = (int)threadIdx.x < tn;
+    const long dstride = (long)M * K;
+    if (nv == 1) {
+        // (every wave of the block goes through the same barriers; the waves beyond the norm's own
+        // block have nothing: they read the first elements again and add zeros)
+        if (M <= 1) norm_short_rows<WAVES, 1>(hs, delta, n_delta, h_out, norm_w, norm_eps, xs, M, K, KP, ss_red, mine);
+        else if (M <= 2) norm_short_rows<WAVES, 2>(hs, delta, n_delta, h_out, norm_w, norm_eps, xs, M, K, KP, ss_red, mine);
+        else if (M <= 4) norm_short_rows<WAVES, 4>(hs, delta, n_delta, h_out, norm_w, norm_eps, xs, M, K, KP, ss_red, mine);
+        else if (M <= 8) norm_short_rows<WAVES, 8>(hs, delta, n_delta, h_out, norm_w, norm_eps, xs, M, K, KP, ss_red, mine);
+        else norm_short_rows<WAVES, 16>(hs, delta, n_delta, h_out, norm_w, norm_eps, xs, M, K, KP, ss_red, mine);
+    } else {
+        // longer rows: two passes over the memory (the second finds it in the cache)
+        for (int m = 0; m < M; ++m) {
+            float ss = 0.f;
+            if (mine) {
+                for (int i = 0; i < nv; ++i) {
+                    const int c = ((int)threadIdx.x + i * tn) * 4;
+                    if (c < K) {
+                        float v[4], d[4];
+                        Vec4<float>::load(hs + (long)m * K + c, v);
+                        for (int s = 0; s < n_delta; ++s) {
+                            Vec4<float>::load(delta + s * dstride + (long)m * K + c, d);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] += d[e];
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) ss += v[e] * v[e];
+                    }
+                }
+            }
+            const float t = wave_sum(ss);
+            if (lane == 0) ss_red[wave][m] = t;
+        }
+        __syncthreads();
+        for (int m = 0; m < M; ++m) {
+            if (!mine) continue;
+            float tot = 0.f;
+            for (int i = 0; i < WAVES; ++i) tot += ss_red[i][m];
+            const float rstd = rsqrtf(tot / (float)K + norm_eps);
+            for (int i = 0; i < nv; ++i) {
+                const int c = ((int)threadIdx.x + i * tn) * 4;
+                if (c < K) {
+                    float v[4], d[4], wv[4], o[4];
+                    Vec4<float>::load(hs + (long)m * K + c, v);
+                    for (int s = 0; s < n_delta; ++s) {
+                        Vec4<float>::load(delta + s * dstride + (long)m * K + c, d);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += d[e];
+                    }
+                    Vec4<float>::load(norm_w + c, wv);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = v[e] * rstd * wv[e];
+                    Vec4<bf16_t>::store(xs + (long)m * KP + c, o);
+                    if (h_out) Vec4<float>::store(h_out + (long)m * K + c, v);
+                }
+            }
+        }
+    }
+    __syncthreads();
+}
+
 // grid (N / (16 NT), S): block (bx, s) sums the chunks [s * cps, (s + 1) * cps) of K.  With S > 1 the
 // epilogue is EPI_PARTIAL: 32-bit partial products out[s][M][N] that the consumer adds up in the
 // order of s (the fused residual-add + norm kernel does), so the sum has one fixed order.
 // NT: tiles of 16 rows of W a block owns.  Every wave reads the activations of its chunks itself
 // (M rows against the block's 16 NT rows of W), so with more than 16 rows of activations most of
 // what a block reads is activations, from the L2; two tiles a block halve that.
-template <int MT, int NT, int EPI, typename TO>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    TO* __restrict__ out, int M, int N, int K, int cps) {
+template <int MT, int NT, int EPI, typename TO, int WAVES, bool NORM>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
+    const void* __restrict__ x_in, const bf16_t* __restrict__ w, const float* __restrict__ bias,
+    TO* __restrict__ out, int M, int N, int K, int cps, const float* __restrict__ norm_w, float norm_eps,
+    const float* __restrict__ delta, int n_delta, float* __restrict__ h_out) {
     constexpr bool SILU = EPI == EPI_SILU_MUL || EPI == EPI_SILU_MUL_IL;
     constexpr int NW = SILU ? 2 : 1;   // weight tiles per tile of outputs
-    constexpr int U = (MT == 1 && !SILU && NT == 1) ? 8 : ((MT <= 2) ? 4 : 2);   // chunks whose loads are issued together
-    __shared__ float red[4][NT][NW][MT][64][4];
+    // chunks whose loads are issued together
+    constexpr int U = (MT == 1 && WAVES >= 8) ? (SILU ? 4 : 8) : ((MT == 1 && !SILU && NT == 1) ? 8 : ((MT <= 2) ? 4 : 2));
+    __shared__ float red[WAVES][NT][NW][MT][64][4];
+    extern __shared__ __align__(16) unsigned char dyn_lds[];       // NORM: the normed rows, bfloat16 [M][K + 8]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r = lane & 15;
     const int n0 = blockIdx.x * 16 * NT;
     const int nchunks = K / 32;
     const int c_begin = blockIdx.y * cps;
     const int c_end = min(nchunks, c_begin + cps);
+    const bf16_t* x = (const bf16_t*)x_in;
+    const int KP = K + 8;                                            // padded row of the normed copy
 
     floatx4 acc[NT][NW][MT];
 #pragma unroll
@@ -66,21 +222,33 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
         tok_ok[j] = j * 16 + r < M;
-        xrow[j] = x + (long)(tok_ok[j] ? j * 16 + r : 0) * K + g * 8;
+        xrow[j] = (NORM ? (const bf16_t*)dyn_lds : x) + (long)(tok_ok[j] ? j * 16 + r : 0) * (NORM ? KP : K) + g * 8;
     }
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-    for (int c = c_begin + wave; c < c_end; c += 4 * U) {
-        bf16x8 a0[U][NT], a1[U][NT], b[U][MT];
+    // The weights of the first round are asked for before the prologue: they come from HBM and do
+    // not depend on it, so the norm runs while they travel.
+    bf16x8 a0[U][NT], a1[U][NT];
+    int c = c_begin + wave;
+#define QE_LOAD_W()                                                                                    \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                    \
+        const int cc = c + WAVES * u;                                                                  \
+        const bool ok = cc < c_end;                                                                    \
+        _Pragma("unroll") for (int q = 0; q < NT; ++q) {                                               \
+            a0[u][q] = (ok && row_ok[q]) ? *(const bf16x8*)(wrow0[q] + cc * 32) : zero;                \
+            if (SILU) a1[u][q] = (ok && row_ok[q]) ? *(const bf16x8*)(wrow1[q] + cc * 32) : zero;      \
+        }                                                                                              \
+    }
+    if (c < c_end) { QE_LOAD_W() }
+    if (NORM)
+        norm_rows_into_lds<WAVES>((const float*)x_in, delta, n_delta, (blockIdx.x == 0 && blockIdx.y == 0) ? h_out : nullptr,
+                                  norm_w, norm_eps, (bf16_t*)dyn_lds, M, K, KP);
+    while (c < c_end) {
+        bf16x8 b[U][MT];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int cc = c + 4 * u;
+            const int cc = c + WAVES * u;
             const bool ok = cc < c_end;
-#pragma unroll
-            for (int q = 0; q < NT; ++q) {
-                a0[u][q] = (ok && row_ok[q]) ? *(const bf16x8*)(wrow0[q] + cc * 32) : zero;
-                if (SILU) a1[u][q] = (ok && row_ok[q]) ? *(const bf16x8*)(wrow1[q] + cc * 32) : zero;
-            }
 #pragma unroll
             for (int j = 0; j < MT; ++j) b[u][j] = (ok && tok_ok[j]) ? *(const bf16x8*)(xrow[j] + cc * 32) : zero;
         }
@@ -94,7 +262,10 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
                     if (SILU)
                         acc[q][1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[u][q], b[u][j], acc[q][1][j], 0, 0, 0);
                 }
+        c += WAVES * U;
+        if (c < c_end) { QE_LOAD_W() }
     }
+#undef QE_LOAD_W
 #pragma unroll
     for (int q = 0; q < NT; ++q)
 #pragma unroll
@@ -104,16 +275,20 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
 #pragma unroll
                 for (int i = 0; i < 4; ++i) red[wave][q][a][j][lane][i] = acc[q][a][j][i];
     __syncthreads();
-    // wave w finishes the (output tile, token tile) pairs w, w + 4, ...
-    for (int qj = wave; qj < NT * MT; qj += 4) {
+    // wave w finishes the (output tile, token tile) pairs w, w + WAVES, ...: the waves' sums in their order
+    for (int qj = wave; qj < NT * MT; qj += WAVES) {
         const int q = qj / MT, j = qj % MT;
         float v[NW][4];
 #pragma unroll
         for (int a = 0; a < NW; ++a)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                v[a][i] = red[0][q][a][j][lane][i] + red[1][q][a][j][lane][i] + red[2][q][a][j][lane][i] +
+            for (int i = 0; i < 4; ++i) {
+                float t = red[0][q][a][j][lane][i] + red[1][q][a][j][lane][i] + red[2][q][a][j][lane][i] +
                           red[3][q][a][j][lane][i];
+#pragma unroll
+                for (int ww = 4; ww < WAVES; ++ww) t += red[ww][q][a][j][lane][i];
+                v[a][i] = t;
+            }
         const int t = j * 16 + r;          // lane (g, r): token t, rows n0 + q * 16 + g * 4 + i
         if (t >= M) continue;
 #pragma unroll
@@ -138,9 +313,20 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
     }
 }
 
+// Shared memory of the normed rows: M rows of K + 8 bfloat16.
+static size_t norm_lds_bytes(int M, int K) { return (size_t)M * (K + 8) * 2; }
+// (a compute unit of gfx950 has 160 KB of shared memory; the kernel's own arrays take up to 17 KB of it)
+#define QE_SKINNY_MAX_NORM_LDS (136 * 1024)
+
+// true if the product can take the norm before it as its prologue
+bool qe_gemm_skinny_norm_ok(int M, int N, int K) {
+    return M >= 1 && M <= 16 && K % 32 == 0 && K >= 32 && K <= 8192 && norm_lds_bytes(M, K) <= QE_SKINNY_MAX_NORM_LDS;
+}
+
 template <int EPI, typename TO>
 static int launch_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                         int splits, hipStream_t stream) {
+                         int splits, const float* norm_w, float norm_eps, const float* delta, int n_delta, float* h_out,
+                         hipStream_t stream) {
     const int cps = qe_cdiv(K / 32, splits);
     const int mt = qe_cdiv(M, 16);
     constexpr bool SILU = EPI == EPI_SILU_MUL || EPI == EPI_SILU_MUL_IL;
@@ -148,10 +334,31 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
     // enough all the same (with silu.mul a tile of outputs is two tiles of W already: only up to 32 rows)
     const bool two = mt >= 2 && (!SILU || mt <= 2) && (long)qe_cdiv(N, 32) * splits >= 256;
     const dim3 grid(qe_cdiv(N, two ? 32 : 16), splits);
-#define QE_SKINNY(MT_, NT_)                                                                            \
-    gemm_skinny_kernel<MT_, NT_, EPI, TO><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, \
-                                                                    (TO*)out, M, N, K, cps)
-    if (two) {
+#define QE_SKINNY_W(MT_, NT_, WAVES_, NORM_)                                                           \
+    do {                                                                                               \
+        auto kern = gemm_skinny_kernel<MT_, NT_, EPI, TO, WAVES_, NORM_>;                              \
+        const size_t dyn = NORM_ ? norm_lds_bytes(M, K) : 0;                                           \
+        if (dyn > 32 * 1024) {                                                                         \
+            static bool raised = false;   /* (once per kernel: the limit of dynamic shared memory) */ \
+            if (!raised) {                                                                             \
+                hipError_t e_ = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                                    QE_SKINNY_MAX_NORM_LDS);                           \
+                if (e_ != hipSuccess) { qe_set_error("skinny gemm: %s", hipGetErrorString(e_)); return (int)e_; } \
+                raised = true;                                                                         \
+            }                                                                                          \
+        }                                                                                              \
+        kern<<<grid, WAVES_ * 64, dyn, stream>>>(x, (const bf16_t*)w, bias, (TO*)out, M, N, K, cps, norm_w, norm_eps, \
+                                                 delta, n_delta, h_out);                               \
+    } while (0)
+#define QE_SKINNY(MT_, NT_) QE_SKINNY_W(MT_, NT_, 4, false)
+    if (norm_w) {
+        QE_REQUIRE(qe_gemm_skinny_norm_ok(M, N, K) && splits == 1, "skinny gemm: the norm prologue takes up to 16 rows, K <= 8192");
+        if constexpr (SILU) QE_SKINNY_W(1, 1, 8, true);
+        else if constexpr (EPI == EPI_STORE) QE_SKINNY_W(1, 1, 4, true);
+        else QE_REQUIRE(false, "skinny gemm: the norm prologue goes with the store and silu-mul epilogues");
+    } else if (mt == 1 && SILU) {
+        if constexpr (SILU) QE_SKINNY_W(1, 1, 8, false);
+    } else if (two) {
         switch (mt) {
             case 2: QE_SKINNY(2, 2); break;
             case 3: if constexpr (!SILU) QE_SKINNY(3, 2); break;
@@ -166,6 +373,7 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
         }
     }
 #undef QE_SKINNY
+#undef QE_SKINNY_W
     QE_LAUNCH_CHECK();
     return 0;
 }
@@ -189,30 +397,38 @@ int qe_gemm_skinny_splits(int N, int K) {
 // EPI_SILU_MUL: w is [2 N, K] (gate rows, then up rows), out [M, N] in dt_o.
 // EPI_SILU_MUL_IL: the same with gate and up rows interleaved in blocks of 32.
 // EPI_PARTIAL: out is float [splits, M, N]; the product is the sum over the first index.
+// norm_w (or null): the weight of an RMSNorm that stands before the product; x is then the 32-bit
+// stream [M, K] and the rows are normed (eps norm_eps) before they are multiplied.  delta (or null):
+// n_delta partial products [n_delta][M][K] of the branch before, added to the stream's rows in
+// order before the norm; the summed rows are written to h_out [M][K], which is not x (the blocks
+// read x while one of them writes).
 int qe_gemm_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                   int dt_o, int epilogue, int splits, hipStream_t stream) {
+                   int dt_o, int epilogue, int splits, const float* norm_w, float norm_eps,
+                   const float* delta, int n_delta, float* h_out, hipStream_t stream) {
+    QE_REQUIRE(norm_w || (!delta && !h_out), "skinny gemm: partial products to add go with the norm prologue");
+    QE_REQUIRE(!delta || (n_delta >= 1 && h_out && h_out != x), "skinny gemm: %d partial products, and the summed stream needs a place of its own", n_delta);
     QE_REQUIRE(M >= 1 && M <= 64 && K % 32 == 0, "skinny gemm: M=%d K=%d not taken", M, K);
     QE_REQUIRE(splits >= 1 && splits <= 64 && (epilogue == EPI_PARTIAL || splits == 1),
                "skinny gemm: %d splits with epilogue %d", splits, epilogue);
     if (epilogue == EPI_PARTIAL) {
         QE_REQUIRE(dt_o == QE_F32, "skinny gemm: partial products are 32-bit");
-        return launch_skinny<EPI_PARTIAL, float>(x, w, bias, out, M, N, K, splits, stream);
+        return launch_skinny<EPI_PARTIAL, float>(x, w, bias, out, M, N, K, splits, norm_w, norm_eps, delta, n_delta, h_out, stream);
     }
     if (epilogue == EPI_RESIDUAL) {
         QE_REQUIRE(dt_o == QE_F32, "skinny gemm: the residual stream is 32-bit");
-        return launch_skinny<EPI_RESIDUAL, float>(x, w, bias, out, M, N, K, 1, stream);
+        return launch_skinny<EPI_RESIDUAL, float>(x, w, bias, out, M, N, K, 1, norm_w, norm_eps, delta, n_delta, h_out, stream);
     }
     if (epilogue == EPI_SILU_MUL) {
         QE_REQUIRE(!bias, "skinny gemm: silu-mul takes no bias");
-        if (dt_o == QE_BF16) return launch_skinny<EPI_SILU_MUL, bf16_t>(x, w, bias, out, M, N, K, 1, stream);
-        return launch_skinny<EPI_SILU_MUL, float>(x, w, bias, out, M, N, K, 1, stream);
+        if (dt_o == QE_BF16) return launch_skinny<EPI_SILU_MUL, bf16_t>(x, w, bias, out, M, N, K, 1, norm_w, norm_eps, delta, n_delta, h_out, stream);
+        return launch_skinny<EPI_SILU_MUL, float>(x, w, bias, out, M, N, K, 1, norm_w, norm_eps, delta, n_delta, h_out, stream);
     }
     if (epilogue == EPI_SILU_MUL_IL) {
         QE_REQUIRE(!bias && N % 32 == 0, "skinny gemm: interleaved silu-mul takes no bias and N in blocks of 32");
-        if (dt_o == QE_BF16) return launch_skinny<EPI_SILU_MUL_IL, bf16_t>(x, w, bias, out, M, N, K, 1, stream);
-        return launch_skinny<EPI_SILU_MUL_IL, float>(x, w, bias, out, M, N, K, 1, stream);
+        if (dt_o == QE_BF16) return launch_skinny<EPI_SILU_MUL_IL, bf16_t>(x, w, bias, out, M, N, K, 1, norm_w, norm_eps, delta, n_delta, h_out, stream);
+        return launch_skinny<EPI_SILU_MUL_IL, float>(x, w, bias, out, M, N, K, 1, norm_w, norm_eps, delta, n_delta, h_out, stream);
     }
     QE_REQUIRE(epilogue == EPI_STORE, "skinny gemm: unknown epilogue %d", epilogue);
-    if (dt_o == QE_BF16) return launch_skinny<EPI_STORE, bf16_t>(x, w, bias, out, M, N, K, 1, stream);
-    return launch_skinny<EPI_STORE, float>(x, w, bias, out, M, N, K, 1, stream);
+    if (dt_o == QE_BF16) return launch_skinny<EPI_STORE, bf16_t>(x, w, bias, out, M, N, K, 1, norm_w, norm_eps, delta, n_delta, h_out, stream);
+    return launch_skinny<EPI_STORE, float>(x, w, bias, out, M, N, K, 1, norm_w, norm_eps, delta, n_delta, h_out, stream);
 }

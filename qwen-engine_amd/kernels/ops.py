@@ -48,7 +48,8 @@ def load_library():
         "qe_scatter_int": [vp, vp, vp, i32, i64, vp],
         "qe_silu_mul": [vp, vp, i32, i32, i32, i32, vp],
         "qe_gemm_silu_supported": [i32, i32, i32, i32, i32],
-        "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
+        "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp, f32, vp, i32, vp, vp],
+        "qe_gemm_norm_supported": [i32, i32, i32, i32],
         "qe_gemm_partial_splits": [i32, i32, i32],
         "qe_gemm_qkv_supported": [i32, i32, i32, i32, i32, i32, i32, i32],
         "qe_gemm_qkv_run": [vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, vp, f32, vp, vp, vp, i32, vp],
@@ -249,9 +250,18 @@ def gemm_silu_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
     return bool(lib.qe_gemm_silu_supported(x.shape[0], w.shape[0] // 2, x.shape[1], _DT[x.dtype], _DT[w.dtype]))
 
 
+def gemm_norm_supported(M: int, w: torch.Tensor) -> bool:
+    """True if gemm can take the RMSNorm that stands before the product as its prologue (``norm_weight``)
+    for M rows of the stream against w: up to 16 rows, bfloat16 weights."""
+    lib = load_library()
+    return w.dtype in _DT and bool(lib.qe_gemm_norm_supported(int(M), w.shape[0], w.shape[1], _DT[w.dtype]))
+
+
 def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
          out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
-         algo: int = ALGO_AUTO, epilogue: int = EPI_STORE, splits: int = 0) -> torch.Tensor:
+         algo: int = ALGO_AUTO, epilogue: int = EPI_STORE, splits: int = 0,
+         norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 0.0,
+         delta: Optional[torch.Tensor] = None, stream_out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x [M, K] . w [N, K]^T (+ bias [N], 32-bit) -> [M, N] in out_dtype (default: x's).
 
     epilogue EPI_RESIDUAL: the product is added into ``out``, the 32-bit stream [M, N].
@@ -260,7 +270,14 @@ def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
     interleaved in blocks of 32 (see interleave_gate_up); needs gemm_silu_supported(x, w).
     epilogue EPI_PARTIAL: the product is cut along K into ``splits`` (0: chosen for the shape)
     partial products, returned as float32 [splits, M, N]; their sum over the first index, taken
-    in order, is the product.  All three need gemm_fused_supported(x, w)."""
+    in order, is the product.  All three need gemm_fused_supported(x, w).
+
+    norm_weight (float32 [K]) with norm_eps: x is the 32-bit stream and the RMSNorm of its rows, rounded
+    to bfloat16 as the norm kernel rounds it, is what is multiplied (out_dtype defaults to bfloat16);
+    needs gemm_norm_supported(M, w); with the store and silu-mul epilogues.  With it, ``delta`` (float32
+    [S, M, K], the partial products of the branch before) is added to the stream's rows, in the order
+    of S, before the norm, and the sums are written to ``stream_out`` [M, K], another tensor than x (every
+    block reads x while one of them writes): the residual sum and the norm without kernels of their own."""
     lib = load_library()
     _need(x, "x", _ACT, (None, None))
     M, K = x.shape
@@ -270,7 +287,24 @@ def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
         if N % 2:
             raise KernelError("gemm: gate|up weights have an odd number of rows")
         N //= 2
-    if x.dtype == torch.float32 and w.dtype != torch.float32:
+    if norm_weight is not None:
+        _need(x, "x (the stream)", torch.float32, (M, K))
+        _need(norm_weight, "norm_weight", torch.float32, (K,), x.device)
+        if not gemm_norm_supported(M, w):
+            raise KernelError(f"gemm: {M} rows against {tuple(w.shape)} are not taken with the norm as prologue")
+        out_dtype = out_dtype or torch.bfloat16
+        if delta is not None:
+            _need(delta, "delta", torch.float32, (None, M, K), x.device)
+            if stream_out is None:
+                raise KernelError("gemm: partial products to add need a place for the summed stream")
+            _need(stream_out, "stream_out", torch.float32, (M, K), x.device)
+            if stream_out.data_ptr() == x.data_ptr():
+                raise KernelError("gemm: the summed stream cannot be written over the stream that is read")
+        elif stream_out is not None:
+            raise KernelError("gemm: stream_out goes with delta")
+    elif delta is not None or stream_out is not None:
+        raise KernelError("gemm: delta and stream_out go with norm_weight")
+    elif x.dtype == torch.float32 and w.dtype != torch.float32:
         raise KernelError("gemm: 32-bit activations need 32-bit weights")
     if bias is not None:
         _need(bias, "bias", torch.float32, (N,), x.device)
@@ -289,7 +323,9 @@ def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
         out = torch.empty(shape, dtype=out_dtype, device=x.device)
     _need(out, "out", out_dtype, shape, x.device)
     _check(lib.qe_gemm(x.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), M, N, K,
-                       _DT[x.dtype], _DT[w.dtype], _DT[out_dtype], algo, epilogue, splits, _stream()), "gemm")
+                       _DT[x.dtype], _DT[w.dtype], _DT[out_dtype], algo, epilogue, splits,
+                       _ptr(norm_weight), float(norm_eps), _ptr(delta), 0 if delta is None else delta.shape[0],
+                       _ptr(stream_out), _stream()), "gemm")
     return out
 
 

@@ -15,7 +15,8 @@ import torch
 
 from ..cache.plan import KVNeed
 from ..kernels import ops
-from .base import CacheBinding, Runtime, TensorInfo
+from .base import CacheBinding, Runtime, StreamInput, TensorInfo
+from .block_sizes import FEW_ROWS, FEW_ROWS_PARTS
 from .registry import build_part, register_part
 
 
@@ -40,6 +41,8 @@ def prefill_tiles(portions, rows_per_tile: int) -> List[int]:
 
 
 class PagedAttention:
+    takes_stream = True       # forward may get a StreamInput: residual sum and norm are then the q|k|v product's prologue
+
     # ---- what the step function prepares for this part (parts.base) --------------------------
     @staticmethod
     def step_extras(seqs) -> dict:
@@ -141,10 +144,17 @@ class PagedAttention:
             self.position.load({}, rt)
 
     # ---- one step -------------------------------------------------------------------
-    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding) -> torch.Tensor:
-        """Returns the mixer's output [T, H], or float32 partial products [S, T, H] of it."""
+    def forward(self, x, ctx, binding: CacheBinding) -> torch.Tensor:
+        """Returns the mixer's output [T, H], or float32 partial products [S, T, H] of it.
+        x: the normed rows, or a StreamInput."""
         if binding.kv is None:
             raise RuntimeError("attention was given no cache")
+        lazy = None
+        if isinstance(x, StreamInput):
+            if ctx.rt.dtype == torch.bfloat16 and ops.gemm_norm_supported(x.rows, self.w_qkv):
+                lazy, x = x, x.stream.h
+            else:
+                x = x.materialize()
         T = x.shape[0]
         g = binding.group
         eps = self.qk_eps if self.qk_eps is not None else 0.0
@@ -156,13 +166,13 @@ class PagedAttention:
         if table is not None and ctx.max_position >= table.shape[0]:
             raise RuntimeError(f"position {ctx.max_position} is beyond the rotation table "
                                f"({table.shape[0]} positions)")
-        if fused_position and ops.gemm_qkv_supported(x, self.w_qkv, cache, self.hq, table):
+        if lazy is None and fused_position and ops.gemm_qkv_supported(x, self.w_qkv, cache, self.hq, table):
             # many rows (portions of prompts): norm, rotation and cache write are the epilogue of the
             # q|k|v product, which never stores its result
             q = ops.gemm_qkv(x, self.w_qkv, self.b_qkv, self.hq, cache, ctx.positions if table is not None else None,
                              self.q_norm, self.k_norm, eps, table, slots)
             return self._attend(q, ctx, cache, g, T)
-        if (fused_position and cache.dtype == torch.bfloat16 and ops.gemm_partial_preferred(x, self.w_qkv) and
+        if (lazy is None and fused_position and cache.dtype == torch.bfloat16 and ops.gemm_partial_preferred(x, self.w_qkv) and
                 ops.qk_rope_store_parts_supported(self.d, table)):
             # 17 to 64 rows against a large matrix: the product is cut along K to fill the chip, and
             # the kernel that norms, rotates and writes the cache adds the parts up as it reads them
@@ -171,7 +181,10 @@ class PagedAttention:
                                         ctx.positions if table is not None else None, self.q_norm, self.k_norm,
                                         eps, table, slots, cache, ctx.page_size)
             return self._attend(q, ctx, cache, g, T)
-        qkv = ops.gemm(x, self.w_qkv, self.b_qkv)
+        if lazy is not None:    # few rows: the norm before the part is the product's prologue
+            qkv = lazy.gemm(ops, self.w_qkv, self.b_qkv)
+        else:
+            qkv = ops.gemm(x, self.w_qkv, self.b_qkv)
         if fused_position:
             ex = self._extras(ctx)
             only_new_tokens = (ex["dec_tokens"] is not None and ex["dec_tokens"].shape[0] == T and
@@ -206,6 +219,8 @@ class PagedAttention:
 
     def _project_out(self, o: torch.Tensor) -> torch.Tensor:
         splits = ops.gemm_branch_splits(o, self.w_o)
+        if o.shape[0] <= FEW_ROWS and splits > FEW_ROWS_PARTS and ops.gemm_fused_supported(o, self.w_o):
+            splits = FEW_ROWS_PARTS
         if splits:
             # the product is cut along K (few rows: to fill the chip; a narrow matrix: to give every
             # compute unit blocks to overlap); the norm that follows adds the parts

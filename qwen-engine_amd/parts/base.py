@@ -16,6 +16,16 @@ Stream prologue   forward(h, ctx) -> None: changes the 32-bit stream in place ri
               embedding (a scale, an added table of positions).
 Logit epilogue    forward(logits, ctx) -> logits on the float32 logits [R, V] (a scale, a soft cap).
 
+Few rows (decode): a step is then a chain of short dependent kernels, each of which costs a few
+microseconds whatever it does, so a norm and a residual sum of their own cost as much as the
+products around them.  A mixer or feed-forward class may therefore say
+  takes_stream = True      forward may get, instead of x, a StreamInput: the 32-bit stream, what the
+                           branch before left to add to it, and the norm that stands before the
+                           part; the part lets its first product do the sum and the norm
+                           (StreamInput.gemm) or calls materialize()
+and a norm class says with ``fusable_weight()`` (its weight and eps, or None) that it is a plain
+RMSNorm that a product can take as its prologue.
+
 What a part needs prepared per step beyond the flat batch, it asks for itself; the step function
 knows none of it.  A part class may define (all optional, all static):
   step_extras(seqs) -> dict      from the step's SeqInfo list, on the host: int32 numpy arrays (sent
@@ -67,6 +77,54 @@ class Runtime:
     def place_vector(self, t: torch.Tensor) -> torch.Tensor:
         """Norm weights and biases enter 32-bit arithmetic only: held in float32 (exact)."""
         return t.to(torch.float32).contiguous().to(self.device)
+
+
+class Stream:
+    """The 32-bit residual stream of a step, [T, H], with a second buffer of the same size: a
+    product that adds a branch's partial products to the stream in its prologue writes the sums
+    into the other buffer (its blocks read the stream while one of them writes), and the two
+    change places."""
+
+    def __init__(self, h: torch.Tensor, spare: Optional[torch.Tensor] = None):
+        self.h, self.spare = h, spare
+
+    def swap(self) -> None:
+        self.h, self.spare = self.spare, self.h
+
+
+@dataclass
+class StreamInput:
+    """The input of a part as (stream, what is still to be added to it, norm before the part)
+    instead of the normed rows."""
+    stream: Stream
+    delta: Optional[torch.Tensor]   # None, or the branch output that the norm before the part adds to the stream
+    norm: object                    # the norm part that stands before the consumer
+    weight: torch.Tensor            # its weight, float32 [H]
+    eps: float
+    rt: "Runtime"
+
+    @property
+    def rows(self) -> int:
+        return self.stream.h.shape[0]
+
+    def fusable(self) -> bool:
+        """True if a product can take the residual sum and the norm as its prologue: nothing to
+        add, or float32 partial products and a second buffer for the sums."""
+        d = self.delta
+        return d is None or (d.dim() == 3 and d.dtype == torch.float32 and self.stream.spare is not None)
+
+    def gemm(self, ops, w: torch.Tensor, bias=None, **kw) -> torch.Tensor:
+        """The product of the normed rows with w, the residual sum and the norm inside it."""
+        if self.delta is None:
+            return ops.gemm(self.stream.h, w, bias, norm_weight=self.weight, norm_eps=self.eps, **kw)
+        y = ops.gemm(self.stream.h, w, bias, norm_weight=self.weight, norm_eps=self.eps, delta=self.delta,
+                     stream_out=self.stream.spare, **kw)
+        self.stream.swap()
+        return y
+
+    def materialize(self) -> torch.Tensor:
+        """The normed rows as a tensor of their own (the norm's kernel, which adds delta into the stream)."""
+        return self.norm.forward(self.stream.h, self.rt, delta=self.delta)
 
 
 @dataclass

@@ -8,7 +8,8 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import CacheBinding, Runtime, TensorInfo, sub_tensors
+from .base import CacheBinding, Runtime, Stream, StreamInput, TensorInfo, sub_tensors
+from .block_sizes import FEW_ROWS as FUSED_NORM_MAX_ROWS
 from .registry import build_part, part_class, register_part
 
 def _names(spec):
@@ -45,15 +46,28 @@ class PreNormBlock:
         for name, part in zip(_names(self.spec), (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)):
             part.load(sub_tensors(tensors, name + "."), rt)
 
-    def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], ctx, binding: CacheBinding) -> torch.Tensor:
-        """h: 32-bit residual stream (updated in place).  pending: branch output not yet
-        added to h, or None.  Returns the feed-forward output, to be added by whoever norms next.
-        A branch output is [T, H] in the activation type, or float32 [S, T, H]: partial products
-        that the norm adds in the order of S."""
-        x = self.mixer_norm.forward(h, ctx.rt, delta=pending)
+    def forward(self, h, pending: Optional[torch.Tensor], ctx, binding: CacheBinding) -> torch.Tensor:
+        """h: the 32-bit residual stream, a tensor (updated in place) or a Stream (whose buffers may
+        change places).  pending: branch output not yet added to the stream, or None.  Returns the
+        feed-forward output, to be added by whoever norms next.  A branch output is [T, H] in the
+        activation type, or float32 [S, T, H]: partial products that the norm adds in the order of S."""
+        stream = h if isinstance(h, Stream) else Stream(h)
+        x = self._input(self.mixer_norm, self.mixer, stream, pending, ctx)
         a = self.mixer.forward(x, ctx, binding)
-        x = self.ffn_norm.forward(h, ctx.rt, delta=a)
+        x = self._input(self.ffn_norm, self.ffn, stream, a, ctx)
         return self.ffn.forward(x, ctx)
+
+    @staticmethod
+    def _input(norm, part, stream: Stream, delta, ctx):
+        """The part's input: the normed rows, or, with few rows and where both the norm and the part
+        can do it, the stream, what is to be added, and the norm, for the part's first product."""
+        if (getattr(part, "takes_stream", False) and hasattr(norm, "fusable_weight") and
+                stream.h.shape[0] <= FUSED_NORM_MAX_ROWS):
+            fw = norm.fusable_weight()
+            si = StreamInput(stream, delta, norm, fw[0], fw[1], ctx.rt) if fw is not None else None
+            if si is not None and si.fusable():
+                return si
+        return norm.forward(stream.h, ctx.rt, delta=delta)
 
 
 register_part("prenorm_block", PreNormBlock)

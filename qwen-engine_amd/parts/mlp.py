@@ -9,11 +9,14 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .base import Runtime, TensorInfo
+from .base import Runtime, StreamInput, TensorInfo
+from .block_sizes import FEW_ROWS, FEW_ROWS_PARTS
 from .registry import register_part
 
 
 class SwiGLU:
+    takes_stream = True       # forward may get a StreamInput: residual sum and norm are then the gate|up product's prologue
+
     def __init__(self, spec, hidden_size: int):
         self.hidden = int(hidden_size)
         self.inter = int(spec.intermediate_size)
@@ -39,15 +42,26 @@ class SwiGLU:
         self.w_gu = rt.place_matrix(ops.interleave_gate_up(g, u) if self.interleaved else torch.cat([g, u], dim=0))
         self.w_down = rt.place_matrix(tensors["down_proj.weight"])
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        """Returns the feed-forward output [T, H], or float32 partial products [S, T, H] of it."""
-        if self.interleaved and ops.gemm_silu_supported(x, self.w_gu):
+    def forward(self, x, ctx) -> torch.Tensor:
+        """Returns the feed-forward output [T, H], or float32 partial products [S, T, H] of it.
+        x: the normed rows, or a StreamInput."""
+        a = None
+        if isinstance(x, StreamInput):
+            if ctx.rt.dtype == torch.bfloat16 and ops.gemm_norm_supported(x.rows, self.w_gu):
+                a = x.gemm(ops, self.w_gu, epilogue=ops.EPI_SILU_MUL_IL if self.interleaved else ops.EPI_SILU_MUL)
+            else:
+                x = x.materialize()
+        if a is not None:
+            pass
+        elif self.interleaved and ops.gemm_silu_supported(x, self.w_gu):
             a = ops.gemm(x, self.w_gu, epilogue=ops.EPI_SILU_MUL_IL)   # silu.mul in the product's epilogue
         elif not self.interleaved and ops.gemm_fused_supported(x, self.w_gu):
             a = ops.gemm(x, self.w_gu, epilogue=ops.EPI_SILU_MUL)
         else:
             a = ops.silu_mul(ops.gemm(x, self.w_gu), interleaved=self.interleaved)
         splits = ops.gemm_branch_splits(a, self.w_down)
+        if a.shape[0] <= FEW_ROWS and splits > FEW_ROWS_PARTS and ops.gemm_fused_supported(a, self.w_down):
+            splits = FEW_ROWS_PARTS
         if splits:   # partial products along K, added by the norm that follows
             return ops.gemm(a, self.w_down, epilogue=ops.EPI_PARTIAL, splits=splits)
         return ops.gemm(a, self.w_down)

@@ -10,7 +10,8 @@ import torch
 from ..cache.plan import CachePlan, plan_cache
 from ..config.spec import ModelSpec
 from ..kernels import ops
-from .base import CacheBinding, Runtime, TensorInfo, sub_tensors
+from .base import CacheBinding, Runtime, Stream, TensorInfo, sub_tensors
+from .block import FUSED_NORM_MAX_ROWS
 from .registry import build_part, part_class
 
 
@@ -127,9 +128,12 @@ class DecoderModel:
             h = ops.embedding(ctx.token_ids, self.embed)
             if self.prologue is not None:
                 self.prologue.forward(h, ctx)
+            # (few rows: a second buffer, so that a product can do the residual sum before it, see Stream)
+            stream = Stream(h, torch.empty_like(h) if h.shape[0] <= FUSED_NORM_MAX_ROWS else None)
             pending = None
             for i, entry in enumerate(self.spec.schedule):
-                pending = self.blocks[entry.layer].forward(h, pending, ctx, bindings[i])
+                pending = self.blocks[entry.layer].forward(stream, pending, ctx, bindings[i])
+            h = stream.h
             R = ctx.logit_rows.shape[0]
             if R == 0:
                 return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=h.device)

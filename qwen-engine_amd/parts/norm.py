@@ -24,6 +24,10 @@ class RMSNorm:
     def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
         self.weight = rt.place_vector(tensors["weight"])
 
+    def fusable_weight(self):
+        """(weight, eps): this is a plain RMSNorm, which a product can take as its prologue."""
+        return self.weight, self.eps
+
     def forward(self, h: torch.Tensor, rt: Runtime, delta: Optional[torch.Tensor] = None,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         return ops.rmsnorm(h, self.weight, self.eps, rt.dtype, delta=delta, rows=rows)

@@ -861,3 +861,66 @@ def test_gemm_for_few_rows_against_the_whole_vocabulary(ops, M):
     # the same through the generic 32-bit kernel, on 32-bit copies of the operands
     got32 = ops.gemm(x.float().to(DEV), w.float().to(DEV), out_dtype=torch.float32, algo=ops.ALGO_GENERIC).cpu()
     close(got32[:, cols], want, torch.float32, scale=float(want.abs().max()))
+
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("N,K", [(4096, 1024), (512, 96), (336, 160), (2048, 4096), (64, 8192)])
+def test_gemm_with_the_norm_as_its_prologue(ops, M, N, K):
+    """The product of few rows that norms the 32-bit stream itself gives, to the bit, what the norm
+    kernel followed by the product gives: the same arithmetic in the same order.  Also with a bias,
+    with silu.mul over gate|up rows (both layouts), and against the plain norm and product."""
+    bf = torch.bfloat16
+    h = rand(M, K, seed=530, scale=3.0).to(DEV)
+    nw = (1 + rand(K, seed=531, scale=0.2)).to(DEV)
+    w = rand(N, K, seed=532, dtype=bf, scale=0.1).to(DEV)
+    bias = rand(N, seed=533).to(DEV)
+    eps = 1e-5
+    # (the normed rows lie in shared memory as bfloat16, with 8 elements of padding a row: up to 136 KB)
+    assert ops.gemm_norm_supported(M, w) == (M * (K + 8) * 2 <= 136 * 1024)
+    if not ops.gemm_norm_supported(M, w):
+        with pytest.raises(ops.KernelError):
+            ops.gemm(h, w, norm_weight=nw, norm_eps=eps)
+        return
+    x = ops.rmsnorm(h, nw, eps, bf)
+    for b in (None, bias):
+        for dt_o in (bf, torch.float32):
+            fused = ops.gemm(h, w, b, out_dtype=dt_o, norm_weight=nw, norm_eps=eps)
+            assert fused.dtype == dt_o and torch.equal(fused, ops.gemm(x, w, b, out_dtype=dt_o))
+    close(x, P.rms_norm(h.cpu().double(), nw.cpu().double(), eps), bf)            # the norm kernel itself
+    want = P.linear(x.cpu().double(), w.cpu().double())
+    close(ops.gemm(h, w, out_dtype=torch.float32, norm_weight=nw, norm_eps=eps), want, torch.float32,
+          scale=float(want.abs().max()))
+    # with the residual sum inside as well: the partial products of the branch before are added to the
+    # stream in order, normed and multiplied, and the sums are written to a second buffer
+    for S in (1, 4):
+        parts = rand(S, M, K, seed=534, scale=1.5).to(DEV)
+        h2 = h.clone()
+        x2 = ops.rmsnorm(h2, nw, eps, bf, delta=parts)                 # (adds the parts into h2)
+        summed = torch.full_like(h, float("nan"))
+        fused = ops.gemm(h, w, bias, norm_weight=nw, norm_eps=eps, delta=parts, stream_out=summed)
+        assert torch.equal(summed, h2) and torch.equal(fused, ops.gemm(x2, w, bias))
+    with pytest.raises(ops.KernelError):
+        ops.gemm(h, w, norm_weight=nw, norm_eps=eps, delta=parts, stream_out=h)     # over the stream that is read
+    if N % 64 == 0:
+        fused = ops.gemm(h, w, epilogue=ops.EPI_SILU_MUL_IL, norm_weight=nw, norm_eps=eps)
+        assert fused.shape == (M, N // 2) and torch.equal(fused, ops.gemm(x, w, epilogue=ops.EPI_SILU_MUL_IL))
+    fused = ops.gemm(h, w, epilogue=ops.EPI_SILU_MUL, norm_weight=nw, norm_eps=eps)
+    assert torch.equal(fused, ops.gemm(x, w, epilogue=ops.EPI_SILU_MUL))
+    g, u = want[:, :N // 2], want[:, N // 2:]
+    close(fused, P.silu_mul(g, u), bf)
+
+
+def test_gemm_norm_prologue_refuses_what_it_does_not_take(ops):
+    bf = torch.bfloat16
+    w = rand(64, 64, seed=540, dtype=bf).to(DEV)
+    nw = torch.ones(64, device=DEV)
+    assert not ops.gemm_norm_supported(17, w)                            # more than 16 rows
+    assert not ops.gemm_norm_supported(4, w.float())                     # 32-bit weights
+    assert not ops.gemm_norm_supported(16, torch.zeros(32, 8192, dtype=bf, device=DEV))     # rows too long for shared memory
+    assert not ops.gemm_norm_supported(2, torch.zeros(32, 16384, dtype=bf, device=DEV))     # beyond the norm kernel's own layout
+    with pytest.raises(ops.KernelError):
+        ops.gemm(torch.zeros(17, 64, device=DEV), w, norm_weight=nw, norm_eps=1e-6)
+    with pytest.raises(ops.KernelError):                                 # the stream is 32-bit
+        ops.gemm(torch.zeros(4, 64, device=DEV, dtype=bf), w, norm_weight=nw, norm_eps=1e-6)
+    with pytest.raises(ops.KernelError):                                 # partial products do not go with it
+        ops.gemm(torch.zeros(4, 64, device=DEV), w, epilogue=ops.EPI_PARTIAL, norm_weight=nw, norm_eps=1e-6)
