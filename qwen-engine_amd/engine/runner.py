@@ -68,6 +68,11 @@ class ModelRunner:
     and replayed, so that their launch cost does not grow with the number of kernels.
     """
 
+    # A step that is one prompt portion of a round length (a whole number of PORTION_GRAPH_STEP tokens,
+    # at least PORTION_GRAPH_MIN) is recorded once per length too: a portion is a few hundred kernels
+    # of some microseconds each, which the host cannot launch as fast as the device runs them.
+    PORTION_GRAPH_MIN = 256
+    PORTION_GRAPH_STEP = 128
     MAX_GRAPHS = 32       # recorded graphs kept (each holds its own activations); the least recently used goes first
 
     def __init__(self, model: DecoderModel, page_size: int, num_pages, max_requests: int,
@@ -122,13 +127,13 @@ class ModelRunner:
         # bounded by its pool)
         self.table_width = [max(1, per_request if grp.window is not None else min(pool.num_pages, per_request))
                             for grp, pool in zip(self.cache.groups, self.cache.pools)]
-        # one row more than there are state slots: the spare row's first entry always names page 0
-        # of its pool.  It is the table row of the rows that fill a recorded decode graph up and of
+        # one row more than there are state slots: the spare row's entries always name page 0
+        # of their pool.  It is the table row of the rows that fill a recorded decode graph up and of
         # the stand-in batch while recording: they stand at position 0 and write nowhere, and what
         # they read there lies inside the storage whatever the live requests hold.
         self.tables = [torch.full((max_requests + 1, w), -1, dtype=torch.int32, device=dev) for w in self.table_width]
         for t in self.tables:
-            t[max_requests, 0] = 0
+            t[max_requests].zero_()            # (every entry: the stand-in of a recorded prompt portion reads them all)
         self.spare_row = max_requests
         # a part with per-request state is recorded into graphs only if it says that it can be
         # (``graph_safe = True`` on the class); any other part unless it says that it cannot
@@ -144,6 +149,9 @@ class ModelRunner:
             if hasattr(cls, "step_extras") and cls not in self._step_classes:
                 self._step_classes.append(cls)
         self._graphs = {}
+        # portions are recorded only if every part that wants something prepared can say what a
+        # recorded portion needs (parts.base: portion_graph_extras)
+        self._portion_graphs = all(hasattr(cls, "portion_graph_extras") for cls in self._step_classes)
         self._stage: Optional[torch.Tensor] = None     # pinned host buffer of a step's integer arrays
         self._stage_np = None
         self._stage_event = torch.cuda.Event()
@@ -403,6 +411,9 @@ class ModelRunner:
         device, in the order of the entries and of their ``want``."""
         if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries) and entries:
             logits = self._decode_step_with_graph(entries)
+        elif self.use_graphs and self._portion_graphs and len(entries) == 1 and len(entries[0].want) <= 1 and \
+                len(entries[0].tokens) >= self.PORTION_GRAPH_MIN and len(entries[0].tokens) % self.PORTION_GRAPH_STEP == 0:
+            logits = self._portion_step_with_graph(entries[0])
         else:
             ctx = self.build_context(entries)
             self._clear_state_of_new_requests(ctx.seqs)
@@ -465,6 +476,94 @@ class ModelRunner:
         rec["graph"].replay()
         self.graph_steps += 1
         return rec["logits"][:n_live].clone()          # the graph's own output is overwritten by the next replay
+
+    # ---- one prompt portion through a recorded graph ----------------------------------------
+    def _portion_step_with_graph(self, entry: StepEntry) -> torch.Tensor:
+        tokens = self._check_and_reserve([entry])
+        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout([entry], tokens)
+        self._check_bounds(seqs, slots, upd_idx, upd_val)
+        self._poison_pages()
+        self._clear_state_of_new_requests(seqs)
+        T, n_want, n_groups = len(token_ids), len(rows), len(self.cache.groups)
+        cap = 2 * (T // self.page_size + 2)
+        i32 = np.int32
+        if any(len(u) > cap for u in upd_idx):
+            for g in range(n_groups):
+                if len(upd_idx[g]):
+                    ops.scatter_int(self.tables[g], torch.from_numpy(upd_idx[g]).to(self.rt.device),
+                                    torch.from_numpy(upd_val[g]).to(self.rt.device))
+                upd_idx[g] = upd_val[g] = np.zeros(0, dtype=i32)
+        key = ("portion", T, n_want)
+        rec = self._graphs.pop(key, None)
+        if rec is None:
+            while len(self._graphs) >= self.MAX_GRAPHS:
+                self._graphs.pop(next(iter(self._graphs)))
+            rec = self._record_portion_graph(T, n_want, cap)
+            self.graphs_recorded += 1
+        self._graphs[key] = rec
+        none, zero = rec["none"], rec["zero"]
+        parts = [token_ids, positions, tok_seq, rows, np.asarray([seqs[0].state_slot], dtype=i32)]
+        for g in range(n_groups):
+            pad = cap - len(upd_idx[g])
+            parts += [slots[g], upd_idx[g], none[:pad], upd_val[g], zero[:pad]]
+        rec["event"].synchronize()
+        np.concatenate(parts, out=rec["host_np"])
+        rec["meta"].copy_(rec["host"], non_blocking=True)
+        rec["event"].record()
+        rec["graph"].replay()
+        self.graph_steps += 1
+        return rec["logits"].clone()
+
+    def _record_portion_graph(self, T: int, n_want: int, cap: int):
+        """Static buffers for a step that is one prompt portion of T tokens with n_want (0 or 1) rows
+        of logits, one run outside the graph, then the recording.  The stand-in batch stands at
+        positions 0 .. T - 1 of the tables' spare row (every entry page 0) and writes nowhere."""
+        dev, n_groups = self.rt.device, len(self.cache.groups)
+        n = 3 * T + n_want + 1 + n_groups * (T + 2 * cap)
+        host = torch.zeros(n, dtype=torch.int32).pin_memory()
+        meta = torch.zeros(n, dtype=torch.int32, device=dev)
+        stand_in = [0] * T + list(range(T)) + [self.spare_row] * T + [T - 1] * n_want + [self.spare_row]
+        for g in range(n_groups):
+            stand_in += [-1] * T + [-1] * cap + [0] * cap
+        meta.copy_(torch.tensor(stand_in, dtype=torch.int32))
+        off = 0
+
+        def take(k):
+            nonlocal off
+            t = meta[off:off + k]
+            off += k
+            return t
+
+        d_tok, d_pos, d_seq, d_rows, d_state = take(T), take(T), take(T), take(n_want), take(1)
+        d_slots, d_upd = [], []
+        for g in range(n_groups):
+            d_slots.append(take(T))
+            d_upd.append((take(cap), take(cap)))
+        seqs = [SeqInfo(None, 0, T, 0, self.spare_row, False)]
+        ctx = StepContext(rt=self.rt, page_size=self.page_size, num_tokens=T, seqs=seqs, token_ids=d_tok,
+                          positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
+                          logit_rows=d_rows, state_slots=d_state, max_position=0,
+                          extras={cls: dict(cls.portion_graph_extras(T, dev)) for cls in self._step_classes})
+
+        def run():
+            for g in range(n_groups):
+                ops.scatter_int(self.tables[g], d_upd[g][0], d_upd[g][1])
+            return self.model.forward(ctx, self.bindings)
+
+        torch.cuda.synchronize()
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            run()                                 # (what the parts keep for the step, ctx.memo, is made here)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            logits = run()
+        torch.cuda.synchronize()
+        event = torch.cuda.Event()
+        event.record()
+        return {"graph": graph, "ctx": ctx, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits,
+                "event": event, "none": np.full(cap, -1, dtype=np.int32), "zero": np.zeros(cap, dtype=np.int32)}
 
     def _record_decode_graph(self, B: int, part_keys: tuple, cap: int):
         """Static buffers for a decode step of B requests whose positions give the parts'

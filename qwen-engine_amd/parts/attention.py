@@ -69,6 +69,13 @@ class PagedAttention:
         return {"dec_tokens": torch.arange(rows, dtype=torch.int32, device=device), "other_tokens": None,
                 "max_dec_position": key * ops.DECODE_SPLIT_KEYS - 1}
 
+    @staticmethod
+    def portion_graph_extras(tokens: int, device) -> dict:
+        """For a recorded step that is one prompt portion of ``tokens`` rows: no single new tokens, all
+        rows in order; its launches do not depend on the positions."""
+        return {"dec_tokens": torch.zeros(0, dtype=torch.int32, device=device),
+                "other_tokens": torch.arange(tokens, dtype=torch.int32, device=device), "max_dec_position": 0}
+
     def _extras(self, ctx) -> dict:
         return ctx.extras.get(PagedAttention) or {"dec_tokens": None, "other_tokens": None, "max_dec_position": 0}
 

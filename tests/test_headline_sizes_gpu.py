@@ -125,7 +125,9 @@ def test_the_small_model_widths_with_the_whole_vocabulary(headline, dtype):
                 assert err <= tol, f"{n_live} rows: request {i} at position {done[i]}: error {err}"
                 done[i] += 1
     if dtype == "bfloat16":
-        assert runner.graph_steps == 3 + 2 + 2          # every decode step went through a recorded graph
+        # every decode step went through a recorded graph, and so did the two portions of 512 tokens
+        # that want at most one row of logits
+        assert runner.graph_steps == 3 + 2 + 2 + 2
     runner.cache.check_invariants()
 
 

@@ -81,3 +81,36 @@ def test_twenty_requests_decode_past_the_window(toy, use_graphs):
             err = float((outs[s][i] - ref[lengths[i] + s]).abs().max()) / float(ref.abs().max())
             assert err <= 2e-2, f"request {i}, step {s}: error {err}"
     runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_prompt_portions_through_recorded_graphs(toy, use_graphs):
+    """Steps that are one prompt portion of a round length are recorded once per length and replayed:
+    two requests, one after the other and then side by side in turns, each in portions of 256 and
+    384 tokens, with windows that give pages back inside the portions; logits at the portions' ends
+    against the plain implementation, and the recorded steps against steps run as they come."""
+    model = load_model(toy, dtype="bfloat16")
+    _, w = P.read_folder(toy)
+    reqs = {"a": _tokens(640, 41), "b": _tokens(896, 42)}
+    refs = {k: plain_forward(w, t, torch.bfloat16) for k, t in reqs.items()}
+    runner = ModelRunner(model, page_size=PAGE, num_pages=100, max_requests=2, use_graphs=use_graphs, debug_poison=True)
+    cuts = {"a": [(0, 256), (256, 640)], "b": [(0, 384), (384, 640), (640, 896)]}
+    got = {}
+    for order in (["a", "b"],):
+        for rid in order:
+            runner.add_request(rid)
+        turns = [("a", 0), ("b", 0), ("b", 1), ("a", 1), ("b", 2)]
+        for rid, i in turns:
+            lo, hi = cuts[rid][i]
+            want = [hi - lo - 1] if (rid, i) != ("b", 0) else []        # one portion wants no logits
+            out = runner.step([StepEntry(rid, reqs[rid][lo:hi], want)])
+            assert out.shape[0] == len(want)
+            if want:
+                got[rid, hi - 1] = out[0].float().cpu()
+    assert (runner.graph_steps == 5) == use_graphs
+    if use_graphs:
+        assert runner.graphs_recorded == 3                  # 256 with logits, 384 with and without
+    for (rid, pos), row in got.items():
+        err = float((row - refs[rid][pos]).abs().max()) / float(refs[rid].abs().max())
+        assert err <= 2e-2, f"request {rid}, position {pos}: error {err}"
+    runner.cache.check_invariants()
