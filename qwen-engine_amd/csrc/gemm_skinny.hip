@@ -120,51 +120,59 @@ __device__ __forceinline__ void norm_rows_into_lds(const float* __restrict__ hs,
         else if (M <= 8) norm_short_rows<WAVES, 8>(hs, delta, n_delta, h_out, norm_w, norm_eps, xs, M, K, KP, ss_red, mine);
         else norm_short_rows<WAVES, 16>(hs, delta, n_delta, h_out, norm_w, norm_eps, xs, M, K, KP, ss_red, mine);
     } else {
-        // longer rows: two passes over the memory (the second finds it in the cache)
+        // longer rows (up to 8 groups of four a thread): a row at a time, everything of the row asked
+        // for at once (the row and four partial products at a time, with addresses that are always
+        // valid), kept in registers from the sum of squares to the store
         for (int m = 0; m < M; ++m) {
-            float ss = 0.f;
-            if (mine) {
-                for (int i = 0; i < nv; ++i) {
-                    const int c = ((int)threadIdx.x + i * tn) * 4;
-                    if (c < K) {
-                        float v[4], d[4];
-                        Vec4<float>::load(hs + (long)m * K + c, v);
-                        for (int s = 0; s < n_delta; ++s) {
-                            Vec4<float>::load(delta + s * dstride + (long)m * K + c, d);
+            float v[8][4];
+            int col[8];
+            bool have[8];
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] += d[e];
-                        }
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) ss += v[e] * v[e];
-                    }
-                }
+            for (int i = 0; i < 8; ++i) {
+                const int c = ((int)threadIdx.x + i * tn) * 4;
+                have[i] = mine && i < nv && c < K;
+                col[i] = have[i] ? c : 0;
+                Vec4<float>::load(hs + (long)m * K + col[i], v[i]);
             }
+            for (int s0 = 0; s0 < n_delta; s0 += 4) {
+                float d[4][8][4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        Vec4<float>::load(delta + min(s0 + j, n_delta - 1) * dstride + (long)m * K + col[i], d[j][i]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (s0 + j < n_delta) {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[i][e] += d[j][i][e];
+                    }
+            }
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (have[i]) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) ss += v[i][e] * v[i][e];
+                }
             const float t = wave_sum(ss);
             if (lane == 0) ss_red[wave][m] = t;
-        }
-        __syncthreads();
-        for (int m = 0; m < M; ++m) {
-            if (!mine) continue;
+            __syncthreads();
             float tot = 0.f;
             for (int i = 0; i < WAVES; ++i) tot += ss_red[i][m];
             const float rstd = rsqrtf(tot / (float)K + norm_eps);
-            for (int i = 0; i < nv; ++i) {
-                const int c = ((int)threadIdx.x + i * tn) * 4;
-                if (c < K) {
-                    float v[4], d[4], wv[4], o[4];
-                    Vec4<float>::load(hs + (long)m * K + c, v);
-                    for (int s = 0; s < n_delta; ++s) {
-                        Vec4<float>::load(delta + s * dstride + (long)m * K + c, d);
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] += d[e];
-                    }
-                    Vec4<float>::load(norm_w + c, wv);
+            for (int i = 0; i < 8; ++i)
+                if (have[i]) {
+                    float wv[4], o[4];
+                    Vec4<float>::load(norm_w + col[i], wv);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = v[e] * rstd * wv[e];
-                    Vec4<bf16_t>::store(xs + (long)m * KP + c, o);
-                    if (h_out) Vec4<float>::store(h_out + (long)m * K + c, v);
+                    for (int e = 0; e < 4; ++e) o[e] = v[i][e] * rstd * wv[e];
+                    Vec4<bf16_t>::store(xs + (long)m * KP + col[i], o);
+                    if (h_out) Vec4<float>::store(h_out + (long)m * K + col[i], v[i]);
                 }
-            }
         }
     }
     __syncthreads();

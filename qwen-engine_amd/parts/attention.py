@@ -16,7 +16,7 @@ import torch
 from ..cache.plan import KVNeed
 from ..kernels import ops
 from .base import CacheBinding, Runtime, StreamInput, TensorInfo
-from .block_sizes import FEW_ROWS, FEW_ROWS_PARTS
+from .block_sizes import FEW_ROWS, FEW_ROWS_MAX_WEIGHT, FEW_ROWS_PARTS
 from .registry import build_part, register_part
 
 
@@ -158,7 +158,7 @@ class PagedAttention:
             raise RuntimeError("attention was given no cache")
         lazy = None
         if isinstance(x, StreamInput):
-            if ctx.rt.dtype == torch.bfloat16 and ops.gemm_norm_supported(x.rows, self.w_qkv):
+            if ctx.rt.dtype == torch.bfloat16 and self.w_qkv.numel() <= FEW_ROWS_MAX_WEIGHT and ops.gemm_norm_supported(x.rows, self.w_qkv):
                 lazy, x = x, x.stream.h
             else:
                 x = x.materialize()

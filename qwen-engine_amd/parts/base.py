@@ -111,11 +111,18 @@ class StreamInput:
     def rows(self) -> int:
         return self.stream.h.shape[0]
 
+    # Every block of the product reads the rows and all partial products of all rows: beyond this
+    # many bytes a block the norm's own kernel, which reads them once, is quicker.
+    FUSED_BYTES_PER_BLOCK = 192 * 1024
+
     def fusable(self) -> bool:
-        """True if a product can take the residual sum and the norm as its prologue: nothing to
-        add, or float32 partial products and a second buffer for the sums."""
+        """True if a product should take the residual sum and the norm as its prologue: nothing to
+        add, or float32 partial products and a second buffer for the sums; and little enough to read."""
         d = self.delta
-        return d is None or (d.dim() == 3 and d.dtype == torch.float32 and self.stream.spare is not None)
+        if d is not None and not (d.dim() == 3 and d.dtype == torch.float32 and self.stream.spare is not None):
+            return False
+        parts = 1 + (d.shape[0] if d is not None else 0)
+        return self.stream.h.numel() * 4 * parts <= self.FUSED_BYTES_PER_BLOCK
 
     def gemm(self, ops, w: torch.Tensor, bias=None, **kw) -> torch.Tensor:
         """The product of the normed rows with w, the residual sum and the norm inside it."""

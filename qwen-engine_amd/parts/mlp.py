@@ -10,7 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import Runtime, StreamInput, TensorInfo
-from .block_sizes import FEW_ROWS, FEW_ROWS_PARTS
+from .block_sizes import FEW_ROWS, FEW_ROWS_MAX_WEIGHT, FEW_ROWS_PARTS
 from .registry import register_part
 
 
@@ -47,7 +47,7 @@ class SwiGLU:
         x: the normed rows, or a StreamInput."""
         a = None
         if isinstance(x, StreamInput):
-            if ctx.rt.dtype == torch.bfloat16 and ops.gemm_norm_supported(x.rows, self.w_gu):
+            if ctx.rt.dtype == torch.bfloat16 and self.w_gu.numel() <= FEW_ROWS_MAX_WEIGHT and ops.gemm_norm_supported(x.rows, self.w_gu):
                 a = x.gemm(ops, self.w_gu, epilogue=ops.EPI_SILU_MUL_IL if self.interleaved else ops.EPI_SILU_MUL)
             else:
                 x = x.materialize()
