@@ -118,7 +118,7 @@ extern "C" int qe_gemm(const void* x, const void* w, const float* bias, void* ou
     }
     if (epilogue == EPI_PARTIAL && (tiled_for_few_rows(M, N, K, dt_a, dt_w) || (!skinny && tiled))) {
         QE_REQUIRE(dt_o == QE_F32, "gemm: partial products are 32-bit");
-        return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, 0, false, splits, stream);
+        return qe_gemm_mfma(x, w, bias, out, M, N, K, dt_o, algo > ALGO_TILE ? algo - ALGO_TILE : 0, false, splits, stream);
     }
     if (epilogue != EPI_STORE) {
         QE_REQUIRE(skinny, "gemm: M=%d N=%d K=%d with these element types is not taken by the kernel for few rows", M, N, K);
