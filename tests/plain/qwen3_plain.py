@@ -224,3 +224,29 @@ def greedy_generate(cfg: dict, w, prompt: List[int], max_new_tokens: int,
         out.append(nxt)
         tokens.append(nxt)
     return out
+
+
+# ----------------------------------------------------------------------------
+# temperature sampling (not in the reference, which is greedy only)
+# ----------------------------------------------------------------------------
+def uniform_number(seed: int, request: int, position: int) -> float:
+    """The engine's rule for the one uniform number of a draw: the first 24 of the 64 bits (little
+    endian) of blake2b-8 over the three numbers as little-endian int64, as a fraction of 2^24."""
+    import hashlib
+    import struct
+    digest = hashlib.blake2b(struct.pack("<qqq", seed, request, position), digest_size=8).digest()
+    return (int.from_bytes(digest, "little") >> 40) / float(1 << 24)
+
+
+def sample_temperature(logits: torch.Tensor, temperature: float, u: float):
+    """Inverse CDF of softmax(logits / temperature): the first token whose running sum of weights
+    (in index order, 64-bit) exceeds u times the total.  Also returns how far u lies from the nearer
+    edge of that token's interval, as a fraction of the total: a draw nearer to an edge than the
+    logits are exact may fall on either side."""
+    z = logits.double() / temperature
+    w = torch.exp(z - z.max())
+    cdf = torch.cumsum(w, dim=0) / w.sum()
+    tok = int(torch.searchsorted(cdf, torch.tensor(u, dtype=torch.float64), right=True))
+    tok = min(tok, logits.numel() - 1)
+    lower = float(cdf[tok - 1]) if tok > 0 else 0.0
+    return tok, min(u - lower, float(cdf[tok]) - u)

@@ -124,6 +124,30 @@ def test_shared_prefix_pages_are_taken_over(folders):
     assert res[1].token_ids == P.greedy_generate(cfg, w, b, 4)
 
 
+def test_temperature_sampling_equals_the_plain_draw(folders):
+    """Every token that the engine draws at temperature 0.8 is the plain implementation's draw from
+    the plain logits of the engine's own sequence, with the same uniform number per (seed, request,
+    output position); draws that lie within 1e-4 of an edge of their token's interval are not judged."""
+    cfg, w = P.read_folder(folders["A"])
+    prompts = prompts_for(cfg, (5, 9, 13, 2), 12)
+    eng = LLMEngine.from_folder(folders["A"], EngineConfig(dtype="float32", block_size=4, max_num_seqs=3, max_model_len=64))
+    first_id = eng._next_id
+    eng.submit(prompts, max_new_tokens=12, temperature=0.8, seed=77, ignore_eos=True)
+    res = eng.run()
+    judged = 0
+    for i, (r, prompt) in enumerate(zip(res, prompts)):
+        logits = P.forward_logits(cfg, w, prompt + r.token_ids[:-1])
+        for k, tok in enumerate(r.token_ids):
+            u = P.uniform_number(77, first_id + i, k)
+            want, margin = P.sample_temperature(logits[len(prompt) - 1 + k], 0.8, u)
+            if margin > 1e-4:
+                assert tok == want, (i, k, tok, want)
+                judged += 1
+    assert judged >= 40
+    greedy = [P.greedy_generate(cfg, w, p, 12) for p in prompts]
+    assert [r.token_ids for r in res] != greedy
+
+
 def test_requests_submitted_together_share_their_beginning(folders):
     """Two prompts with 32 tokens in common and one that shares nothing, submitted in one call (the
     reference's prompts 2 and 3 begin alike, main.py:64-68): the second of the pair waits for the

@@ -238,3 +238,27 @@ def test_the_per_head_norm_runs_before_the_rotation(tmp_path):
 
 def test_greedy_takes_the_lowest_index_on_ties():
     assert P.greedy(torch.tensor([[1.0, 3.0, 3.0, 2.0], [0.0, 0.0, 0.0, 0.0]])) == [1, 0]
+
+
+def test_temperature_draw_is_the_inverse_cdf_of_the_softmax():
+    logits = torch.tensor([0.3, -1.0, 2.0, 0.3, 1.1])
+    p = torch.softmax(logits.double() / 0.7, dim=0)
+    edges = torch.cumsum(p, 0)
+    # a draw just inside each token's interval gives that token; the margin is the distance to its edge
+    for tok in range(5):
+        lo = float(edges[tok - 1]) if tok else 0.0
+        got, margin = P.sample_temperature(logits, 0.7, lo + 0.25 * float(p[tok]))
+        assert got == tok and abs(margin - 0.25 * float(p[tok])) < 1e-12
+    assert P.sample_temperature(logits, 0.7, 0.0)[0] == 0 and P.sample_temperature(logits, 0.7, 0.999999)[0] == 4
+    # over evenly spread draws the tokens come with the softmax's frequencies
+    n = 20000
+    counts = torch.zeros(5)
+    for i in range(n):
+        counts[P.sample_temperature(logits, 0.7, (i + 0.5) / n)[0]] += 1
+    assert float((counts / n - p.float()).abs().max()) < 1e-3
+    # a low temperature draws the largest logit whatever the number
+    assert all(P.sample_temperature(logits, 0.01, u)[0] == 2 for u in (1e-9, 0.3, 0.9999))
+    # the uniform number: 24 bits, fixed by its three arguments, different for neighbours
+    u = P.uniform_number(5, 2, 9)
+    assert 0.0 <= u < 1.0 and u * (1 << 24) == int(u * (1 << 24)) and u == P.uniform_number(5, 2, 9)
+    assert len({P.uniform_number(5, 2, k) for k in range(50)}) == 50
