@@ -1,5 +1,7 @@
 // Attention of a flat batch of new tokens over the paged cache, any sizes, all
-// arithmetic in 32-bit.  One wave per (token, query head).
+// arithmetic in 32-bit.  One wave per (token, query head).  (The fallback of the bfloat16 mode for
+// sizes the MFMA kernels refuse, and of the float32 mode for head sizes that are no multiple of 16;
+// float32 otherwise goes to attention_f32.hip.)
 //
 // The query of token t at absolute position p = positions[t] of request
 // s = tok_seq[t] sees the keys at positions lo..p of that request, read through
@@ -86,10 +88,23 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     }
 }
 
+bool qe_attention_f32_ok(int Hq, int Hkv, int D, int P);
+int qe_attention_f32(const float* q, float* out, const float* cache, const int* positions, const int* tok_seq,
+                     const int* block_table, int max_blocks, const int* tokens, int T, int Hq, int Hkv, int D,
+                     int P, float scale, int window, hipStream_t stream);
+
+// 32-bit attention goes to the kernel on the matrix units (attention_f32.hip) where it takes the
+// sizes; qe_attention_use_matrix_f32(0) keeps it on the kernel below (for comparing the two).
+static int g_matrix_f32 = 1;
+extern "C" void qe_attention_use_matrix_f32(int on) { g_matrix_f32 = on; }
+
 int qe_attention_generic(const void* q, void* out, const void* cache, const int* positions,
                          const int* tok_seq, const int* block_table, int max_blocks, const int* tokens,
                          int T, int Hq, int Hkv, int D, int P, float scale, int window, int dt_a,
                          hipStream_t stream) {
+    if (dt_a == QE_F32 && g_matrix_f32 && qe_attention_f32_ok(Hq, Hkv, D, P))
+        return qe_attention_f32((const float*)q, (float*)out, (const float*)cache, positions, tok_seq, block_table,
+                                max_blocks, tokens, T, Hq, Hkv, D, P, scale, window, stream);
     QE_REQUIRE(D <= ATTN_MAX_D, "attention: head_dim=%d exceeds %d", D, ATTN_MAX_D);
     QE_REQUIRE(Hq <= 65535, "attention: too many heads");
     dim3 grid(T, Hq);

@@ -924,3 +924,57 @@ def test_gemm_norm_prologue_refuses_what_it_does_not_take(ops):
         ops.gemm(torch.zeros(4, 64, device=DEV, dtype=bf), w, norm_weight=nw, norm_eps=1e-6)
     with pytest.raises(ops.KernelError):                                 # partial products do not go with it
         ops.gemm(torch.zeros(4, 64, device=DEV), w, epilogue=ops.EPI_PARTIAL, norm_weight=nw, norm_eps=1e-6)
+
+
+@pytest.mark.parametrize("hq,hkv,d,page", [(4, 2, 16, 4), (6, 1, 32, 3), (6, 2, 48, 16), (40, 2, 64, 5), (3, 3, 80, 1),
+                                           (16, 8, 128, 16), (2, 1, 256, 64), (34, 1, 16, 8)])
+@pytest.mark.parametrize("window", [0, 37])
+def test_float32_attention_on_the_matrix_units(ops, hq, hkv, d, page, window):
+    """The float32 kernel on the matrix units (heads as columns, 16 keys a tile, any page size, more
+    than 16 heads a group in several waves) against the plain attention and against the
+    one-wave-a-head kernel, which sums in another order: portions and single tokens of three
+    requests, one of them starting at position 0; unused pages and the ends of pages hold NaN."""
+    scale = 0.7 / math.sqrt(d)
+    lens = [(140, 9), (70, 1), (0, 21)]
+    qs, pos, seq, tables, caches, want = [], [], [], [], [], []
+    base_page = 0
+    for b, (before, n) in enumerate(lens):
+        L = before + n
+        k, v = rand(L, hkv, d, seed=610 + b), rand(L, hkv, d, seed=620 + b)
+        q = rand(n, hq, d, seed=630 + b)
+        cache, ids = paged_cache(k, v, page, 640 + b, torch.float32)
+        tables.append(ids + base_page)
+        base_page += cache.shape[0]
+        caches.append(cache)
+        qs.append(q)
+        pos += list(range(before, L))
+        seq += [b] * n
+        want.append(P.attention(q, k, v, scale, window=window or None))
+    width = max(len(t) for t in tables)
+    table = torch.full((len(lens), width), -1, dtype=torch.int32)
+    for b, t in enumerate(tables):
+        table[b, :len(t)] = t
+    args = (torch.cat(qs).to(DEV), torch.cat(caches).to(DEV), torch.tensor(pos, dtype=torch.int32, device=DEV),
+            torch.tensor(seq, dtype=torch.int32, device=DEV), table.to(DEV), scale)
+    out = ops.attention(*args, window=window)
+    assert not torch.isnan(out).any()
+    close(out, torch.cat(want), torch.float32)
+    try:
+        ops.attention_use_matrix_f32(False)
+        other = ops.attention(*args, window=window)
+    finally:
+        ops.attention_use_matrix_f32(True)
+    close(other, torch.cat(want), torch.float32)
+    assert not torch.equal(other, out) or d == 16          # (two kernels, two orders of the sums)
+    # a subset of the rows, as the engine asks for when the others go to another kernel
+    rows = torch.tensor([0, 9, 10, 30], dtype=torch.int32, device=DEV)
+    part = torch.full_like(out, float("nan"))
+    q_all = args[0]
+    from qwen_engine_amd.kernels.ops import load_library, _DT
+    lib = load_library()
+    rc = lib.qe_attention(q_all.data_ptr(), part.data_ptr(), args[1].data_ptr(), args[2].data_ptr(), args[3].data_ptr(),
+                          args[4].data_ptr(), args[4].shape[1], rows.data_ptr(), 4, hq, hkv, d, page, scale, window, 0,
+                          torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(part[rows.long()], out[rows.long()]) and torch.isnan(part[1]).all()
