@@ -94,15 +94,14 @@ int qe_attention_f32(const float* q, float* out, const float* cache, const int* 
                      int P, float scale, int window, hipStream_t stream);
 
 // 32-bit attention goes to the kernel on the matrix units (attention_f32.hip) where it takes the
-// sizes; qe_attention_use_matrix_f32(0) keeps it on the kernel below (for comparing the two).
-static int g_matrix_f32 = 1;
-extern "C" void qe_attention_use_matrix_f32(int on) { g_matrix_f32 = on; }
+// sizes, unless qe_use_matrix_f32(0) has switched that off.
+extern int g_qe_matrix_f32;
 
 int qe_attention_generic(const void* q, void* out, const void* cache, const int* positions,
                          const int* tok_seq, const int* block_table, int max_blocks, const int* tokens,
                          int T, int Hq, int Hkv, int D, int P, float scale, int window, int dt_a,
                          hipStream_t stream) {
-    if (dt_a == QE_F32 && g_matrix_f32 && qe_attention_f32_ok(Hq, Hkv, D, P))
+    if (dt_a == QE_F32 && g_qe_matrix_f32 && qe_attention_f32_ok(Hq, Hkv, D, P))
         return qe_attention_f32((const float*)q, (float*)out, (const float*)cache, positions, tok_seq, block_table,
                                 max_blocks, tokens, T, Hq, Hkv, D, P, scale, window, stream);
     QE_REQUIRE(D <= ATTN_MAX_D, "attention: head_dim=%d exceeds %d", D, ATTN_MAX_D);

@@ -1,7 +1,7 @@
 // out[M, N] = x[M, K] . W[N, K]^T (+ bias), every multiply-add in IEEE 32-bit.
 // Takes any M, N, K and every pairing of activation/weight/output element type
-// that the engine uses.  This is the kernel of the float32 mode and the fallback
-// of the bfloat16 mode for shapes the MFMA kernels refuse.
+// that the engine uses.  This is the fallback of the bfloat16 mode for shapes the MFMA
+// kernels refuse (the float32 mode's products go to gemm_f32.hip).
 //
 // 64x64 output tile per block of 256 threads, 4x4 outputs per thread, K in steps
 // of 16 through shared memory.  Each output is summed over k in ascending order,
@@ -76,9 +76,15 @@ static int launch_generic(const void* x, const void* w, const float* bias, void*
     return 0;
 }
 
+int qe_gemm_f32(const float* x, const float* w, const float* bias, float* out, int M, int N, int K,
+                hipStream_t stream);
+extern int g_qe_matrix_f32;      // the all-float32 product goes to the matrix units (gemm_f32.hip) unless switched off
+
 int qe_gemm_generic(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                     int dt_a, int dt_w, int dt_o, hipStream_t stream) {
     QE_REQUIRE(qe_cdiv(M, GT) <= 65535, "gemm: M=%d is too large for one launch", M);
+    if (dt_a == QE_F32 && dt_w == QE_F32 && dt_o == QE_F32 && g_qe_matrix_f32)
+        return qe_gemm_f32((const float*)x, (const float*)w, bias, (float*)out, M, N, K, stream);
     if (dt_a == QE_F32 && dt_w == QE_F32 && dt_o == QE_F32)
         return launch_generic<float, float, float>(x, w, bias, out, M, N, K, stream);
     if (dt_a == QE_BF16 && dt_w == QE_BF16 && dt_o == QE_BF16)

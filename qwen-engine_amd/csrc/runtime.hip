@@ -15,3 +15,9 @@ void qe_set_error(const char* fmt, ...) {
 extern "C" const char* qe_last_error() { return g_error; }
 
 extern "C" int qe_abi_version() { return 1; }
+
+// The float32 mode's attention and matrix products run on the matrix units (attention_f32.hip,
+// gemm_f32.hip) unless this is switched off: then on the vector units' kernels, which sum in another
+// order (for comparing the two).
+int g_qe_matrix_f32 = 1;
+extern "C" void qe_use_matrix_f32(int on) { g_qe_matrix_f32 = on; }

@@ -74,8 +74,8 @@ def load_library():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = ctypes.c_int
-    lib.qe_attention_use_matrix_f32.argtypes = [i32]
-    lib.qe_attention_use_matrix_f32.restype = None
+    lib.qe_use_matrix_f32.argtypes = [i32]
+    lib.qe_use_matrix_f32.restype = None
     lib.qe_mfma_probe.argtypes = [vp, i32, i32, ctypes.POINTER(ctypes.c_double), vp]
     lib.qe_mfma_probe.restype = ctypes.c_int
     lib.qe_argmax_workspace_bytes.argtypes = [i32, i32]
@@ -498,9 +498,10 @@ def qk_rope_store_parts(parts: torch.Tensor, bias: Optional[torch.Tensor], num_h
     return q_out
 
 
-def attention_use_matrix_f32(on: bool) -> None:
-    """float32 attention on the matrix units (the default) or on the one-wave-a-head kernel."""
-    load_library().qe_attention_use_matrix_f32(int(bool(on)))
+def use_matrix_f32(on: bool) -> None:
+    """The float32 mode's attention and products on the matrix units (the default), or on the vector
+    units' kernels, which sum in another order (for comparing the two)."""
+    load_library().qe_use_matrix_f32(int(bool(on)))
 
 
 def attention_decode_supported(q: torch.Tensor, cache: torch.Tensor) -> bool:

@@ -960,10 +960,10 @@ def test_float32_attention_on_the_matrix_units(ops, hq, hkv, d, page, window):
     assert not torch.isnan(out).any()
     close(out, torch.cat(want), torch.float32)
     try:
-        ops.attention_use_matrix_f32(False)
+        ops.use_matrix_f32(False)
         other = ops.attention(*args, window=window)
     finally:
-        ops.attention_use_matrix_f32(True)
+        ops.use_matrix_f32(True)
     close(other, torch.cat(want), torch.float32)
     assert not torch.equal(other, out) or d == 16          # (two kernels, two orders of the sums)
     # a subset of the rows, as the engine asks for when the others go to another kernel
@@ -978,3 +978,25 @@ def test_float32_attention_on_the_matrix_units(ops, hq, hkv, d, page, window):
     assert rc == 0
     torch.cuda.synchronize()
     assert torch.equal(part[rows.long()], out[rows.long()]) and torch.isnan(part[1]).all()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 500, 96), (5, 331, 80), (64, 64, 64), (130, 77, 200), (3, 2048, 1024), (257, 130, 30),
+                                   (70, 65, 17), (2048, 192, 1024)])
+def test_float32_gemm_on_the_matrix_units(ops, M, N, K):
+    """The float32 product on the matrix units against the 64-bit product, tighter than the vector
+    units' kernel needs, and against that kernel; rows give the same bits whatever else is in the batch."""
+    x, w = rand(M, K, seed=650), rand(N, K, seed=651, scale=0.1)
+    bias = rand(N, seed=652)
+    want = P.linear(x.double(), w.double())
+    got = ops.gemm(x.to(DEV), w.to(DEV))
+    close(got, want, torch.float32)
+    close(ops.gemm(x.to(DEV), w.to(DEV), bias.to(DEV)), want + bias.double(), torch.float32)
+    try:
+        ops.use_matrix_f32(False)
+        other = ops.gemm(x.to(DEV), w.to(DEV))
+    finally:
+        ops.use_matrix_f32(True)
+    close(other, want, torch.float32)
+    # a row alone and the same row among the others: the same bits
+    alone = ops.gemm(x[M // 2:M // 2 + 1].to(DEV), w.to(DEV))
+    assert torch.equal(alone[0], got[M // 2])
