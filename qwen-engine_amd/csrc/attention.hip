@@ -20,7 +20,11 @@ int qe_attention_decode(const void* q, void* out, const void* cache, const int* 
 
 int qe_attention_prefill(const void* q, void* out, const void* cache, const int* tiles, int num_tiles,
                          const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
-                         int Hq, int Hkv, int D, int P, float scale, int window, int groups, hipStream_t stream);
+                         int Hq, int Hkv, int D, int P, float scale, int window, int groups,
+                         int seg_keys, int max_keys, void* workspace, size_t workspace_bytes, hipStream_t stream);
+int qe_attention_prefill_segment_keys(long blocks, int max_keys);
+int qe_attention_prefill_uncut_keys();
+size_t qe_attention_prefill_workspace(int num_tiles, int Hq, int Hkv, int D, int segments);
 
 int qe_attention_prefill_tile_rows(int Hq, int Hkv);
 
@@ -30,16 +34,38 @@ extern "C" int qe_attention_prefill_rows(int Hq, int Hkv) {
     return qe_attention_prefill_tile_rows(Hq, Hkv);
 }
 
+// Into segments of how many keys the prefill kernel's walks are best cut for num_tiles tiles whose
+// rows see at most max_keys keys: 0 for not at all.
+extern "C" int qe_attention_prefill_plan(int num_tiles, int Hq, int Hkv, int max_keys) {
+    if (num_tiles <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || max_keys <= 0) return 0;
+    const int R = qe_attention_prefill_tile_rows(Hq, Hkv);
+    return qe_attention_prefill_segment_keys((long)(num_tiles / 4) * Hkv * ((Hq / Hkv) / (32 / R)), max_keys);
+}
+
+// up to this many keys the plan is never to cut
+extern "C" int qe_attention_prefill_plan_uncut_keys() { return qe_attention_prefill_uncut_keys(); }
+
+// bytes of workspace for segments of seg_keys keys (> 0)
+extern "C" long qe_attention_prefill_workspace_bytes(int num_tiles, int Hq, int Hkv, int D, int max_keys, int seg_keys) {
+    if (seg_keys <= 0 || max_keys <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv) return 0;
+    return (long)qe_attention_prefill_workspace(num_tiles, Hq, Hkv, D, (max_keys + seg_keys - 1) / seg_keys);
+}
+
 // tiles: num_tiles pairs (first row of q, rows <= qe_attention_prefill_rows) of consecutive new
 // tokens of one request.  Takes what qe_attention_prefill_supported takes.  groups: wave groups
 // a block that share the key tiles between them, 1 or 2, or 0 to choose by the number of blocks.
+// seg_keys: 0, or the keys of a segment (a multiple of 64) into which the walks are cut; then no row
+// sees more than max_keys keys and the workspace has qe_attention_prefill_workspace_bytes bytes.
 extern "C" int qe_attention_prefill_run(const void* q, void* out, const void* cache, const int* tiles,
                                         int num_tiles, const int* positions, const int* tok_seq,
                                         const int* block_table, int max_blocks, int Hq, int Hkv, int D, int P,
-                                        float scale, int window, int groups, hipStream_t stream) {
-    QE_REQUIRE(num_tiles >= 0 && Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0, "prefill attention: bad sizes");
+                                        float scale, int window, int groups, int seg_keys, int max_keys,
+                                        void* workspace, long workspace_bytes, hipStream_t stream) {
+    QE_REQUIRE(num_tiles >= 0 && Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && seg_keys >= 0 &&
+               workspace_bytes >= 0, "prefill attention: bad sizes");
     return qe_attention_prefill(q, out, cache, tiles, num_tiles, positions, tok_seq, block_table, max_blocks,
-                                Hq, Hkv, D, P, scale, window, groups, stream);
+                                Hq, Hkv, D, P, scale, window, groups, seg_keys, max_keys, workspace,
+                                (size_t)workspace_bytes, stream);
 }
 
 // tokens: null for all T rows of q, else n_tokens row indices.

@@ -28,6 +28,14 @@
 // end group 0 merges the two partial results (maxima, sums, accumulators) through shared memory.
 // That halves the length of the longest block, which is what the time of a causal prompt hangs on
 // when there are no more blocks than compute units.  The longest blocks are started first.
+//
+// Key segments: with few blocks and many keys (a portion of a prompt far into its context; one
+// whole prompt, whose last rows see all of it) the keys are cut at absolute multiples of seg_keys
+// and block z of the grid's third dimension walks only the keys of segment z.  A block whose rows'
+// keys lie in one segment writes its result as before (the blocks of the other segments leave at
+// once); else the blocks of the segments that hold keys of its rows leave their maxima, sums and
+// accumulators, as the lanes hold them, in a workspace, and attention_prefill_merge_kernel, with the
+// same grid and the same lanes, weighs and adds them in the order of the segments.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -57,7 +65,25 @@ __device__ __forceinline__ float sum_of_both_halves(float v) {
     return a + b;
 }
 
+#define QE_PREFILL_UNCUT_KEYS 1024
 #define VROW 48   // bytes of a staged value row: 16 keys = 32 bytes of data + 16 of padding
+
+// A lane's share of its column's result: the accumulators' element 4 b + j of block db is feature
+// 32 db + 8 b + 4 g + j.
+template <int D>
+__device__ __forceinline__ void store_columns(bf16_t* __restrict__ out, const floatx16 (&acc)[D / 32], float inv,
+                                              int row, int head, int Hq, int g) {
+    bf16_t* orow = out + ((long)row * Hq + head) * D + 4 * g;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            bf16x4 o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = (__bf16)(acc[db][4 * b + j] * inv);
+            *(bf16x4*)(orow + db * 32 + 8 * b) = o;
+        }
+}
 
 // Two waves per SIMD (at most 256 registers a lane), as two blocks of one group or one block of
 // two: while one wave waits for its next tile or at its barrier, the other computes.
@@ -66,7 +92,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ tiles, const int* __restrict__ positions, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int max_blocks,
-    int Hq, int Hkv, int P, int log2P, float scale_log2, int window, int R) {
+    int Hq, int Hkv, int P, int log2P, float scale_log2, int window, int R, int seg_keys, float* __restrict__ part) {
     constexpr int KROW = D * 2 + 16;                 // bytes of a staged key row
     constexpr int KBYTES = 32 * KROW, VBYTES = 2 * D * VROW, BUF = KBYTES + VBYTES;
     constexpr int KP = 32 * (D / 8) / 256;           // 16-byte key pieces per thread (2 for D = 128)
@@ -81,18 +107,33 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     const int g = lane >> 5, r = lane & 31;
     const int G = Hq / Hkv;
     const int GH = 32 / R;                                 // heads per wave
-    const int kvh = blockIdx.y / (G / GH);
-    const int head = kvh * G + (blockIdx.y % (G / GH)) * GH + r / R;   // this lane's column: head and row
+    // The grid is (head waves, segments, tile groups): blocks start in the order of the first
+    // dimension first, so all heads and segments of the last rows (the longest walks) start before
+    // anything of earlier rows, and a compute unit that is done takes the longest of what is left.
+    const int bhead = blockIdx.x, bseg = blockIdx.y, bgroup = blockIdx.z;
+    const int kvh = bhead / (G / GH);
+    const int head = kvh * G + (bhead % (G / GH)) * GH + r / R;   // this lane's column: head and row
 
     // the block's four tiles belong to one request, in ascending rows; tiles of 0 rows pad the group
-    const int* bt4 = tiles + 8 * (gridDim.x - 1 - blockIdx.x);   // later rows see more keys: they start first
+    const int* bt4 = tiles + 8 * (gridDim.z - 1 - bgroup);   // later rows see more keys: they start first
     const int row_first = bt4[0];
     int last = 0;
 #pragma unroll
     for (int j = 1; j < 4; ++j) if (bt4[2 * j + 1] > 0) last = j;
     const int p_block = positions[row_first];
-    const int kmin = (window > 0 && p_block - window + 1 > 0) ? p_block - window + 1 : 0;
-    const int kmax = positions[bt4[2 * last]] + bt4[2 * last + 1];
+    int kmin = (window > 0 && p_block - window + 1 > 0) ? p_block - window + 1 : 0;
+    int kmax = positions[bt4[2 * last]] + bt4[2 * last + 1];
+    // key segments: this block walks the keys of segment bseg only
+    bool partial = false;
+    if (seg_keys > 0) {
+        const int z = bseg, z_lo = kmin / seg_keys, z_hi = (kmax - 1) / seg_keys;
+        if (z < z_lo || z > z_hi) return;                  // (the whole block: no barrier has been met yet)
+        partial = z_hi > z_lo;
+        if (partial) {
+            kmin = max(kmin, z * seg_keys);
+            kmax = min(kmax, (z + 1) * seg_keys);
+        }
+    }
     const int* bt = block_table + (long)tok_seq[row_first] * max_blocks;
     const long page_stride = 2L * Hkv * P * D;
 
@@ -230,7 +271,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
         const int kk_1 = TILE_KEY(i + 1), kk_2 = TILE_KEY(i + 2);   // (values, not expressions in i: the macros have loops over i)
         STAGE_LOAD(buf, EXISTING(kk_2))                   // this set's tile went to shared memory a round ago
         __builtin_amdgcn_sched_barrier(0);                // keep the loads ahead of the computation
-        if (wave_on && kk < k_stop && kk + 32 > k_start) { // some row of the wave sees some key of the tile (none beyond kmax)
+        if (wave_on && kk < k_stop && kk + 32 > k_start && kk < kmax) {   // some row of the wave sees some key of the tile, and it is a tile of this block's keys
             const unsigned char* ks_ = smem + buf * BUF + r * KROW + g * 16;
             const unsigned char* vs_ = smem + buf * BUF + KBYTES + r * VROW + g * 16;
             // all key fragments are read before the first MFMA, all value fragments before the
@@ -320,6 +361,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
             a_own = __builtin_amdgcn_exp2f(m - ref);       // 0 for a side that has seen no key
             a_other = __builtin_amdgcn_exp2f(m1 - ref);
             l = l * a_own + l1 * a_other;
+            m = mt;
         }
 #pragma unroll
         for (int db = 0; db < D / 32; ++db) {
@@ -336,18 +378,74 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
         }
         if (grp == 1) return;
     }
-    if (col_ok) {
-        const float inv = 1.f / l;
-        bf16_t* orow = out + ((long)row * Hq + head) * D + 4 * g;
+    if (partial) {
+        // as the lanes hold them: [segment][block][wave][value][lane], value = m, l, then the accumulators
+        constexpr int NV = 2 + (D / 32) * 16;
+        float* dst = part + ((((long)bseg * gridDim.x + bhead) * gridDim.z + bgroup) * 4 + wave) * NV * 64 + lane;
+        dst[0] = m;
+        dst[64] = l;
+        if (m != -INFINITY) {                              // (a column that saw no key of the segment: nothing else is read of it)
 #pragma unroll
-        for (int db = 0; db < D / 32; ++db)
+            for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                bf16x4 o;
+                for (int e = 0; e < 16; ++e) dst[(2 + db * 16 + e) * 64] = acc[db][e];
+        }
+        return;
+    }
+    if (col_ok) store_columns<D>(out, acc, 1.f / l, row, head, Hq, g);
+}
+
+// The segments' partial results of the blocks that left some: the same first two grid dimensions
+// and the same lanes as the kernel above, the third dimension being the block of 32 features;
+// lane by lane, in the order of the segments.
+template <int D>
+__global__ __launch_bounds__(256) void attention_prefill_merge_kernel(
+    const float* __restrict__ part, bf16_t* __restrict__ out, const int* __restrict__ tiles,
+    const int* __restrict__ positions, int Hq, int Hkv, int window, int R, int seg_keys) {
+    constexpr int NV = 2 + (D / 32) * 16;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 5, r = lane & 31;
+    const int G = Hq / Hkv, GH = 32 / R;
+    const int bhead = blockIdx.x, db = blockIdx.y, bgroup = blockIdx.z;     // (head waves, feature blocks, tile groups)
+    const int kvh = bhead / (G / GH);
+    const int head = kvh * G + (bhead % (G / GH)) * GH + r / R;
+    const int* bt4 = tiles + 8 * (gridDim.z - 1 - bgroup);
+    const int row_first = bt4[0];
+    int last = 0;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) o[j] = (__bf16)(acc[db][4 * b + j] * inv);
-                *(bf16x4*)(orow + db * 32 + 8 * b) = o;
-            }
+    for (int j = 1; j < 4; ++j) if (bt4[2 * j + 1] > 0) last = j;
+    const int p_block = positions[row_first];
+    const int kmin = (window > 0 && p_block - window + 1 > 0) ? p_block - window + 1 : 0;
+    const int kmax = positions[bt4[2 * last]] + bt4[2 * last + 1];
+    const int z_lo = kmin / seg_keys, z_hi = (kmax - 1) / seg_keys;
+    if (z_hi <= z_lo) return;                              // the block wrote its result itself
+    const int row0 = bt4[2 * wave], cnt = bt4[2 * wave + 1];
+    const int rr = r % R;
+    if (cnt <= 0 || rr >= cnt) return;
+    const int row = row0 + rr;
+    const long zstride = (long)gridDim.x * gridDim.z * 4 * NV * 64;
+    const float* src = part + (((long)bhead * gridDim.z + bgroup) * 4 + wave) * NV * 64 + lane;
+    float M = -INFINITY;
+    for (int z = z_lo; z <= z_hi; ++z) M = fmaxf(M, src[z * zstride]);
+    float l = 0.f;
+    floatx16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+    for (int z = z_lo; z <= z_hi; ++z) {
+        const float mz = src[z * zstride];
+        if (mz == -INFINITY) continue;                     // no key of this segment was seen by the column
+        const float wgt = __builtin_amdgcn_exp2f(mz - M);
+        l += wgt * src[z * zstride + 64];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[e] += wgt * src[z * zstride + (2 + db * 16 + e) * 64];
+    }
+    const float inv = 1.f / l;
+    bf16_t* orow = out + ((long)row * Hq + head) * D + 4 * g + db * 32;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        bf16x4 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = (__bf16)(acc[4 * b + j] * inv);
+        *(bf16x4*)(orow + 8 * b) = o;
     }
 }
 
@@ -358,12 +456,38 @@ int qe_attention_prefill_tile_rows(int Hq, int Hkv) {
     return 32 / (pow2 ? G : 1);
 }
 
+// How the keys of a call are best cut into segments: 0 (not at all) or the keys a segment (a multiple
+// of 64).  blocks: blocks of the grid without segments; max_keys: the most keys a row of the call
+// sees.  Every segment costs a trip of the partial results through memory, and more blocks than
+// compute units gained nothing where it was measured (a whole prompt of 1536 or 2048 tokens took
+// longer in two segments than in one), so there are only as many segments as fill the chip, of at
+// least 512 keys; up to QE_PREFILL_UNCUT_KEYS keys a walk is too short to be worth one.
+int qe_attention_prefill_uncut_keys() { return QE_PREFILL_UNCUT_KEYS; }
+
+int qe_attention_prefill_segment_keys(long blocks, int max_keys) {
+    if (blocks <= 0 || blocks > 128 || max_keys <= QE_PREFILL_UNCUT_KEYS) return 0;
+    long ks = 256 / blocks;                                // as many blocks as there are compute units, not more
+    if (ks > 8) ks = 8;
+    int seg = (int)(((max_keys + ks - 1) / ks + 63) / 64 * 64);
+    if (seg < 512) seg = 512;
+    return seg >= max_keys ? 0 : seg;
+}
+
+size_t qe_attention_prefill_workspace(int num_tiles, int Hq, int Hkv, int D, int segments) {
+    const int R = qe_attention_prefill_tile_rows(Hq, Hkv);
+    const long blocks = (long)(num_tiles / 4) * Hkv * ((Hq / Hkv) / (32 / R));
+    return (size_t)segments * blocks * 4 * (2 + (D / 32) * 16) * 64 * sizeof(float);
+}
+
 // tiles: num_tiles pairs (first row of q, number of rows <= qe_attention_prefill_tile_rows), in
 // groups of four that belong to one request, in ascending rows, with consecutive positions
 // through the group; a group is filled up with pairs of 0 rows.  num_tiles is a multiple of 4.
+// seg_keys: 0, or the keys of a segment (a multiple of 64) with max_keys, the most keys a row sees,
+// and a workspace of qe_attention_prefill_workspace(..., segments = ceil(max_keys / seg_keys)) bytes.
 int qe_attention_prefill(const void* q, void* out, const void* cache, const int* tiles, int num_tiles,
                          const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
-                         int Hq, int Hkv, int D, int P, float scale, int window, int groups, hipStream_t stream) {
+                         int Hq, int Hkv, int D, int P, float scale, int window, int groups,
+                         int seg_keys, int max_keys, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     QE_REQUIRE((D == 64 || D == 128) && P >= 16 && (P & (P - 1)) == 0 && Hq % Hkv == 0,
                "prefill attention: sizes not taken");
     int log2P = 0;
@@ -373,20 +497,39 @@ int qe_attention_prefill(const void* q, void* out, const void* cache, const int*
     if (num_tiles == 0) return 0;
     const int R = qe_attention_prefill_tile_rows(Hq, Hkv);
     const int waves_per_kv = (Hq / Hkv) / (32 / R);
-    QE_REQUIRE(Hkv * waves_per_kv <= 65535, "prefill attention: too many heads");
-    dim3 grid(num_tiles / 4, Hkv * waves_per_kv);
+    int segments = 1;
+    if (seg_keys > 0) {
+        QE_REQUIRE(seg_keys % 64 == 0 && max_keys > 0, "prefill attention: segments of %d keys (a multiple of 64), %d keys", seg_keys, max_keys);
+        segments = qe_cdiv(max_keys, seg_keys);
+        QE_REQUIRE(segments <= 64, "prefill attention: %d segments", segments);
+        if (segments <= 1) { seg_keys = 0; segments = 1; }
+        else
+            QE_REQUIRE(workspace && workspace_bytes >= qe_attention_prefill_workspace(num_tiles, Hq, Hkv, D, segments),
+                       "prefill attention: workspace of %zu bytes is too small", workspace_bytes);
+    }
+    QE_REQUIRE(num_tiles / 4 <= 65535, "prefill attention: %d tiles are too many for one launch", num_tiles);
+    dim3 grid(Hkv * waves_per_kv, segments, num_tiles / 4);
+    dim3 mgrid(Hkv * waves_per_kv, D / 32, num_tiles / 4);
     const float scale_log2 = scale * 1.4426950408889634f;
     // two groups a block where the blocks do not fill the compute units twice anyway
     // (groups: 0 = choose, 1 or 2)
-    if (groups == 0) groups = (long)grid.x * grid.y <= 256 ? 2 : 1;
+    if (groups == 0) groups = (long)grid.x * grid.z <= 256 ? 2 : 1;
     QE_REQUIRE(groups == 1 || groups == 2, "prefill attention: %d groups a block", groups);
 #define QE_PREFILL(D_, NG_)                                                                         \
     attention_prefill_kernel<D_, NG_><<<grid, 256 * NG_, 0, stream>>>(                              \
         (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, tiles, positions, tok_seq, block_table, \
-        max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R)
+        max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R, seg_keys, (float*)workspace)
     if (D == 128) { if (groups == 2) QE_PREFILL(128, 2); else QE_PREFILL(128, 1); }
     else          { if (groups == 2) QE_PREFILL(64, 2); else QE_PREFILL(64, 1); }
 #undef QE_PREFILL
+    if (seg_keys > 0) {
+        if (D == 128)
+            attention_prefill_merge_kernel<128><<<mgrid, 256, 0, stream>>>((const float*)workspace, (bf16_t*)out, tiles,
+                                                                           positions, Hq, Hkv, window, R, seg_keys);
+        else
+            attention_prefill_merge_kernel<64><<<mgrid, 256, 0, stream>>>((const float*)workspace, (bf16_t*)out, tiles,
+                                                                          positions, Hq, Hkv, window, R, seg_keys);
+    }
     QE_LAUNCH_CHECK();
     return 0;
 }

@@ -493,12 +493,14 @@ class ModelRunner:
                     ops.scatter_int(self.tables[g], torch.from_numpy(upd_idx[g]).to(self.rt.device),
                                     torch.from_numpy(upd_val[g]).to(self.rt.device))
                 upd_idx[g] = upd_val[g] = np.zeros(0, dtype=i32)
-        key = ("portion", T, n_want)
+        part_keys = tuple(cls.portion_graph_key(T, seqs[0].kv_before + T) if hasattr(cls, "portion_graph_key") else None
+                          for cls in self._step_classes)
+        key = ("portion", T, n_want, part_keys)
         rec = self._graphs.pop(key, None)
         if rec is None:
             while len(self._graphs) >= self.MAX_GRAPHS:
                 self._graphs.pop(next(iter(self._graphs)))
-            rec = self._record_portion_graph(T, n_want, cap)
+            rec = self._record_portion_graph(T, n_want, cap, part_keys)
             self.graphs_recorded += 1
         self._graphs[key] = rec
         none, zero = rec["none"], rec["zero"]
@@ -514,9 +516,10 @@ class ModelRunner:
         self.graph_steps += 1
         return rec["logits"].clone()
 
-    def _record_portion_graph(self, T: int, n_want: int, cap: int):
+    def _record_portion_graph(self, T: int, n_want: int, cap: int, part_keys: tuple):
         """Static buffers for a step that is one prompt portion of T tokens with n_want (0 or 1) rows
-        of logits, one run outside the graph, then the recording.  The stand-in batch stands at
+        of logits, at a place that gives the parts' ``part_keys``, one run outside the graph, then the
+        recording.  The stand-in batch stands at
         positions 0 .. T - 1 of the tables' spare row (every entry page 0) and writes nowhere."""
         dev, n_groups = self.rt.device, len(self.cache.groups)
         n = 3 * T + n_want + 1 + n_groups * (T + 2 * cap)
@@ -543,7 +546,9 @@ class ModelRunner:
         ctx = StepContext(rt=self.rt, page_size=self.page_size, num_tokens=T, seqs=seqs, token_ids=d_tok,
                           positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
                           logit_rows=d_rows, state_slots=d_state, max_position=0,
-                          extras={cls: dict(cls.portion_graph_extras(T, dev)) for cls in self._step_classes})
+                          extras={cls: dict(cls.portion_graph_extras(T, dev) if k is None
+                                            else cls.portion_graph_extras(T, dev, k))
+                                  for cls, k in zip(self._step_classes, part_keys)})
 
         def run():
             for g in range(n_groups):

@@ -57,7 +57,11 @@ def load_library():
         "qe_attention_decode_supported": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_supported": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_rows": [i32, i32],
-        "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
+        "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, i32,
+                                     vp, i64, vp],
+        "qe_attention_prefill_plan": [i32, i32, i32, i32],
+        "qe_attention_prefill_plan_uncut_keys": [],
+        "qe_attention_prefill_workspace_bytes": [i32, i32, i32, i32, i32, i32],
         "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
         "qe_attention_decode_fused_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, f32, vp,
                                           i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
@@ -525,12 +529,19 @@ def prefill_tile_rows(num_heads: int, num_kv_heads: int) -> int:
     return load_library().qe_attention_prefill_rows(num_heads, num_kv_heads)
 
 
+def prefill_uncut_keys() -> int:
+    """Up to this many keys a row sees, the prefill attention kernel never cuts its walks into
+    segments of keys."""
+    return load_library().qe_attention_prefill_plan_uncut_keys()
+
+
 def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
               block_table: torch.Tensor, scale: float, window: int = 0,
               out: Optional[torch.Tensor] = None, algo: int = ALGO_AUTO,
               dec_tokens: Optional[torch.Tensor] = None, max_dec_position: int = 0,
               other_tokens: Optional[torch.Tensor] = None,
-              other_tiles: Optional[torch.Tensor] = None, prefill_groups: int = 0) -> torch.Tensor:
+              other_tiles: Optional[torch.Tensor] = None, prefill_groups: int = 0,
+              max_other_keys: int = 0, prefill_segment_keys: int = -1) -> torch.Tensor:
     """q [T, Hq, D]; cache [pages, 2, Hkv, P, D] (key tiles [P][D], value tiles transposed [D][P]);
     positions, tok_seq int32 [T]; block_table int32 [B, max_blocks].  Token t sees the keys at
     positions max(0, p - window + 1) .. p of request tok_seq[t] (window 0: all).  The caller
@@ -541,6 +552,9 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
     other_tokens are the remaining rows, and other_tiles (int32 [tiles, 2]: first row, number of
     rows <= prefill_tile_rows(Hq, Hkv), consecutive tokens of one request) the same rows cut
     for the prefill kernel (prefill_groups: its wave groups a block, 1 or 2, 0 to let it choose).
+    max_other_keys: no row of other_tiles sees more keys than this (its position + 1); when given,
+    the prefill kernel may cut long walks of few blocks into segments of keys (prefill_segment_keys:
+    their length, a multiple of 64; 0 for none; -1 to let it choose).
     Without the lists every row is treated alike."""
     lib = load_library()
     _need(q, "q", _ACT, (None, None, None))
@@ -585,11 +599,23 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
         _need(other_tokens, "other_tokens", torch.int32, (None,), dev)
         if other_tiles is not None and algo != ALGO_GENERIC and attention_prefill_supported(q, cache):
             _need(other_tiles, "other_tiles", torch.int32, (None, 2), dev)
+            n_tiles, max_keys, seg, ws, nbytes = other_tiles.shape[0], int(max_other_keys), 0, None, 0
+            if max_keys > 0:
+                seg = int(prefill_segment_keys)
+                if seg < 0:
+                    seg = lib.qe_attention_prefill_plan(n_tiles, Hq, Hkv, max_keys)
+                if seg >= max_keys:
+                    seg = 0
+            elif prefill_segment_keys > 0:
+                raise KernelError("attention: segments of keys need max_other_keys")
+            if seg > 0:
+                nbytes = lib.qe_attention_prefill_workspace_bytes(n_tiles, Hq, Hkv, D, max_keys, seg)
+                ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
             _check(lib.qe_attention_prefill_run(q.data_ptr(), out.data_ptr(), cache.data_ptr(),
-                                                other_tiles.data_ptr(), other_tiles.shape[0],
+                                                other_tiles.data_ptr(), n_tiles,
                                                 positions.data_ptr(), tok_seq.data_ptr(), block_table.data_ptr(),
                                                 max_blocks, Hq, Hkv, D, P, float(scale), int(window),
-                                                int(prefill_groups), _stream()),
+                                                int(prefill_groups), seg, max_keys, _ptr(ws), nbytes, _stream()),
                    "attention (prefill)")
         else:
             generic(other_tokens)

@@ -52,7 +52,8 @@ class PagedAttention:
         other = [np.arange(s.q_start, s.q_start + s.q_len, dtype=np.int32) for s in seqs if s.q_len > 1]
         return {"dec_tokens": np.asarray(dec, dtype=np.int32),
                 "other_tokens": np.concatenate(other) if other else np.zeros(0, dtype=np.int32),
-                "max_dec_position": max([s.kv_before for s in seqs if s.q_len == 1], default=0)}
+                "max_dec_position": max([s.kv_before for s in seqs if s.q_len == 1], default=0),
+                "max_other_keys": max([s.kv_before + s.q_len for s in seqs if s.q_len > 1], default=0)}
 
     GRAPH_SPLIT_BUCKET = 8      # a recorded decode step serves positions up to the next multiple of this many key splits
 
@@ -70,14 +71,25 @@ class PagedAttention:
                 "max_dec_position": key * ops.DECODE_SPLIT_KEYS - 1}
 
     @staticmethod
-    def portion_graph_extras(tokens: int, device) -> dict:
-        """For a recorded step that is one prompt portion of ``tokens`` rows: no single new tokens, all
-        rows in order; its launches do not depend on the positions."""
+    def portion_graph_key(tokens: int, keys: int) -> int:
+        """The prefill kernel cuts long walks into segments of keys by the most keys a row sees: a
+        recorded portion serves up to the next power of two of them."""
+        bound = ops.prefill_uncut_keys()                  # (up to here it cuts nothing: one recorded step for all)
+        while bound < keys:
+            bound *= 2
+        return bound
+
+    @staticmethod
+    def portion_graph_extras(tokens: int, device, key: int = 0) -> dict:
+        """For a recorded step that is one prompt portion of ``tokens`` rows whose last row sees at most
+        ``key`` keys: no single new tokens, all rows in order."""
         return {"dec_tokens": torch.zeros(0, dtype=torch.int32, device=device),
-                "other_tokens": torch.arange(tokens, dtype=torch.int32, device=device), "max_dec_position": 0}
+                "other_tokens": torch.arange(tokens, dtype=torch.int32, device=device), "max_dec_position": 0,
+                "max_other_keys": int(key)}
 
     def _extras(self, ctx) -> dict:
-        return ctx.extras.get(PagedAttention) or {"dec_tokens": None, "other_tokens": None, "max_dec_position": 0}
+        return ctx.extras.get(PagedAttention) or {"dec_tokens": None, "other_tokens": None, "max_dec_position": 0,
+                                                  "max_other_keys": 0}
 
     def _other_tiles(self, ctx) -> Optional[torch.Tensor]:
         """The rows of requests that bring several tokens, cut into tiles for the prefill kernel: built
@@ -221,7 +233,8 @@ class PagedAttention:
         o = ops.attention(q, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g], self.scale, self.window,
                           dec_tokens=ex["dec_tokens"], max_dec_position=ex["max_dec_position"],
                           other_tokens=ex["other_tokens"],
-                          other_tiles=self._other_tiles(ctx) if ex["other_tokens"] is not None else None)
+                          other_tiles=self._other_tiles(ctx) if ex["other_tokens"] is not None else None,
+                          max_other_keys=ex.get("max_other_keys", 0))
         return self._project_out(o.view(T, self.hq * self.d))
 
     def _project_out(self, o: torch.Tensor) -> torch.Tensor:

@@ -36,10 +36,14 @@ knows none of it.  A part class may define (all optional, all static):
   graph_extras(rows, key, device) -> dict   the same entries as step_extras for a recorded step of
                                  ``rows`` single new tokens whose positions give ``key``, as
                                  tensors that stay as they are for every replay
-  portion_graph_extras(tokens, device) -> dict   the same for a recorded step that is one prompt
-                                 portion of ``tokens`` rows (such steps are recorded per length only:
-                                 nothing of a part's launches may depend on their positions); without
-                                 it, portions of a model with this part run as they come
+  portion_graph_extras(tokens, device[, key]) -> dict   the same for a recorded step that is one
+                                 prompt portion of ``tokens`` rows; without it, portions of a model
+                                 with this part run as they come
+  portion_graph_key(tokens, keys)   what of such a portion's place the part's launches depend on
+                                 (keys: the keys its last row sees); the recorded step is replayed
+                                 only for the same key, which portion_graph_extras gets as its third
+                                 argument.  Without it nothing of the part's launches may depend on
+                                 the portion's positions.
 """
 from __future__ import annotations
 

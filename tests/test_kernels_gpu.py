@@ -791,6 +791,69 @@ def test_prefill_kernel_one_far_key_decides(ops, key_pos):
     assert float((want[last_seen:, 0] - v[key_pos, 0].float()).abs().max()) < 0.05
 
 
+@pytest.mark.parametrize("hq,hkv,d,page", [(16, 8, 128, 16), (4, 4, 64, 16), (8, 1, 128, 32), (6, 2, 64, 64)])
+@pytest.mark.parametrize("window", [0, 200, 70])
+def test_prefill_attention_over_key_segments(ops, hq, hkv, d, page, window):
+    """The keys cut into segments of 64 to 512 (and as the kernel chooses): a portion of 300 rows after
+    700 cached tokens, a whole prompt of 330 and two rows after 513, beside a decoded token.  Blocks
+    whose keys lie in one segment write their rows themselves, the others leave partial results
+    that the merge adds; the first key of the first request stands out for its first head, so every
+    row of that head (that still sees it) gets its weight from the first segment."""
+    bf = torch.bfloat16
+    scale = 1 / math.sqrt(d)
+    lens = [(700, 300), (0, 330), (513, 2), (90, 1)]
+    qs, pos, seq, tables, caches, want, portions, dec, other = [], [], [], [], [], [], [], [], []
+    base, row = 0, 0
+    R = ops.prefill_tile_rows(hq, hkv)
+    direction = rand(d, seed=119)
+    for b, (before, n) in enumerate(lens):
+        L = before + n
+        k, v = rand(L, hkv, d, seed=120 + b, dtype=bf, scale=0.3), rand(L, hkv, d, seed=130 + b, dtype=bf)
+        q = rand(n, hq, d, seed=140 + b, dtype=bf)
+        if b == 0:
+            q[:, 0] = (direction[None] + 0.05 * rand(n, d, seed=118)).to(bf)
+            k[0, 0] = (direction * 4).to(bf)
+        cache, ids = paged_cache(k, v, page, 150 + b, bf)
+        tables.append(ids + base)
+        base += cache.shape[0]
+        caches.append(cache)
+        qs.append(q)
+        pos += list(range(before, L))
+        seq += [b] * n
+        want.append(P.attention(q.float(), k.float(), v.float(), scale, window=window or None))
+        if b == 0 and not window:
+            assert float((want[-1][:, 0] - v[0, 0].float()).abs().max()) < 0.05
+        if n == 1:
+            dec.append(row)
+        else:
+            other += list(range(row, row + n))
+            portions.append((row, n))
+        row += n
+    from qwen_engine_amd.parts.attention import prefill_tiles
+    tiles = torch.tensor(prefill_tiles(portions, R), dtype=torch.int32).view(-1, 2).tolist()
+    width = max(len(t) for t in tables)
+    table = torch.full((len(lens), width), -1, dtype=torch.int32)
+    for b, t in enumerate(tables):
+        table[b, :len(t)] = t
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    args = (torch.cat(qs).to(DEV), torch.cat(caches).to(DEV), i32(pos), i32(seq), table.to(DEV), scale)
+    whole = ops.attention(*args, window=window, dec_tokens=i32(dec), max_dec_position=90, other_tokens=i32(other),
+                          other_tiles=i32(tiles), max_other_keys=1000, prefill_segment_keys=0)
+    close(whole, torch.cat(want), bf)
+    for seg, groups in ((64, 1), (64, 2), (128, 0), (256, 2), (512, 1), (512, 2), (960, 0), (-1, 0)):
+        out = ops.attention(*args, window=window, dec_tokens=i32(dec), max_dec_position=90, other_tokens=i32(other),
+                            other_tiles=i32(tiles), prefill_groups=groups, max_other_keys=1000 if seg != 960 else 1024,
+                            prefill_segment_keys=seg)
+        assert not torch.isnan(out.float()).any(), (seg, groups)
+        close(out, torch.cat(want), bf)
+        # rows whose keys lie in one segment come from the same sums as without segments
+        if seg == 512 and groups == 2:
+            assert torch.equal(out[300:630], whole[300:630])                 # the whole prompt of 330: keys 0 .. 329
+    with pytest.raises(ops.KernelError):
+        ops.attention(*args, other_tokens=i32(other), dec_tokens=i32(dec), max_dec_position=90, other_tiles=i32(tiles),
+                      max_other_keys=1000, prefill_segment_keys=100)
+
+
 @pytest.mark.parametrize("M", [1, 8, 64, 65, 200, 1024])
 @pytest.mark.parametrize("I,K", [(160, 96), (192, 64), (3072, 1024)])
 def test_gemm_with_silu_mul_over_interleaved_rows(ops, M, I, K):
