@@ -25,6 +25,7 @@ Other sizes and workloads (not what the default line reports):
                             portions of 512 tokens beside decoded tokens.  value = generated tokens a second
   --workload shared-prefix  N requests (default 32) that share a 1024-token prefix, each with 1024 tokens
                             of its own and 512 new tokens; the prefix's pages are shared
+  --prefill-portion N       the prefill in portions of N tokens, one step each, instead of one step
   --warmup-passes N         both: untimed passes over the workload with other tokens before the timed
                             one (default 1: the decode graphs are recorded there, as in a server that
                             has run for a while; 0 times the recording too)
@@ -67,6 +68,8 @@ def parse():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--prefill-portion", type=int, default=0,
+                    help="run the prefill in portions of this many tokens, one step each (0: one step)")
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
     ap.add_argument("--seed", type=int, default=0)
@@ -235,12 +238,15 @@ def main() -> int:
     def prefill_run(T, reps=3):
         runner = ModelRunner(model, page_size=P, num_pages=(T + P - 1) // P + 1, max_requests=1)
         toks = torch.randint(0, V, (T,), generator=g).tolist()
+        portion = args.prefill_portion or T
         best = None
         for _ in range(reps + 1):
             runner.add_request("p")
             torch.cuda.synchronize()
             t = time.perf_counter()
-            logits = runner.step([StepEntry("p", toks, [T - 1])])
+            for a in range(0, T, portion):
+                part = toks[a:a + portion]
+                logits = runner.step([StepEntry("p", part, [len(part) - 1] if a + portion >= T else [])])
             ops.argmax(logits).tolist()
             torch.cuda.synchronize()
             dt = time.perf_counter() - t
@@ -298,6 +304,7 @@ def main() -> int:
             "intermediate_size": I, "vocab_size": V, "tie_word_embeddings": cfg.tie_word_embeddings,
             "global_batch": args.batch, "seq_len": args.context, "page_size": P,
             "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU",
+            **({"prefill_portion": args.prefill_portion} if args.prefill_portion else {}),
         },
         "prefill": {"value": round(prefill["value"], 1), "tokens": prefill["tokens"],
                     "ms": round(prefill["ms"], 3), "frac": round(prefill["frac"], 4)},

@@ -21,8 +21,10 @@ int qe_attention_decode(const void* q, void* out, const void* cache, const int* 
 int qe_attention_prefill(const void* q, void* out, const void* cache, const int* tiles, int num_tiles,
                          const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
                          int Hq, int Hkv, int D, int P, float scale, int window, int groups,
-                         int seg_keys, int max_keys, void* workspace, size_t workspace_bytes, hipStream_t stream);
+                         int seg_keys, int max_keys, int keys_row, void* workspace, size_t workspace_bytes,
+                         hipStream_t stream);
 int qe_attention_prefill_segment_keys(long blocks, int max_keys);
+int qe_attention_prefill_segments(long blocks);
 int qe_attention_prefill_uncut_keys();
 size_t qe_attention_prefill_workspace(int num_tiles, int Hq, int Hkv, int D, int segments);
 
@@ -42,6 +44,13 @@ extern "C" int qe_attention_prefill_plan(int num_tiles, int Hq, int Hkv, int max
     return qe_attention_prefill_segment_keys((long)(num_tiles / 4) * Hkv * ((Hq / Hkv) / (32 / R)), max_keys);
 }
 
+// Into how many segments at most (1: not at all): for a caller that leaves their length to the device.
+extern "C" int qe_attention_prefill_plan_segments(int num_tiles, int Hq, int Hkv) {
+    if (num_tiles <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv) return 1;
+    const int R = qe_attention_prefill_tile_rows(Hq, Hkv);
+    return qe_attention_prefill_segments((long)(num_tiles / 4) * Hkv * ((Hq / Hkv) / (32 / R)));
+}
+
 // up to this many keys the plan is never to cut
 extern "C" int qe_attention_prefill_plan_uncut_keys() { return qe_attention_prefill_uncut_keys(); }
 
@@ -51,20 +60,29 @@ extern "C" long qe_attention_prefill_workspace_bytes(int num_tiles, int Hq, int 
     return (long)qe_attention_prefill_workspace(num_tiles, Hq, Hkv, D, (max_keys + seg_keys - 1) / seg_keys);
 }
 
+// ... and for a number of segments
+extern "C" long qe_attention_prefill_workspace_bytes_for(int num_tiles, int Hq, int Hkv, int D, int segments) {
+    if (segments <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv) return 0;
+    return (long)qe_attention_prefill_workspace(num_tiles, Hq, Hkv, D, segments);
+}
+
 // tiles: num_tiles pairs (first row of q, rows <= qe_attention_prefill_rows) of consecutive new
 // tokens of one request.  Takes what qe_attention_prefill_supported takes.  groups: wave groups
 // a block that share the key tiles between them, 1 or 2, or 0 to choose by the number of blocks.
 // seg_keys: 0, or the keys of a segment (a multiple of 64) into which the walks are cut; then no row
-// sees more than max_keys keys and the workspace has qe_attention_prefill_workspace_bytes bytes.
+// sees more than max_keys keys and the workspace has qe_attention_prefill_workspace_bytes bytes.  Or
+// minus a number of segments (2 to 8): the kernels take the keys that row keys_row of q sees (no row
+// sees more) from its position and cut them into that many segments, or fewer, themselves; the
+// workspace then has qe_attention_prefill_workspace_bytes_for that number.
 extern "C" int qe_attention_prefill_run(const void* q, void* out, const void* cache, const int* tiles,
                                         int num_tiles, const int* positions, const int* tok_seq,
                                         const int* block_table, int max_blocks, int Hq, int Hkv, int D, int P,
                                         float scale, int window, int groups, int seg_keys, int max_keys,
-                                        void* workspace, long workspace_bytes, hipStream_t stream) {
-    QE_REQUIRE(num_tiles >= 0 && Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && seg_keys >= 0 &&
-               workspace_bytes >= 0, "prefill attention: bad sizes");
+                                        int keys_row, void* workspace, long workspace_bytes, hipStream_t stream) {
+    QE_REQUIRE(num_tiles >= 0 && Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && workspace_bytes >= 0,
+               "prefill attention: bad sizes");
     return qe_attention_prefill(q, out, cache, tiles, num_tiles, positions, tok_seq, block_table, max_blocks,
-                                Hq, Hkv, D, P, scale, window, groups, seg_keys, max_keys, workspace,
+                                Hq, Hkv, D, P, scale, window, groups, seg_keys, max_keys, keys_row, workspace,
                                 (size_t)workspace_bytes, stream);
 }
 

@@ -66,7 +66,21 @@ __device__ __forceinline__ float sum_of_both_halves(float v) {
 }
 
 #define QE_PREFILL_UNCUT_KEYS 1024
+#define QE_PREFILL_MIN_SEGMENT 512
 #define VROW 48   // bytes of a staged value row: 16 keys = 32 bytes of data + 16 of padding
+
+// The keys of a segment when the host does not know the positions (a recorded step): seg_param < 0
+// asks for -seg_param segments of the keys that row keys_row sees, each a multiple of 64 and at least
+// QE_PREFILL_MIN_SEGMENT keys; up to QE_PREFILL_UNCUT_KEYS keys nothing is cut (0).  The same value
+// in every block of the two kernels.
+__device__ __forceinline__ int segment_keys(int seg_param, const int* __restrict__ positions, int keys_row) {
+    if (seg_param >= 0) return seg_param;
+    const int keys = positions[keys_row] + 1;
+    if (keys <= QE_PREFILL_UNCUT_KEYS) return 0;
+    const int ks = -seg_param;
+    const int seg = ((keys + ks - 1) / ks + 63) / 64 * 64;
+    return seg < QE_PREFILL_MIN_SEGMENT ? QE_PREFILL_MIN_SEGMENT : seg;
+}
 
 // A lane's share of its column's result: the accumulators' element 4 b + j of block db is feature
 // 32 db + 8 b + 4 g + j.
@@ -92,7 +106,8 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ tiles, const int* __restrict__ positions, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int max_blocks,
-    int Hq, int Hkv, int P, int log2P, float scale_log2, int window, int R, int seg_keys, float* __restrict__ part) {
+    int Hq, int Hkv, int P, int log2P, float scale_log2, int window, int R, int seg_param, int keys_row,
+    float* __restrict__ part) {
     constexpr int KROW = D * 2 + 16;                 // bytes of a staged key row
     constexpr int KBYTES = 32 * KROW, VBYTES = 2 * D * VROW, BUF = KBYTES + VBYTES;
     constexpr int KP = 32 * (D / 8) / 256;           // 16-byte key pieces per thread (2 for D = 128)
@@ -125,6 +140,8 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     int kmax = positions[bt4[2 * last]] + bt4[2 * last + 1];
     // key segments: this block walks the keys of segment bseg only
     bool partial = false;
+    const int seg_keys = segment_keys(seg_param, positions, keys_row);
+    if (seg_keys <= 0 && bseg > 0) return;                 // (asked for segments, but the keys are too few to cut)
     if (seg_keys > 0) {
         const int z = bseg, z_lo = kmin / seg_keys, z_hi = (kmax - 1) / seg_keys;
         if (z < z_lo || z > z_hi) return;                  // (the whole block: no barrier has been met yet)
@@ -401,7 +418,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
 template <int D>
 __global__ __launch_bounds__(256) void attention_prefill_merge_kernel(
     const float* __restrict__ part, bf16_t* __restrict__ out, const int* __restrict__ tiles,
-    const int* __restrict__ positions, int Hq, int Hkv, int window, int R, int seg_keys) {
+    const int* __restrict__ positions, int Hq, int Hkv, int window, int R, int seg_param, int keys_row) {
     constexpr int NV = 2 + (D / 32) * 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 5, r = lane & 31;
     const int G = Hq / Hkv, GH = 32 / R;
@@ -416,6 +433,8 @@ __global__ __launch_bounds__(256) void attention_prefill_merge_kernel(
     const int p_block = positions[row_first];
     const int kmin = (window > 0 && p_block - window + 1 > 0) ? p_block - window + 1 : 0;
     const int kmax = positions[bt4[2 * last]] + bt4[2 * last + 1];
+    const int seg_keys = segment_keys(seg_param, positions, keys_row);
+    if (seg_keys <= 0) return;                             // nothing was cut
     const int z_lo = kmin / seg_keys, z_hi = (kmax - 1) / seg_keys;
     if (z_hi <= z_lo) return;                              // the block wrote its result itself
     const int row0 = bt4[2 * wave], cnt = bt4[2 * wave + 1];
@@ -464,12 +483,17 @@ int qe_attention_prefill_tile_rows(int Hq, int Hkv) {
 // least 512 keys; up to QE_PREFILL_UNCUT_KEYS keys a walk is too short to be worth one.
 int qe_attention_prefill_uncut_keys() { return QE_PREFILL_UNCUT_KEYS; }
 
+int qe_attention_prefill_segments(long blocks) {
+    if (blocks <= 0 || blocks > 128) return 1;
+    const long ks = 256 / blocks;                          // as many blocks as there are compute units, not more
+    return ks > 8 ? 8 : (int)ks;
+}
+
 int qe_attention_prefill_segment_keys(long blocks, int max_keys) {
-    if (blocks <= 0 || blocks > 128 || max_keys <= QE_PREFILL_UNCUT_KEYS) return 0;
-    long ks = 256 / blocks;                                // as many blocks as there are compute units, not more
-    if (ks > 8) ks = 8;
-    int seg = (int)(((max_keys + ks - 1) / ks + 63) / 64 * 64);
-    if (seg < 512) seg = 512;
+    const int ks = qe_attention_prefill_segments(blocks);
+    if (ks <= 1 || max_keys <= QE_PREFILL_UNCUT_KEYS) return 0;
+    int seg = ((max_keys + ks - 1) / ks + 63) / 64 * 64;   // (segment_keys() computes the same on the device)
+    if (seg < QE_PREFILL_MIN_SEGMENT) seg = QE_PREFILL_MIN_SEGMENT;
     return seg >= max_keys ? 0 : seg;
 }
 
@@ -482,12 +506,15 @@ size_t qe_attention_prefill_workspace(int num_tiles, int Hq, int Hkv, int D, int
 // tiles: num_tiles pairs (first row of q, number of rows <= qe_attention_prefill_tile_rows), in
 // groups of four that belong to one request, in ascending rows, with consecutive positions
 // through the group; a group is filled up with pairs of 0 rows.  num_tiles is a multiple of 4.
-// seg_keys: 0, or the keys of a segment (a multiple of 64) with max_keys, the most keys a row sees,
-// and a workspace of qe_attention_prefill_workspace(..., segments = ceil(max_keys / seg_keys)) bytes.
+// seg_keys: 0; or the keys of a segment (a multiple of 64) with max_keys, the most keys a row sees; or,
+// for a caller that does not know the positions, minus the number of segments (at most 8) into which
+// the keys of row keys_row, which sees the most, are to be cut.  The workspace has
+// qe_attention_prefill_workspace(..., segments) bytes.
 int qe_attention_prefill(const void* q, void* out, const void* cache, const int* tiles, int num_tiles,
                          const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
                          int Hq, int Hkv, int D, int P, float scale, int window, int groups,
-                         int seg_keys, int max_keys, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                         int seg_keys, int max_keys, int keys_row, void* workspace, size_t workspace_bytes,
+                         hipStream_t stream) {
     QE_REQUIRE((D == 64 || D == 128) && P >= 16 && (P & (P - 1)) == 0 && Hq % Hkv == 0,
                "prefill attention: sizes not taken");
     int log2P = 0;
@@ -503,10 +530,14 @@ int qe_attention_prefill(const void* q, void* out, const void* cache, const int*
         segments = qe_cdiv(max_keys, seg_keys);
         QE_REQUIRE(segments <= 64, "prefill attention: %d segments", segments);
         if (segments <= 1) { seg_keys = 0; segments = 1; }
-        else
-            QE_REQUIRE(workspace && workspace_bytes >= qe_attention_prefill_workspace(num_tiles, Hq, Hkv, D, segments),
-                       "prefill attention: workspace of %zu bytes is too small", workspace_bytes);
+    } else if (seg_keys < 0) {
+        segments = -seg_keys;
+        QE_REQUIRE(segments <= 8 && keys_row >= 0, "prefill attention: %d segments of the keys of row %d", segments, keys_row);
+        if (segments == 1) seg_keys = 0;
     }
+    if (segments > 1)
+        QE_REQUIRE(workspace && workspace_bytes >= qe_attention_prefill_workspace(num_tiles, Hq, Hkv, D, segments),
+                   "prefill attention: workspace of %zu bytes is too small", workspace_bytes);
     QE_REQUIRE(num_tiles / 4 <= 65535, "prefill attention: %d tiles are too many for one launch", num_tiles);
     dim3 grid(Hkv * waves_per_kv, segments, num_tiles / 4);
     dim3 mgrid(Hkv * waves_per_kv, D / 32, num_tiles / 4);
@@ -518,17 +549,17 @@ int qe_attention_prefill(const void* q, void* out, const void* cache, const int*
 #define QE_PREFILL(D_, NG_)                                                                         \
     attention_prefill_kernel<D_, NG_><<<grid, 256 * NG_, 0, stream>>>(                              \
         (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, tiles, positions, tok_seq, block_table, \
-        max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R, seg_keys, (float*)workspace)
+        max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R, seg_keys, keys_row, (float*)workspace)
     if (D == 128) { if (groups == 2) QE_PREFILL(128, 2); else QE_PREFILL(128, 1); }
     else          { if (groups == 2) QE_PREFILL(64, 2); else QE_PREFILL(64, 1); }
 #undef QE_PREFILL
-    if (seg_keys > 0) {
+    if (seg_keys != 0) {
         if (D == 128)
             attention_prefill_merge_kernel<128><<<mgrid, 256, 0, stream>>>((const float*)workspace, (bf16_t*)out, tiles,
-                                                                           positions, Hq, Hkv, window, R, seg_keys);
+                                                                           positions, Hq, Hkv, window, R, seg_keys, keys_row);
         else
             attention_prefill_merge_kernel<64><<<mgrid, 256, 0, stream>>>((const float*)workspace, (bf16_t*)out, tiles,
-                                                                          positions, Hq, Hkv, window, R, seg_keys);
+                                                                          positions, Hq, Hkv, window, R, seg_keys, keys_row);
     }
     QE_LAUNCH_CHECK();
     return 0;

@@ -58,7 +58,9 @@ def load_library():
         "qe_attention_prefill_supported": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_rows": [i32, i32],
         "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, i32,
-                                     vp, i64, vp],
+                                     i32, vp, i64, vp],
+        "qe_attention_prefill_plan_segments": [i32, i32, i32],
+        "qe_attention_prefill_workspace_bytes_for": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_plan": [i32, i32, i32, i32],
         "qe_attention_prefill_plan_uncut_keys": [],
         "qe_attention_prefill_workspace_bytes": [i32, i32, i32, i32, i32, i32],
@@ -541,7 +543,8 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
               dec_tokens: Optional[torch.Tensor] = None, max_dec_position: int = 0,
               other_tokens: Optional[torch.Tensor] = None,
               other_tiles: Optional[torch.Tensor] = None, prefill_groups: int = 0,
-              max_other_keys: int = 0, prefill_segment_keys: int = -1) -> torch.Tensor:
+              max_other_keys: int = 0, prefill_segment_keys: int = -1,
+              other_keys_row: Optional[int] = None) -> torch.Tensor:
     """q [T, Hq, D]; cache [pages, 2, Hkv, P, D] (key tiles [P][D], value tiles transposed [D][P]);
     positions, tok_seq int32 [T]; block_table int32 [B, max_blocks].  Token t sees the keys at
     positions max(0, p - window + 1) .. p of request tok_seq[t] (window 0: all).  The caller
@@ -554,7 +557,9 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
     for the prefill kernel (prefill_groups: its wave groups a block, 1 or 2, 0 to let it choose).
     max_other_keys: no row of other_tiles sees more keys than this (its position + 1); when given,
     the prefill kernel may cut long walks of few blocks into segments of keys (prefill_segment_keys:
-    their length, a multiple of 64; 0 for none; -1 to let it choose).
+    their length, a multiple of 64; 0 for none; -1 to let it choose).  A caller that does not know
+    the positions (a recorded step) names the row of q that sees the most keys instead
+    (other_keys_row): the kernel then cuts by that row's position.
     Without the lists every row is treated alike."""
     lib = load_library()
     _need(q, "q", _ACT, (None, None, None))
@@ -600,7 +605,16 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
         if other_tiles is not None and algo != ALGO_GENERIC and attention_prefill_supported(q, cache):
             _need(other_tiles, "other_tiles", torch.int32, (None, 2), dev)
             n_tiles, max_keys, seg, ws, nbytes = other_tiles.shape[0], int(max_other_keys), 0, None, 0
-            if max_keys > 0:
+            keys_row = -1
+            if other_keys_row is not None:
+                if not 0 <= int(other_keys_row) < T or max_keys > 0:
+                    raise KernelError(f"attention: other_keys_row {other_keys_row} (of {T} rows) stands instead of max_other_keys")
+                ks = lib.qe_attention_prefill_plan_segments(n_tiles, Hq, Hkv) if prefill_segment_keys else 1
+                if ks > 1:
+                    seg, keys_row = -ks, int(other_keys_row)
+                    nbytes = lib.qe_attention_prefill_workspace_bytes_for(n_tiles, Hq, Hkv, D, ks)
+                    ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+            elif max_keys > 0:
                 seg = int(prefill_segment_keys)
                 if seg < 0:
                     seg = lib.qe_attention_prefill_plan(n_tiles, Hq, Hkv, max_keys)
@@ -615,7 +629,8 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
                                                 other_tiles.data_ptr(), n_tiles,
                                                 positions.data_ptr(), tok_seq.data_ptr(), block_table.data_ptr(),
                                                 max_blocks, Hq, Hkv, D, P, float(scale), int(window),
-                                                int(prefill_groups), seg, max_keys, _ptr(ws), nbytes, _stream()),
+                                                int(prefill_groups), seg, max_keys, keys_row, _ptr(ws), nbytes,
+                                                _stream()),
                    "attention (prefill)")
         else:
             generic(other_tokens)

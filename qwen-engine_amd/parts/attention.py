@@ -71,21 +71,18 @@ class PagedAttention:
                 "max_dec_position": key * ops.DECODE_SPLIT_KEYS - 1}
 
     @staticmethod
-    def portion_graph_key(tokens: int, keys: int) -> int:
-        """The prefill kernel cuts long walks into segments of keys by the most keys a row sees: a
-        recorded portion serves up to the next power of two of them."""
-        bound = ops.prefill_uncut_keys()                  # (up to here it cuts nothing: one recorded step for all)
-        while bound < keys:
-            bound *= 2
-        return bound
+    def portion_graph_key(tokens: int, keys: int) -> bool:
+        """Beyond a number of keys the prefill kernel cuts long walks into segments and a second kernel
+        merges them; how long a segment is the kernels take from the last row's position themselves."""
+        return keys > ops.prefill_uncut_keys()
 
     @staticmethod
-    def portion_graph_extras(tokens: int, device, key: int = 0) -> dict:
-        """For a recorded step that is one prompt portion of ``tokens`` rows whose last row sees at most
-        ``key`` keys: no single new tokens, all rows in order."""
+    def portion_graph_extras(tokens: int, device, key: bool = False) -> dict:
+        """For a recorded step that is one prompt portion of ``tokens`` rows: no single new tokens, all
+        rows in order; the last row sees the most keys."""
         return {"dec_tokens": torch.zeros(0, dtype=torch.int32, device=device),
                 "other_tokens": torch.arange(tokens, dtype=torch.int32, device=device), "max_dec_position": 0,
-                "max_other_keys": int(key)}
+                "max_other_keys": 0, "other_keys_row": tokens - 1 if key else None}
 
     def _extras(self, ctx) -> dict:
         return ctx.extras.get(PagedAttention) or {"dec_tokens": None, "other_tokens": None, "max_dec_position": 0,
@@ -234,7 +231,7 @@ class PagedAttention:
                           dec_tokens=ex["dec_tokens"], max_dec_position=ex["max_dec_position"],
                           other_tokens=ex["other_tokens"],
                           other_tiles=self._other_tiles(ctx) if ex["other_tokens"] is not None else None,
-                          max_other_keys=ex.get("max_other_keys", 0))
+                          max_other_keys=ex.get("max_other_keys", 0), other_keys_row=ex.get("other_keys_row"))
         return self._project_out(o.view(T, self.hq * self.d))
 
     def _project_out(self, o: torch.Tensor) -> torch.Tensor:

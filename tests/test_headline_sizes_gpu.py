@@ -182,3 +182,41 @@ def test_twenty_four_requests_decode_together_beyond_1024_keys(long_model, dtype
         for s in range(3):
             err = float((outs[s][i] - ref[s]).abs().max()) / float(ref.abs().max())
             assert err <= TOL[dtype], f"request {i} (prompt {n}), step {s}: error {err}"
+
+
+# ---- (c) portions of prompts deep in a context: the prefill kernel's key segments -------------------
+@pytest.mark.parametrize("use_graphs", [True, False])
+@pytest.mark.parametrize("heads", [(4, 2, 128), (8, 1, 64)])
+def test_portions_deep_in_a_context(heads, use_graphs):
+    """A prompt of some 4000 tokens in portions of 2 to 1500 tokens: from 1024 keys on, a portion of
+    few tiles has its keys cut into segments whose partial results a second kernel merges, and a
+    portion of a round length is replayed from a graph recorded for its bucket of keys.  The last
+    row of every portion against the plain implementation (src/layers/fused_ops/attn.py:243-420 is the
+    reference's attention over a paged cache, without such segments)."""
+    hq, hkv, d = heads
+    cfg_dict = dict(CFG_LONG, num_attention_heads=hq, num_key_value_heads=hkv, head_dim=d)
+    cfg, w, plain_w = make_weights(cfg_dict, 13, 0.06)
+    sizes = [1500, 512, 2, 256, 640, 17, 384, 128, 512, 77]
+    L = sum(sizes)
+    toks = tokens(L, cfg_dict["vocab_size"], 41)
+    ends = [sum(sizes[:i + 1]) for i in range(len(sizes))]
+    ref = P.forward_logits(cfg_dict, plain_w, toks, act_dtype=torch.bfloat16, rows=[e - 1 for e in ends])
+    model = DecoderModel(cfg.to_model_spec())
+    model.load(w, Runtime(torch.device("cuda:0"), torch.bfloat16))
+    runner = ModelRunner(model, page_size=16, num_pages=L // 16 + 3, max_requests=1, use_graphs=use_graphs,
+                         debug_poison=True)
+    runner.add_request("r")
+    got, a = [], 0
+    for n in sizes:
+        got.append(runner.step([StepEntry("r", toks[a:a + n], [n - 1])]))
+        a += n
+    got = torch.cat(got).float().cpu()
+    assert torch.isfinite(got).all()
+    err = (got - ref).abs().amax(dim=1) / float(ref.abs().max())
+    bad = torch.nonzero(err > TOL["bfloat16"])
+    assert bad.numel() == 0, f"first wrong portion ends at {ends[int(bad[0])]}, error {float(err[bad[0]])}"
+    if use_graphs:
+        # 512 (twice), 256, 640 and 384 tokens, all beyond the keys up to which nothing is cut; 128 tokens
+        # are too few to be recorded
+        assert runner.graph_steps == 5 and runner.graphs_recorded == 4
+    runner.cache.check_invariants()

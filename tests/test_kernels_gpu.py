@@ -849,9 +849,20 @@ def test_prefill_attention_over_key_segments(ops, hq, hkv, d, page, window):
         # rows whose keys lie in one segment come from the same sums as without segments
         if seg == 512 and groups == 2:
             assert torch.equal(out[300:630], whole[300:630])                 # the whole prompt of 330: keys 0 .. 329
+    # a caller that does not know the positions names the row that sees the most keys (row 299, at
+    # position 999): the kernels cut by its position, as the host would have
+    by_row = ops.attention(*args, window=window, dec_tokens=i32(dec), max_dec_position=90, other_tokens=i32(other),
+                           other_tiles=i32(tiles), other_keys_row=299)
+    by_host = ops.attention(*args, window=window, dec_tokens=i32(dec), max_dec_position=90, other_tokens=i32(other),
+                            other_tiles=i32(tiles), max_other_keys=1000)
+    close(by_row, torch.cat(want), bf)
+    assert torch.equal(by_row, by_host)
     with pytest.raises(ops.KernelError):
         ops.attention(*args, other_tokens=i32(other), dec_tokens=i32(dec), max_dec_position=90, other_tiles=i32(tiles),
                       max_other_keys=1000, prefill_segment_keys=100)
+    with pytest.raises(ops.KernelError):
+        ops.attention(*args, other_tokens=i32(other), dec_tokens=i32(dec), max_dec_position=90, other_tiles=i32(tiles),
+                      other_keys_row=len(pos))
 
 
 @pytest.mark.parametrize("M", [1, 8, 64, 65, 200, 1024])
