@@ -183,7 +183,8 @@ __device__ __forceinline__ void norm_rows_into_lds(const float* __restrict__ hs,
 // order of s (the fused residual-add + norm kernel does), so the sum has one fixed order.
 // NT: tiles of 16 rows of W a block owns.  Every wave reads the activations of its chunks itself
 // (M rows against the block's 16 NT rows of W), so with more than 16 rows of activations most of
-// what a block reads is activations, from the L2; two tiles a block halve that.
+// what a block reads is activations, from the L2; two tiles a block halve that, four quarter it
+// (8 rows against the logits' matrix: 4.15 TB/s of weights with one tile a block, 6.07 with one row).
 template <int MT, int NT, int EPI, typename TO, int WAVES, bool NORM>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     const void* __restrict__ x_in, const bf16_t* __restrict__ w, const float* __restrict__ bias,
@@ -341,7 +342,10 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
     // two tiles of outputs a block where the activations have more than 16 rows and there are blocks
     // enough all the same (with silu.mul a tile of outputs is two tiles of W already: only up to 32 rows)
     const bool two = mt >= 2 && (!SILU || mt <= 2) && (long)qe_cdiv(N, 32) * splits >= 256;
-    const dim3 grid(qe_cdiv(N, two ? 32 : 16), splits);
+    // ... and four where 2 to 16 rows meet a matrix of very many rows (the logits'): with 8 rows the
+    // activations are then an eighth of what a block reads instead of a third
+    const bool four = !SILU && mt == 1 && M > 1 && (long)qe_cdiv(N, 64) * splits >= 2048;
+    const dim3 grid(qe_cdiv(N, four ? 64 : (two ? 32 : 16)), splits);
 #define QE_SKINNY_W(MT_, NT_, WAVES_, NORM_)                                                           \
     do {                                                                                               \
         auto kern = gemm_skinny_kernel<MT_, NT_, EPI, TO, WAVES_, NORM_>;                              \
@@ -366,6 +370,8 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
         else QE_REQUIRE(false, "skinny gemm: the norm prologue goes with the store and silu-mul epilogues");
     } else if (mt == 1 && SILU) {
         if constexpr (SILU) QE_SKINNY_W(1, 1, 8, false);
+    } else if (four) {
+        if constexpr (!SILU) QE_SKINNY(1, 4);
     } else if (two) {
         switch (mt) {
             case 2: QE_SKINNY(2, 2); break;

@@ -919,15 +919,20 @@ def test_decode_kernel_with_more_than_32_splits(ops, L):
     close(out, want, bf)
 
 
-@pytest.mark.parametrize("M", [1, 8, 64])
+@pytest.mark.parametrize("M", [1, 2, 5, 8, 16, 64])
 def test_gemm_for_few_rows_against_the_whole_vocabulary(ops, M):
     """The head's product at the family's vocabulary: [M, 1024] against [151936, 1024], 32-bit logits,
-    compared in 64-bit on the first and last columns and on 3000 drawn ones."""
+    compared in 64-bit on the first and last columns and on 3000 drawn ones.  Up to 16 rows (one tile
+    of rows, whether a block owns one tile of outputs or four) a row's logits are the same bits
+    whatever else is in the batch."""
     bf = torch.bfloat16
     N, K = 151936, 1024
     x, w = rand(M, K, seed=520, dtype=bf), rand(N, K, seed=521, dtype=bf, scale=0.02)
     got = ops.gemm(x.to(DEV), w.to(DEV), out_dtype=torch.float32).cpu()
     assert got.shape == (M, N) and torch.isfinite(got).all()
+    if M <= 16:
+        alone = ops.gemm(x[M - 1:].to(DEV), w.to(DEV), out_dtype=torch.float32).cpu()
+        assert torch.equal(alone[0], got[M - 1])
     cols = torch.cat([torch.arange(0, 80), torch.arange(N - 120, N),
                       torch.randint(0, N, (3000,), generator=torch.Generator().manual_seed(522))])
     want = x.double() @ w[cols].double().t()
