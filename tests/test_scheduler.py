@@ -102,6 +102,51 @@ def test_prompts_are_cut_under_the_budget_and_mixed_with_decodes():
     assert all(sum(n for _, n, _ in step) <= 8 for step in log)
 
 
+def test_a_prompt_takes_the_whole_budget_while_nothing_decodes():
+    """The portion limit protects the requests that decode: an idle engine runs a long prompt in steps
+    of the whole budget, and goes back to the limit as soon as a request decodes beside it."""
+    sched, cache = make(num_pages=200, budget=32, chunk=8, max_model_len=400)
+    a = Request(0, list(range(3, 103)), SamplingParams(max_new_tokens=3))          # 100 tokens
+    sched.add(a)
+    log = []
+    drive(sched, cache, log)
+    assert [step for step in log[:4]] == [[(0, 32, False)], [(0, 32, False)], [(0, 32, False)], [(0, 4, True)]]
+    assert a.output == expected_output(a.prompt, 3)
+    # a short request decodes while a long prompt arrives: the long one goes in portions of the limit
+    sched, cache = make(num_pages=200, budget=32, chunk=8, max_model_len=400)
+    short = Request(1, [5, 6, 7], SamplingParams(max_new_tokens=20))
+    long = Request(2, list(range(3, 63)), SamplingParams(max_new_tokens=2))         # 60 tokens
+    sched.add(short)
+    log = []
+    planned = sched.plan()
+    assert [(p.request.req_id, len(p.tokens)) for p in planned] == [(1, 3)]
+    sampled = []
+    for p in planned:
+        cache.reserve(p.request.req_id, len(p.tokens)); cache.commit(p.request.req_id, p.tokens)
+        sampled.append(fake_next(p.request.known))
+    sched.update(planned, sampled)
+    sched.add(long)
+    drive(sched, cache, log)
+    portions = [n for step in log for rid, n, _ in step if rid == 2 and n > 1]
+    assert portions[:7] == [8] * 7 and portions[7] == 4            # while request 1 decodes beside it
+    assert short.output == expected_output(short.prompt, 20) and long.output == expected_output(long.prompt, 2)
+
+
+def test_a_first_portion_of_the_whole_budget_that_does_not_fit_is_made_smaller():
+    """12 pages of 4 tokens: a prompt of 40 tokens cannot take a first portion of the whole budget (64
+    tokens would be the limit, 40 tokens are 10 pages, and 5 pages are held by another request), but a
+    smaller one fits: it is admitted with that instead of waiting or failing."""
+    sched, cache = make(num_pages=12, page=4, budget=64, chunk=8, max_model_len=64, max_num_seqs=2)
+    cache.add_request("other")
+    cache.reserve("other", 20)
+    cache.commit("other", list(range(20)))
+    r = Request(0, list(range(3, 43)), SamplingParams(max_new_tokens=1))
+    sched.add(r)
+    planned = sched.plan()
+    assert [(p.request.req_id, len(p.tokens)) for p in planned] == [(0, 20)]       # 40 -> 20 tokens: 5 pages fit beside the 5
+    assert r.status != "failed"
+
+
 def test_admission_is_first_in_first_out_and_bounded():
     sched, cache = make(max_num_seqs=2)
     reqs = [Request(i, [7 + i] * 6, SamplingParams(max_new_tokens=3)) for i in range(5)]
