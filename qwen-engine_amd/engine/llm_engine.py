@@ -97,7 +97,7 @@ class LLMEngine:
         logits = self.runner.step(entries)
         sampling = [p.request for p in planned if p.sample]
         temps = [r.params.temperature for r in sampling]
-        us = [uniform_for(r.params.seed, r.req_id, len(r.output)) for r in sampling]
+        us = [uniform_for(r.params.seed, r.req_id, len(r.output)) if t > 0 else 0.0 for r, t in zip(sampling, temps)]
         tokens = self.sampler.sample(logits, temps, us)
         return self.scheduler.update(planned, tokens)
 

@@ -72,6 +72,16 @@ class Request:
     def num_known(self) -> int:
         return len(self.prompt) + len(self.output)
 
+    def known_span(self, start: int, n: int) -> List[int]:
+        """known[start:start + n] without joining the two lists when the span lies in one of them
+        (a decoding request's span is its last output token, every step)."""
+        lp = len(self.prompt)
+        if start >= lp:
+            return self.output[start - lp:start - lp + n]
+        if start + n <= lp:
+            return self.prompt[start:start + n]
+        return self.known[start:start + n]
+
 
 @dataclass
 class Planned:
@@ -202,7 +212,7 @@ class Scheduler:
                 if n == 0:
                     blocked = blocked or r
                     continue
-                toks = r.known[r.num_computed:r.num_computed + n]
+                toks = r.known_span(r.num_computed, n)
                 planned.append(Planned(r, toks, sample=(r.num_computed + n == r.num_known)))
                 budget -= n
             if blocked is not None:
@@ -247,7 +257,7 @@ class Scheduler:
                 self._admitted += 1
                 self.running.append(r)
                 self.stats["shared_prefix_tokens"] += start
-                planned.append(Planned(r, r.known[start:start + n], sample=(start + n == r.num_known)))
+                planned.append(Planned(r, r.known_span(start, n), sample=(start + n == r.num_known)))
                 budget -= n
             self.waiting.extendleft(reversed(held))            # back to the front, in their order
             if not planned and self.waiting and not self.running:
