@@ -88,6 +88,8 @@ def load_library():
     lib.qe_argmax_workspace_bytes.restype = ctypes.c_long
     lib.qe_attention_decode_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]
     lib.qe_attention_decode_workspace_bytes.restype = ctypes.c_long
+    lib.qe_attention_prefill_workspace_bytes.restype = ctypes.c_long
+    lib.qe_attention_prefill_workspace_bytes_for.restype = ctypes.c_long
     _lib = lib
     return lib
 
