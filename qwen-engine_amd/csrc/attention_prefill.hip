@@ -29,13 +29,14 @@
 // That halves the length of the longest block, which is what the time of a causal prompt hangs on
 // when there are no more blocks than compute units.  The longest blocks are started first.
 //
-// Key segments: with few blocks and many keys (a portion of a prompt far into its context; one
-// whole prompt, whose last rows see all of it) the keys are cut at absolute multiples of seg_keys
-// and block z of the grid's third dimension walks only the keys of segment z.  A block whose rows'
-// keys lie in one segment writes its result as before (the blocks of the other segments leave at
-// once); else the blocks of the segments that hold keys of its rows leave their maxima, sums and
-// accumulators, as the lanes hold them, in a workspace, and attention_prefill_merge_kernel, with the
-// same grid and the same lanes, weighs and adds them in the order of the segments.
+// Key segments: with fewer blocks than compute units and many keys (a portion of a prompt far into
+// its context) the keys are cut at absolute multiples of a segment length, and the blocks of the
+// grid's second dimension walk one segment each.  A block whose rows' keys lie in one segment writes
+// its result as before (the blocks of the other segments leave at once); else the blocks of the
+// segments that hold keys of its rows leave their maxima, sums and accumulators, as the lanes hold
+// them, in a workspace, and attention_prefill_merge_kernel, with the same lanes, weighs and adds them
+// in the order of the segments.  The segment length comes from the host, or, where the host does not
+// know the positions (a recorded step), from the position of the row that sees the most keys.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
