@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 
 H, V, HQ, HKV, D, I, PAGE = 128, 300, 8, 2, 64, 192, 16
 WINDOWS = (40, None, 17)            # per layer: two pages and a half; all keys; barely more than a page
-EPS, THETA, MAXPOS = 1e-6, 10000.0, 1024
+EPS, THETA, MAXPOS = 1e-6, 10000.0, 3072
 
 
 class ToyWindowConfig:
@@ -102,3 +102,35 @@ def test_window_layers_in_every_cutting(toy, tmp_path, dtype, cut):
     got = traces.collect(trace, out_dir, V)
     bad, worst = traces.first_mismatch(got, ref, 1e-4 if dtype == "float32" else 2e-2)
     assert bad is None, f"first wrong logits at (request, position, relative error) {bad}"
+
+
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_windows_far_into_a_context(toy, use_graphs):
+    """One request of 2600 tokens in portions of 1500, 512, 2, 256 and 330, then four decoded tokens:
+    beyond 1024 keys the prefill kernel cuts the keys of a portion into segments (all of them matter
+    in the layer over all keys; in the windowed layers a block's keys lie in one or two segments, and
+    the pages behind the window have been given back), and round portions are replayed from recorded
+    graphs.  The last row of every step against the plain implementation, pages poisoned."""
+    from qwen_engine_amd.engine import ModelRunner, StepEntry, load_model
+    model = load_model(toy, dtype="bfloat16")
+    _, w = P.read_folder(toy)
+    sizes = [1500, 512, 2, 256, 330, 1, 1, 1, 1]
+    L = sum(sizes)
+    toks = torch.randint(0, V, (L,), generator=torch.Generator().manual_seed(43)).tolist()
+    ref = plain_forward(w, toks, torch.bfloat16)
+    runner = ModelRunner(model, page_size=PAGE, num_pages=L // PAGE + 8, max_requests=1, use_graphs=use_graphs,
+                         debug_poison=True)
+    runner.add_request("r")
+    a = 0
+    for n in sizes:
+        got = runner.step([StepEntry("r", toks[a:a + n], [n - 1])])[0].float().cpu()
+        a += n
+        assert torch.isfinite(got).all(), f"the step that ends at {a}"
+        err = float((got - ref[a - 1]).abs().max()) / float(ref.abs().max())
+        assert err <= 2e-2, f"the step that ends at {a}: error {err}"
+    if use_graphs:
+        assert runner.graph_steps == 2 + 4                 # the portions of 512 and 256 tokens, and the decoded tokens
+    # the windowed groups hold what their windows need, not the whole context
+    held = sorted(sum(1 for p in t if p >= 0) for t in runner.cache.get("r").tables)
+    assert held[-1] == math.ceil(L / PAGE) and held[0] <= 3 and held[1] <= 4
+    runner.cache.check_invariants()
