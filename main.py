@@ -42,7 +42,7 @@ def parse_args(argv=None):
                     choices=["bfloat16", "float32"])
     ap.add_argument("--temperature", type=float, default=0.0, help="0: greedy")
     ap.add_argument("--max-step-tokens", type=int, default=2048, help="token budget of one step")
-    ap.add_argument("--prefill-chunk", type=int, default=512, help="largest portion of a prompt in a step")
+    ap.add_argument("--prefill-chunk", type=int, default=512, help="largest portion of a prompt in a step in which some request decodes (else the whole budget)")
     ap.add_argument("--ignore-eos", action="store_true")
     ap.add_argument("--no-prefix-sharing", action="store_true")
     ap.add_argument("--debug-poison", action="store_true",

@@ -15,7 +15,7 @@ class EngineConfig:
     max_num_seqs: int = 4            # requests that run at a time
     max_model_len: int = 256         # prompt + generated tokens of one request
     max_step_tokens: int = 2048      # token budget of one step
-    prefill_chunk: int = 512         # largest portion of one prompt in a step
+    prefill_chunk: int = 512         # largest portion of one prompt in a step in which some request decodes
     enable_prefix_sharing: bool = True
     keep_freed_prefixes: bool = True   # shared pages of finished requests stay until their memory is needed
     seed: int = 0
