@@ -73,7 +73,11 @@ class ModelRunner:
     # of some microseconds each, which the host cannot launch as fast as the device runs them.
     PORTION_GRAPH_MIN = 256
     PORTION_GRAPH_STEP = 128
-    MAX_GRAPHS = 32       # recorded graphs kept (each holds its own activations); the least recently used goes first
+    # Recorded graphs kept; the least recently used goes first.  Each holds its own activations and
+    # workspaces (tens of MB at the small model's sizes, more for long contexts).  A server whose batch
+    # and contexts wander passes through 15 row counts up to 64 rows times a bucket per 1024 keys, and
+    # recording a step again costs several replays of it.
+    MAX_GRAPHS = 96
 
     def __init__(self, model: DecoderModel, page_size: int, num_pages, max_requests: int,
                  prefix_sharing: bool = False, use_graphs: Optional[bool] = None,

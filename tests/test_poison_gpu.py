@@ -114,3 +114,31 @@ def test_prompt_portions_through_recorded_graphs(toy, use_graphs):
         err = float((row - refs[rid][pos]).abs().max()) / float(refs[rid].abs().max())
         assert err <= 2e-2, f"request {rid}, position {pos}: error {err}"
     runner.cache.check_invariants()
+
+
+def test_recorded_graphs_are_dropped_and_recorded_again(toy):
+    """A runner that keeps two graphs: decode steps of 1, 2 and 3 requests in turns drop the graph used
+    longest ago and record it again when its batch comes back; every step's logits stay right."""
+    model = load_model(toy, dtype="bfloat16")
+    _, w = P.read_folder(toy)
+    reqs = {i: _tokens(60 + 7 * i, 70 + i) for i in range(3)}
+    refs = {i: plain_forward(w, t, torch.bfloat16) for i, t in reqs.items()}
+    runner = ModelRunner(model, page_size=PAGE, num_pages=40, max_requests=3, debug_poison=True)
+    runner.MAX_GRAPHS = 2
+    done = {}
+    for i, t in reqs.items():
+        runner.add_request(i)
+        runner.step([StepEntry(i, t[:20], [])])
+        done[i] = 20
+    recorded_at = []
+    for live in (1, 2, 3, 1, 2, 3, 3, 1):
+        out = runner.step([StepEntry(i, [reqs[i][done[i]]], [0]) for i in range(live)]).float().cpu()
+        for i in range(live):
+            err = float((out[i] - refs[i][done[i]]).abs().max()) / float(refs[i].abs().max())
+            assert err <= 2e-2, f"{live} requests, request {i} at position {done[i]}: error {err}"
+            done[i] += 1
+        assert len(runner._graphs) <= 2
+        recorded_at.append(runner.graphs_recorded)
+    # 1, 2, 3 record; 1 again (dropped when 3 came), 2 again, 3 again; 3 is there; 1 again
+    assert recorded_at == [1, 2, 3, 4, 5, 6, 6, 7]
+    runner.cache.check_invariants()
