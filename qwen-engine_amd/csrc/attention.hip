@@ -29,6 +29,16 @@ int qe_attention_prefill_uncut_keys();
 size_t qe_attention_prefill_workspace(int num_tiles, int Hq, int Hkv, int D, int segments);
 
 int qe_attention_prefill_tile_rows(int Hq, int Hkv);
+int qe_attention_prefill_tiles(const int* portions, int n_portions, int rows_per_tile, int* tiles, int max_groups,
+                               hipStream_t stream);
+
+// The tile list for qe_attention_prefill_run from portions [n_portions][2] = (first row, rows) that lie
+// on the device: tiles [4 max_groups][2], whatever is beyond the portions' groups being groups of no
+// rows.  The caller guarantees that the portions have at most max_groups groups of 4 tiles.
+extern "C" int qe_attention_prefill_tiles_run(const int* portions, int n_portions, int rows_per_tile, int* tiles,
+                                              int max_groups, hipStream_t stream) {
+    return qe_attention_prefill_tiles(portions, n_portions, rows_per_tile, tiles, max_groups, stream);
+}
 
 // rows of a tile for these head counts
 extern "C" int qe_attention_prefill_rows(int Hq, int Hkv) {

@@ -132,6 +132,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
 
     // the block's four tiles belong to one request, in ascending rows; tiles of 0 rows pad the group
     const int* bt4 = tiles + 8 * (gridDim.z - 1 - bgroup);   // later rows see more keys: they start first
+    if (bt4[1] <= 0) return;                               // a group without rows (a list filled up to a fixed length)
     const int row_first = bt4[0];
     int last = 0;
 #pragma unroll
@@ -427,6 +428,7 @@ __global__ __launch_bounds__(256) void attention_prefill_merge_kernel(
     const int kvh = bhead / (G / GH);
     const int head = kvh * G + (bhead % (G / GH)) * GH + r / R;
     const int* bt4 = tiles + 8 * (gridDim.z - 1 - bgroup);
+    if (bt4[1] <= 0) return;
     const int row_first = bt4[0];
     int last = 0;
 #pragma unroll
@@ -467,6 +469,44 @@ __global__ __launch_bounds__(256) void attention_prefill_merge_kernel(
         for (int j = 0; j < 4; ++j) o[j] = (__bf16)(acc[4 * b + j] * inv);
         *(bf16x4*)(orow + 8 * b) = o;
     }
+}
+
+// The tile list of qe_attention_prefill from the step's portions, made on the device (a recorded step
+// does not know its portions' lengths on the host): portions [n_portions][2] = (first row, rows), each
+// cut into tiles of at most `rows_per_tile` rows in groups of four, a group filled up with tiles of no
+// rows; the list is filled up to max_groups groups with groups of no rows.  One thread per group.
+__global__ void prefill_tiles_kernel(const int* __restrict__ portions, int n_portions, int rows_per_tile,
+                                     int* __restrict__ tiles, int max_groups) {
+    const int grp = blockIdx.x * blockDim.x + threadIdx.x;
+    if (grp >= max_groups) return;
+    int first = 0, start = 0, rows = 0, in_portion = -1;   // which portion the group lies in, and the group's place in it
+    for (int i = 0; i < n_portions; ++i) {
+        const int n = portions[2 * i + 1];
+        const int groups = n > 0 ? (n + 4 * rows_per_tile - 1) / (4 * rows_per_tile) : 0;
+        if (in_portion < 0 && grp < first + groups) {
+            in_portion = grp - first;
+            start = portions[2 * i];
+            rows = n;
+        }
+        first += groups;
+    }
+    int* out = tiles + 8 * grp;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int r = in_portion < 0 ? rows : (4 * in_portion + j) * rows_per_tile;    // rows before this tile in its portion
+        const int cnt = in_portion < 0 || r >= rows ? 0 : min(rows_per_tile, rows - r);
+        out[2 * j] = cnt > 0 ? start + r : start;
+        out[2 * j + 1] = cnt;
+    }
+}
+
+int qe_attention_prefill_tiles(const int* portions, int n_portions, int rows_per_tile, int* tiles, int max_groups,
+                               hipStream_t stream) {
+    QE_REQUIRE(portions && tiles && n_portions >= 1 && n_portions <= 64 && rows_per_tile >= 1 && max_groups >= 1,
+               "prefill tiles: %d portions, tiles of %d rows, %d groups", n_portions, rows_per_tile, max_groups);
+    prefill_tiles_kernel<<<qe_cdiv(max_groups, 64), 64, 0, stream>>>(portions, n_portions, rows_per_tile, tiles, max_groups);
+    QE_LAUNCH_CHECK();
+    return 0;
 }
 
 // Rows per tile for a model's head counts: 32 / (heads that one wave serves).

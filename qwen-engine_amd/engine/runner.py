@@ -73,6 +73,13 @@ class ModelRunner:
     # of some microseconds each, which the host cannot launch as fast as the device runs them.
     PORTION_GRAPH_MIN = 256
     PORTION_GRAPH_STEP = 128
+    # A step of single new tokens beside exactly one prompt portion (what a server runs while requests
+    # keep arriving) is recorded too: the single tokens' rows are filled up as in a decode graph, the
+    # portion to a multiple of MIXED_GRAPH_STEP tokens with rows of the tables' spare row that write
+    # nowhere.  Run as it comes, such a step costs the host some 370 launches (3.7 ms at the small
+    # model's sizes, more than its kernels take).
+    MIXED_GRAPH_STEP = 128
+    MIXED_GRAPH_MAX_TOKENS = 2048
     # Recorded graphs kept; the least recently used goes first.  Each holds its own activations and
     # workspaces (tens of MB at the small model's sizes, more for long contexts).  A server whose batch
     # and contexts wander passes through 15 row counts up to 64 rows times a bucket per 1024 keys, and
@@ -156,11 +163,14 @@ class ModelRunner:
         # portions are recorded only if every part that wants something prepared can say what a
         # recorded portion needs (parts.base: portion_graph_extras)
         self._portion_graphs = all(hasattr(cls, "portion_graph_extras") for cls in self._step_classes)
+        # ... and mixed steps only if they can say the same for those, and no part keeps state of its own
+        self._mixed_graphs = all(hasattr(cls, "mixed_graph_extras") for cls in self._step_classes) and not has_state
         self._stage: Optional[torch.Tensor] = None     # pinned host buffer of a step's integer arrays
         self._stage_np = None
         self._stage_event = torch.cuda.Event()
         self.steps_run = 0
-        self.graph_steps = 0
+        self.graph_steps = 0                       # steps replayed from a recorded graph, and by what they were:
+        self.graph_steps_of = {"decode": 0, "portion": 0, "mixed": 0}
         self.graphs_recorded = 0
 
     @staticmethod
@@ -418,6 +428,8 @@ class ModelRunner:
         elif self.use_graphs and self._portion_graphs and len(entries) == 1 and len(entries[0].want) <= 1 and \
                 len(entries[0].tokens) >= self.PORTION_GRAPH_MIN and len(entries[0].tokens) % self.PORTION_GRAPH_STEP == 0:
             logits = self._portion_step_with_graph(entries[0])
+        elif self.use_graphs and self._mixed_graphs and self._is_mixed_step(entries):
+            logits = self._mixed_step_with_graph(entries)
         else:
             ctx = self.build_context(entries)
             self._clear_state_of_new_requests(ctx.seqs)
@@ -479,7 +491,155 @@ class ModelRunner:
         rec["event"].record()
         rec["graph"].replay()
         self.graph_steps += 1
+        self.graph_steps_of["decode"] += 1
         return rec["logits"][:n_live].clone()          # the graph's own output is overwritten by the next replay
+
+    # ---- single new tokens beside one prompt portion through a recorded graph -----------------
+    def _is_mixed_step(self, entries: Sequence[StepEntry]) -> bool:
+        """Single tokens that want their logits, and exactly one portion of 2 to MIXED_GRAPH_MAX_TOKENS
+        tokens that wants its last row's logits or none."""
+        portion = None
+        for e in entries:
+            n = len(e.tokens)
+            if n == 1:
+                if list(e.want) != [0]:
+                    return False
+            elif portion is not None or n < 2 or n > self.MIXED_GRAPH_MAX_TOKENS or list(e.want) not in ([], [n - 1]) \
+                    or -(-n // self.MIXED_GRAPH_STEP) * self.MIXED_GRAPH_STEP > self.model.spec.max_positions:
+                return False                              # (the stand-in batch stands at the positions 0 .. T - 1)
+            else:
+                portion = e
+        return portion is not None
+
+    def _mixed_step_with_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        # the single tokens first, the portion last; the logits go back into the entries' order
+        order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) > 1)
+        ordered = [entries[i] for i in order]
+        tokens = self._check_and_reserve(ordered)
+        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(ordered, tokens)
+        self._check_bounds(seqs, slots, upd_idx, upd_val)
+        self._poison_pages()
+        n_dec, n_groups, i32 = len(ordered) - 1, len(self.cache.groups), np.int32
+        T1 = len(ordered[-1].tokens)
+        B = self.graph_rows(n_dec)
+        T = -(-T1 // self.MIXED_GRAPH_STEP) * self.MIXED_GRAPH_STEP
+        fill, pad = B - n_dec, T - T1
+        spare = self.spare_row
+
+        def padded(x, fill_value, pad_values):
+            return np.concatenate([x[:n_dec], np.full(fill, fill_value, dtype=i32), pad_values, x[n_dec:]])
+
+        zeros_pad = np.zeros(pad, dtype=i32)
+        token_ids = padded(token_ids, 0, zeros_pad)
+        positions_all = padded(positions, 0, np.arange(pad, dtype=i32))
+        tok_seq = padded(tok_seq, spare, np.full(pad, spare, dtype=i32))
+        slots = [padded(x, -1, np.full(pad, -1, dtype=i32)) for x in slots]
+        cap = 2 * B + 2 * (T // self.page_size + 2)
+        if any(len(u) > cap for u in upd_idx):
+            for g in range(n_groups):
+                if len(upd_idx[g]):
+                    ops.scatter_int(self.tables[g], torch.from_numpy(upd_idx[g]).to(self.rt.device),
+                                    torch.from_numpy(upd_val[g]).to(self.rt.device))
+                upd_idx[g] = upd_val[g] = np.zeros(0, dtype=i32)
+        max_dec_position = int(positions[:n_dec].max()) if n_dec else 0
+        portion_keys = seqs[-1].kv_before + T1
+        part_keys = tuple(cls.mixed_graph_key(max_dec_position, portion_keys) for cls in self._step_classes)
+        key = ("mixed", B, T, part_keys)
+        rec = self._graphs.pop(key, None)
+        if rec is None:
+            while len(self._graphs) >= self.MAX_GRAPHS:
+                self._graphs.pop(next(iter(self._graphs)))
+            rec = self._record_mixed_graph(B, T, part_keys, cap)
+            self.graphs_recorded += 1
+        self._graphs[key] = rec
+        none, zero = rec["none"], rec["zero"]
+        parts = [token_ids, positions_all, tok_seq]
+        for g in range(n_groups):
+            pad_u = cap - len(upd_idx[g])
+            parts += [slots[g], upd_idx[g], none[:pad_u], upd_val[g], zero[:pad_u]]
+        for cls in self._step_classes:
+            parts.append(np.asarray(cls.mixed_graph_dynamic(B, pad, T), dtype=i32))
+        rec["event"].synchronize()
+        np.concatenate(parts, out=rec["host_np"])
+        rec["meta"].copy_(rec["host"], non_blocking=True)
+        rec["event"].record()
+        rec["graph"].replay()
+        self.graph_steps += 1
+        self.graph_steps_of["mixed"] += 1
+        # rows of the recorded logits: the B rows of the single tokens, then the portion's last row
+        picked = []
+        for i in range(len(entries)):
+            at = order.index(i)
+            if at < n_dec:
+                picked.append(at)
+            elif entries[i].want:
+                picked.append(B)
+        logits = rec["logits"]
+        if picked == list(range(n_dec)) + [B]:            # the usual order: no index has to travel
+            return torch.cat([logits[:n_dec], logits[B:B + 1]]) if n_dec < B else logits[:B + 1].clone()
+        if picked == list(range(n_dec)):
+            return logits[:n_dec].clone()
+        return logits[torch.tensor(picked, dtype=torch.long).to(self.rt.device)]
+
+    def _record_mixed_graph(self, B: int, T: int, part_keys: tuple, cap: int):
+        """Static buffers for a step of B single new tokens beside one prompt portion filled up to T
+        tokens, one run outside the graph, then the recording.  The stand-in batch: every single token
+        at position 0 of the tables' spare row, the portion at its positions 0 .. T - 1, writing nowhere."""
+        dev, n_groups = self.rt.device, len(self.cache.groups)
+        dyn_sizes = [int(cls.mixed_graph_dynamic_size) for cls in self._step_classes]
+        n = 3 * (B + T) + n_groups * (B + T + 2 * cap) + sum(dyn_sizes)
+        host = torch.zeros(n, dtype=torch.int32).pin_memory()
+        meta = torch.zeros(n, dtype=torch.int32, device=dev)
+        stand_in = [0] * (B + T) + [0] * B + list(range(T)) + [self.spare_row] * (B + T)
+        for g in range(n_groups):
+            stand_in += [-1] * (B + T) + [-1] * cap + [0] * cap
+        for cls in self._step_classes:
+            stand_in += [int(v) for v in cls.mixed_graph_dynamic(B, 0, T)]
+        meta.copy_(torch.tensor(stand_in, dtype=torch.int32))
+        off = 0
+
+        def take(k):
+            nonlocal off
+            t = meta[off:off + k]
+            off += k
+            return t
+
+        d_tok, d_pos, d_seq = take(B + T), take(B + T), take(B + T)
+        d_slots, d_upd = [], []
+        for g in range(n_groups):
+            d_slots.append(take(B + T))
+            d_upd.append((take(cap), take(cap)))
+        d_dyn = [take(k) for k in dyn_sizes]
+        d_rows = torch.tensor(list(range(B)) + [B + T - 1], dtype=torch.int32, device=dev)
+        d_state = torch.full((B + 1,), self.spare_row, dtype=torch.int32, device=dev)
+        seqs = [SeqInfo(None, i, 1, 0, self.spare_row, False) for i in range(B)] + \
+            [SeqInfo(None, B, T, 0, self.spare_row, False)]
+        ctx = StepContext(rt=self.rt, page_size=self.page_size, num_tokens=B + T, seqs=seqs, token_ids=d_tok,
+                          positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
+                          logit_rows=d_rows, state_slots=d_state, max_position=0,
+                          extras={cls: dict(cls.mixed_graph_extras(B, T, k, dev, dyn))
+                                  for cls, k, dyn in zip(self._step_classes, part_keys, d_dyn)})
+
+        def run():
+            for g in range(n_groups):
+                ops.scatter_int(self.tables[g], d_upd[g][0], d_upd[g][1])
+            return self.model.forward(ctx, self.bindings)
+
+        torch.cuda.synchronize()
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            run()
+        stream.synchronize()
+        ctx.memo.clear()                          # (what the parts made for the first run is made again inside the graph)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            logits = run()
+        torch.cuda.synchronize()
+        event = torch.cuda.Event()
+        event.record()
+        return {"graph": graph, "ctx": ctx, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits,
+                "event": event, "none": np.full(cap, -1, dtype=np.int32), "zero": np.zeros(cap, dtype=np.int32)}
 
     # ---- one prompt portion through a recorded graph ----------------------------------------
     def _portion_step_with_graph(self, entry: StepEntry) -> torch.Tensor:
@@ -518,6 +678,7 @@ class ModelRunner:
         rec["event"].record()
         rec["graph"].replay()
         self.graph_steps += 1
+        self.graph_steps_of["portion"] += 1
         return rec["logits"].clone()
 
     def _record_portion_graph(self, T: int, n_want: int, cap: int, part_keys: tuple):

@@ -60,6 +60,7 @@ def load_library():
         "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, i32,
                                      i32, vp, i64, vp],
         "qe_attention_prefill_plan_segments": [i32, i32, i32],
+        "qe_attention_prefill_tiles_run": [vp, i32, i32, vp, i32, vp],
         "qe_attention_prefill_workspace_bytes_for": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_plan": [i32, i32, i32, i32],
         "qe_attention_prefill_plan_uncut_keys": [],
@@ -531,6 +532,19 @@ def attention_prefill_supported(q: torch.Tensor, cache: torch.Tensor) -> bool:
 def prefill_tile_rows(num_heads: int, num_kv_heads: int) -> int:
     """Rows of a tile of the prefill attention kernel for these head counts (``other_tiles``)."""
     return load_library().qe_attention_prefill_rows(num_heads, num_kv_heads)
+
+
+def prefill_tiles_on_device(portions: torch.Tensor, rows_per_tile: int, max_groups: int) -> torch.Tensor:
+    """The ``other_tiles`` of attention() for portions int32 [n, 2] = (first row, rows) that lie on the
+    device (a recorded step does not know them on the host): int32 [4 * max_groups, 2], groups of no rows
+    beyond what the portions need.  The caller guarantees that the portions need at most max_groups
+    groups of four tiles (every portion: ceil(rows / (4 * rows_per_tile)))."""
+    lib = load_library()
+    _need(portions, "portions", torch.int32, (None, 2))
+    tiles = torch.empty((4 * int(max_groups), 2), dtype=torch.int32, device=portions.device)
+    _check(lib.qe_attention_prefill_tiles_run(portions.data_ptr(), portions.shape[0], int(rows_per_tile),
+                                              tiles.data_ptr(), int(max_groups), _stream()), "prefill tiles")
+    return tiles
 
 
 def prefill_uncut_keys() -> int:

@@ -84,6 +84,30 @@ class PagedAttention:
                 "other_tokens": torch.arange(tokens, dtype=torch.int32, device=device), "max_dec_position": 0,
                 "max_other_keys": 0, "other_keys_row": tokens - 1 if key else None}
 
+    # A recorded step of single new tokens beside one prompt portion (parts.base): the rows of the
+    # single tokens come first, then rows that fill the portion up to a round length (a portion of the
+    # tables' spare row that writes nowhere), then the portion, whose last row is the step's last.
+    mixed_graph_dynamic_size = 4
+
+    @staticmethod
+    def mixed_graph_key(max_dec_position: int, portion_keys: int):
+        return PagedAttention.graph_key(max_dec_position), portion_keys > ops.prefill_uncut_keys()
+
+    @staticmethod
+    def mixed_graph_dynamic(rows: int, pad: int, tokens: int) -> List[int]:
+        """What changes from replay to replay: the two portions (first row, rows) that the prefill
+        kernel's tiles are cut from, on the device."""
+        return [rows, pad, rows + pad, tokens - pad]
+
+    @staticmethod
+    def mixed_graph_extras(rows: int, tokens: int, key, device, dynamic: torch.Tensor) -> dict:
+        splits, cut = key
+        return {"dec_tokens": torch.arange(rows, dtype=torch.int32, device=device),
+                "other_tokens": torch.arange(rows, rows + tokens, dtype=torch.int32, device=device),
+                "max_dec_position": splits * ops.DECODE_SPLIT_KEYS - 1, "max_other_keys": 0,
+                "other_keys_row": rows + tokens - 1 if cut else None,
+                "portions": dynamic.view(2, 2), "portion_rows": int(tokens)}
+
     def _extras(self, ctx) -> dict:
         return ctx.extras.get(PagedAttention) or {"dec_tokens": None, "other_tokens": None, "max_dec_position": 0,
                                                   "max_other_keys": 0}
@@ -95,6 +119,12 @@ class PagedAttention:
         if rows_per_tile <= 0:
             return None
         key = ("paged_attention.tiles", rows_per_tile)
+        ex = self._extras(ctx)
+        if key not in ctx.memo and ex.get("portions") is not None:
+            # a recorded step: the portions' lengths are known on the device only
+            portions = ex["portions"]
+            groups = -(-ex["portion_rows"] // (4 * rows_per_tile)) + portions.shape[0]
+            ctx.memo[key] = ops.prefill_tiles_on_device(portions, rows_per_tile, groups)
         if key not in ctx.memo:
             flat = prefill_tiles([(s.q_start, s.q_len) for s in ctx.seqs if s.q_len > 1], rows_per_tile)
             ctx.memo[key] = torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(ctx.rt.device) if flat else None

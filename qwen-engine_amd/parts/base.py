@@ -44,6 +44,16 @@ knows none of it.  A part class may define (all optional, all static):
                                  only for the same key, which portion_graph_extras gets as its third
                                  argument.  Without it nothing of the part's launches may depend on
                                  the portion's positions.
+  mixed_graph_key(max_position, keys), mixed_graph_extras(rows, tokens, key, device, dynamic),
+  mixed_graph_dynamic(rows, pad, tokens) with mixed_graph_dynamic_size
+                                 the same for a recorded step of ``rows`` single new tokens (the step's
+                                 first rows; max_position: their largest position) beside one prompt
+                                 portion filled up to ``tokens`` rows: ``pad`` rows of the tables' spare
+                                 row, which write nowhere, then the portion, whose last row (seeing
+                                 ``keys`` keys) is the step's last.  What differs from replay to replay
+                                 the part computes on the host as mixed_graph_dynamic_size integers
+                                 (mixed_graph_dynamic) and finds on the device as ``dynamic`` (int32).
+                                 Without these hooks such steps of a model with this part run as they come.
 """
 from __future__ import annotations
 

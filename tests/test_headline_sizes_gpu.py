@@ -127,7 +127,8 @@ def test_the_small_model_widths_with_the_whole_vocabulary(headline, dtype):
     if dtype == "bfloat16":
         # every decode step went through a recorded graph, and so did the two portions of 512 tokens
         # that want at most one row of logits
-        assert runner.graph_steps == 3 + 2 + 2 + 2
+        assert runner.graph_steps_of["decode"] == 3 + 2 + 2 and runner.graph_steps_of["portion"] == 2
+        assert runner.graph_steps_of["mixed"] == 63           # the other requests' prompts, each filled up to a round length
     runner.cache.check_invariants()
 
 
@@ -161,7 +162,7 @@ def test_decoding_across_the_positions_where_the_graph_changes(long_model, dtype
     bad = torch.nonzero(err > TOL[dtype])
     assert bad.numel() == 0, f"first wrong position {decoded[int(bad[0])]}, error {float(err[bad[0]])}"
     if dtype == "bfloat16":
-        assert runner.graph_steps == len(decoded) and runner.graphs_recorded >= 4
+        assert runner.graph_steps_of["decode"] == len(decoded) and runner.graphs_recorded >= 4
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -216,7 +217,7 @@ def test_portions_deep_in_a_context(heads, use_graphs):
     bad = torch.nonzero(err > TOL["bfloat16"])
     assert bad.numel() == 0, f"first wrong portion ends at {ends[int(bad[0])]}, error {float(err[bad[0]])}"
     if use_graphs:
-        # 512 (twice), 256, 640 and 384 tokens, all beyond the keys up to which nothing is cut; 128 tokens
-        # are too few to be recorded
-        assert runner.graph_steps == 5 and runner.graphs_recorded == 4
+        # 512 (twice), 256, 640 and 384 tokens, all beyond the keys up to which nothing is cut; the other
+        # portions are filled up to 1536 and (four of them) to 128 rows and replayed as well
+        assert runner.graph_steps_of == {"decode": 0, "portion": 5, "mixed": 5} and runner.graphs_recorded == 4 + 2
     runner.cache.check_invariants()

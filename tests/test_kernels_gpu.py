@@ -765,6 +765,22 @@ def test_prefill_attention_kernel(ops, hq, hkv, d, page, window):
         close(out, torch.cat(want), bf)
 
 
+@pytest.mark.parametrize("rows_per_tile", [16, 32, 4])
+def test_prefill_tiles_made_on_the_device(ops, rows_per_tile):
+    """The tile list cut from portions that lie on the device equals the list made on the host, filled up
+    with groups of no rows; a portion of no rows gives none."""
+    from qwen_engine_amd.parts.attention import prefill_tiles
+    for portions in ([(0, 75)], [(3, 0), (3, 500)], [(8, 37), (45, 91)], [(0, 1), (1, 2), (3, 300)], [(16, 127), (143, 385)]):
+        want = prefill_tiles([p for p in portions if p[1] > 0], rows_per_tile)
+        groups = len(want) // 8
+        dev = torch.tensor(portions, dtype=torch.int32, device=DEV)
+        got = ops.prefill_tiles_on_device(dev, rows_per_tile, groups + 2).cpu()
+        assert got.shape == (4 * (groups + 2), 2)
+        assert got[:4 * groups].flatten().tolist() == want
+        assert got[4 * groups:, 1].tolist() == [0] * 8                       # groups of no rows
+        assert int(got[:, 0].min()) >= 0 and int(got[:, 0].max()) < portions[-1][0] + max(portions[-1][1], 1)
+
+
 @pytest.mark.parametrize("key_pos", [0, 15, 16, 200, 255, 256, 299])
 def test_prefill_kernel_one_far_key_decides(ops, key_pos):
     """Rows 256..299 of a request; the row at position 299 (and every row at or after the key)

@@ -73,7 +73,7 @@ def test_twenty_requests_decode_past_the_window(toy, use_graphs):
         assert runner.cache.get(i).tables[0][0] == -1 or runner.cache.groups[0].window is None
     outs = [runner.step([StepEntry(i, [reqs[i][lengths[i] + s]], [0]) for i in range(20)]).float().cpu()
             for s in range(6)]
-    assert (runner.graph_steps == 6) == use_graphs
+    assert (runner.graph_steps_of["decode"] == 6) == use_graphs
     assert all(torch.isfinite(o).all() for o in outs)
     for i in (0, 7, 19):
         ref = plain_forward(w, reqs[i], torch.bfloat16)
@@ -126,10 +126,12 @@ def test_recorded_graphs_are_dropped_and_recorded_again(toy):
     runner = ModelRunner(model, page_size=PAGE, num_pages=40, max_requests=3, debug_poison=True)
     runner.MAX_GRAPHS = 2
     done = {}
+    runner.use_graphs = False                      # (the prompts as they come: this test counts the decode steps' graphs)
     for i, t in reqs.items():
         runner.add_request(i)
         runner.step([StepEntry(i, t[:20], [])])
         done[i] = 20
+    runner.use_graphs = True
     recorded_at = []
     for live in (1, 2, 3, 1, 2, 3, 3, 1):
         out = runner.step([StepEntry(i, [reqs[i][done[i]]], [0]) for i in range(live)]).float().cpu()
@@ -141,4 +143,64 @@ def test_recorded_graphs_are_dropped_and_recorded_again(toy):
         recorded_at.append(runner.graphs_recorded)
     # 1, 2, 3 record; 1 again (dropped when 3 came), 2 again, 3 again; 3 is there; 1 again
     assert recorded_at == [1, 2, 3, 4, 5, 6, 6, 7]
+    runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_single_tokens_beside_one_portion_through_recorded_graphs(toy, use_graphs):
+    """What a server runs while requests keep arriving: some requests decode, and beside them one new
+    request brings its prompt in portions of any length.  Such steps are recorded with the portion
+    filled up to a round length by rows that write nowhere, and replayed; the portion stands anywhere
+    among the entries, wants its last row or nothing, and the windows give pages back meanwhile.
+    Every wanted row against the plain implementation."""
+    model = load_model(toy, dtype="bfloat16")
+    _, w = P.read_folder(toy)
+    reqs = {"a": _tokens(90, 81), "b": _tokens(75, 82), "c": _tokens(303, 83), "d": _tokens(260, 84)}
+    refs = {k: plain_forward(w, t, torch.bfloat16) for k, t in reqs.items()}
+    runner = ModelRunner(model, page_size=PAGE, num_pages=120, max_requests=4, use_graphs=use_graphs, debug_poison=True)
+    done = {}
+
+    def check(entries, out):
+        row = 0
+        for e in entries:
+            for wpos in e.want:
+                pos = done[e.req_id] + wpos
+                got = out[row].float().cpu()
+                assert torch.isfinite(got).all(), f"request {e.req_id} at {pos}"
+                err = float((got - refs[e.req_id][pos]).abs().max()) / float(refs[e.req_id].abs().max())
+                assert err <= 2e-2, f"request {e.req_id} at position {pos}: error {err}"
+                row += 1
+        assert row == out.shape[0]
+        for e in entries:
+            done[e.req_id] += len(e.tokens)
+
+    def entry(rid, n, want_last=True):
+        lo = done[rid]
+        return StepEntry(rid, reqs[rid][lo:lo + n], [n - 1] if want_last else [])
+
+    for rid in ("a", "b"):                             # two requests that will decode: their prompts alone
+        runner.add_request(rid)
+        done[rid] = 0
+        e = [entry(rid, 40)]
+        check(e, runner.step(e))
+    runner.add_request("c")
+    done["c"] = 0
+    # the portion first, in the middle, last; with and without its last row; of 2 to 150 tokens
+    plan = [(["c", "a", "b"], 150, False), (["a", "c", "b"], 2, True), (["a", "b", "c"], 100, True),
+            (["a", "c"], 17, False), (["c", "b", "a"], 31, True)]
+    for order, n, want_last in plan:
+        e = [entry(r, n, want_last) if r == "c" else entry(r, 1) for r in order]
+        check(e, runner.step(e))
+    # a fourth request arrives while three decode: its whole prompt of 260 tokens beside them
+    runner.add_request("d")
+    done["d"] = 0
+    e = [entry("a", 1), entry("b", 1), entry("c", 1), entry("d", 259, True)]
+    check(e, runner.step(e))
+    e = [entry(r, 1) for r in ("d", "c", "b", "a")]
+    check(e, runner.step(e))
+    if use_graphs:
+        # the two prompts alone (filled up to 128 rows), the six mixed steps; the last step decodes
+        assert runner.graph_steps_of == {"decode": 1, "portion": 0, "mixed": 2 + 6}
+    else:
+        assert runner.graph_steps == 0
     runner.cache.check_invariants()
