@@ -146,6 +146,8 @@ class ModelRunner:
         for t in self.tables:
             t[max_requests].zero_()            # (every entry: the stand-in of a recorded prompt portion reads them all)
         self.spare_row = max_requests
+        # positions that a row standing on the spare row may have: inside every group's table row, and the model's
+        self._spare_positions = min([w * page_size for w in self.table_width] + [model.spec.max_positions])
         # a part with per-request state is recorded into graphs only if it says that it can be
         # (``graph_safe = True`` on the class); any other part unless it says that it cannot
         stateful_ok = all(self.plan.entry_state[i] is None or
@@ -505,9 +507,9 @@ class ModelRunner:
                 if list(e.want) != [0]:
                     return False
             elif portion is not None or n < 2 or n > self.MIXED_GRAPH_MAX_TOKENS or list(e.want) not in ([], [n - 1]) \
-                    or -(-n // self.MIXED_GRAPH_STEP) * self.MIXED_GRAPH_STEP > self.model.spec.max_positions:
-                return False                              # (the stand-in batch stands at the positions 0 .. T - 1)
-            else:
+                    or -(-n // self.MIXED_GRAPH_STEP) * self.MIXED_GRAPH_STEP > self._spare_positions:
+                return False                              # (the rows that fill up, and the stand-in batch, stand at the
+            else:                                         # positions 0 .. T - 1 of the spare table row)
                 portion = e
         return portion is not None
 

@@ -204,3 +204,21 @@ def test_single_tokens_beside_one_portion_through_recorded_graphs(toy, use_graph
     else:
         assert runner.graph_steps == 0
     runner.cache.check_invariants()
+
+
+def test_a_portion_is_not_filled_up_beyond_the_table_row(toy):
+    """A pool of 7 pages: the group that keeps all keys has table rows of 7 entries (112 positions), and
+    the rows that would fill a portion up to 128 would stand at positions beyond them.  Such a step
+    runs as it comes; with 8 pages it is recorded."""
+    model = load_model(toy, dtype="bfloat16")
+    _, w = P.read_folder(toy)
+    toks = _tokens(60, 91)
+    ref = plain_forward(w, toks, torch.bfloat16)
+    for pages, recorded in ((7, 0), (8, 2)):
+        runner = ModelRunner(model, page_size=PAGE, num_pages=pages, max_requests=1, debug_poison=True)
+        runner.add_request("r")
+        a = runner.step([StepEntry("r", toks[:50], [49])])[0].float().cpu()
+        b = runner.step([StepEntry("r", toks[50:59], [8])])[0].float().cpu()
+        for got, pos in ((a, 49), (b, 58)):
+            assert float((got - ref[pos]).abs().max()) <= 2e-2 * float(ref.abs().max())
+        assert runner.graph_steps_of["mixed"] == recorded
