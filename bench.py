@@ -26,6 +26,10 @@ Other sizes and workloads (not what the default line reports):
   --workload shared-prefix  N requests (default 32) that share a 1024-token prefix, each with 1024 tokens
                             of its own and 512 new tokens; the prefix's pages are shared
   --prefill-portion N       the prefill in portions of N tokens, one step each, instead of one step
+  --workload arrivals       N requests (default 160) with prompts uniform in [128, 512] and 128 new tokens that
+                            arrive one every --arrive-every steps (default 8: some 16 alive at a time), so that
+                            most steps are single new tokens beside one prompt portion
+  --eager-mixed-steps       all three: run such steps as they come instead of replaying a recorded graph
   --warmup-passes N         both: untimed passes over the workload with other tokens before the timed
                             one (default 1: the decode graphs are recorded there, as in a server that
                             has run for a while; 0 times the recording too)
@@ -74,7 +78,10 @@ def parse():
     ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--model", default="0.6b", choices=sorted(SIZES), help="whose layer sizes")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "shared-prefix"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "shared-prefix", "arrivals"])
+    ap.add_argument("--arrive-every", type=int, default=8, help="arrivals: a request arrives every this many steps")
+    ap.add_argument("--eager-mixed-steps", action="store_true",
+                    help="run steps of single new tokens beside a prompt portion as they come, not from a recorded graph")
     ap.add_argument("--requests", type=int, default=None, help="requests of the serving workloads")
     ap.add_argument("--warmup-passes", type=int, default=1,
                     help="serving workloads: untimed passes before the timed one (they record the decode graphs)")
@@ -88,10 +95,15 @@ def serving_run(args, cfg, model, layers, full_layers) -> int:
     from qwen_engine_amd.engine.llm_engine import LLMEngine
 
     V = cfg.vocab_size
+    arrive_every = 0
     if args.workload == "serving":
         n = args.requests or 64
         new_tokens, sharing = 256, False
         what = f"{n} requests, prompts uniform in [128, 2048], {new_tokens} new tokens each, portions of 512"
+    elif args.workload == "arrivals":
+        n = args.requests or 160
+        new_tokens, sharing, arrive_every = 128, False, max(1, args.arrive_every)
+        what = f"{n} requests, one every {arrive_every} steps, prompts uniform in [128, 512], {new_tokens} new tokens each"
     else:
         n = args.requests or 32
         new_tokens, sharing = 512, True
@@ -102,34 +114,52 @@ def serving_run(args, cfg, model, layers, full_layers) -> int:
         if args.workload == "serving":
             lens = torch.randint(128, 2049, (n,), generator=g).tolist()
             return [torch.randint(0, V, (k,), generator=g).tolist() for k in lens]
+        if args.workload == "arrivals":
+            # (the same lengths in every pass, other tokens: a server that has run for a while has met
+            # the shapes of its steps before)
+            lens = torch.randint(128, 513, (n,), generator=torch.Generator().manual_seed(args.seed + 2)).tolist()
+            return [torch.randint(0, V, (k,), generator=g).tolist() for k in lens]
         prefix = torch.randint(0, V, (1024,), generator=g).tolist()
         return [prefix + torch.randint(0, V, (1024,), generator=g).tolist() for _ in range(n)]
 
     prompts = make_prompts(args.seed + 2)
-    longest = 2048 + new_tokens
+    longest = (512 if arrive_every else 2048) + new_tokens
     P = args.block_size
-    pages = n * ((longest + P - 1) // P + 1)
+    live = min(n, 64) if arrive_every else n
+    pages = live * ((longest + P - 1) // P + 1)
     ecfg = EngineConfig(dtype="bfloat16" if args.dtype == "bf16" else "float32", block_size=P, num_blocks=pages,
-                        max_num_seqs=n, max_model_len=longest, max_step_tokens=2048, prefill_chunk=512,
+                        max_num_seqs=live, max_model_len=longest, max_step_tokens=2048, prefill_chunk=512,
                         enable_prefix_sharing=sharing, seed=args.seed)
     engine = LLMEngine(model, None, ecfg)
-    # Untimed passes over the same workload with other tokens: a server records its decode graphs
+    if args.eager_mixed_steps:
+        engine.runner._mixed_graphs = False
+
+    def run_all(ps):
+        """All at once, or one request every arrive_every steps; returns the steps."""
+        steps, nxt, last = 0, 0, time.perf_counter()
+        if not arrive_every:
+            engine.submit(ps, max_new_tokens=new_tokens, ignore_eos=True)
+            nxt = len(ps)
+        while nxt < len(ps) or engine.scheduler.has_work():
+            if nxt < len(ps) and steps % arrive_every == 0:
+                engine.submit([ps[nxt]], max_new_tokens=new_tokens, ignore_eos=True)
+                nxt += 1
+            engine.step()
+            steps += 1
+            if time.perf_counter() - last > 30:
+                last = time.perf_counter()
+                print(f"[bench] {steps} steps, {engine.stats()}", file=sys.stderr, flush=True)
+        return steps
+
+    # Untimed passes over the same workload with other tokens: a server records its graphs
     # once and runs for long, so the timed pass should find them recorded.
     for i in range(args.warmup_passes):
-        engine.submit(make_prompts(args.seed + 100 + i), max_new_tokens=new_tokens, ignore_eos=True)
+        run_all(make_prompts(args.seed + 100 + i))
         engine.run()
     before = engine.stats()
-    engine.submit(prompts, max_new_tokens=new_tokens, ignore_eos=True)
     torch.cuda.synchronize()
     t = time.perf_counter()
-    steps = 0
-    last = t
-    while engine.scheduler.has_work():
-        engine.step()
-        steps += 1
-        if time.perf_counter() - last > 30:
-            last = time.perf_counter()
-            print(f"[bench] {steps} steps, {engine.stats()}", file=sys.stderr, flush=True)
+    steps = run_all(prompts)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t
     stats = engine.stats()
