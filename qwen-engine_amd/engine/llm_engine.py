@@ -136,6 +136,8 @@ class LLMEngine:
         d["free_pages"] = [p.num_free for p in self.runner.cache.pools]
         d["kept_pages"] = self.runner.cache.num_kept
         d["graph_steps"] = self.runner.graph_steps
+        for kind, n in self.runner.graph_steps_of.items():
+            d[f"graph_steps_{kind}"] = n
         d["graphs_recorded"] = self.runner.graphs_recorded
         return d
 
