@@ -262,3 +262,37 @@ def test_temperature_draw_is_the_inverse_cdf_of_the_softmax():
     u = P.uniform_number(5, 2, 9)
     assert 0.0 <= u < 1.0 and u * (1 << 24) == int(u * (1 << 24)) and u == P.uniform_number(5, 2, 9)
     assert len({P.uniform_number(5, 2, k) for k in range(50)}) == 50
+
+
+# ---- the layer skeleton, by weights that give the logits a closed form -----------------------------
+import skeleton
+
+
+@pytest.mark.parametrize("name", sorted(skeleton.CASES))
+def test_skeleton_by_closed_forms(tmp_path, name):
+    """Where the residual is taken, where the norms stand, the final norm, the one eps and the scores'
+    divisor (model.py:278-298,345-359,177-178; config.py:46), each by a model whose logits are known
+    without running the plain implementation; and each expectation is far from what the mistake it
+    guards against would give."""
+    cfg, w, ids, want, mistakes = skeleton.build(name, tmp_path)
+    got = P.forward_logits(cfg, w, ids)
+    assert skeleton.relative_error(got, want) < 2e-5
+    for what, other in mistakes.items():
+        assert skeleton.relative_error(other, want) > 1e-2, what
+
+
+def test_skeleton_cases_tell_the_mistakes_apart(tmp_path):
+    """The closed forms are not blind: a block that keeps the normed rows as its stream, a model without
+    its final norm and a norm on the residual all miss them by far."""
+    cfg, w, ids, want, _ = skeleton.build("stream_passes_untouched", tmp_path)
+    E = w["model.embed_tokens.weight"][torch.tensor(ids)]
+    no_final_norm = E @ w["model.embed_tokens.weight"].t()
+    assert skeleton.relative_error(no_final_norm, want) > 1e-2
+    normed_stream = E
+    for i in range(cfg["num_hidden_layers"]):                       # x = norm(x) kept as the stream
+        normed_stream = P.rms_norm(normed_stream, w[f"model.layers.{i}.input_layernorm.weight"], cfg["rms_norm_eps"])
+        normed_stream = P.rms_norm(normed_stream, w[f"model.layers.{i}.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+    wrong = P.linear(P.rms_norm(normed_stream, w["model.norm.weight"], cfg["rms_norm_eps"]), w["model.embed_tokens.weight"])
+    assert skeleton.relative_error(wrong, want) > 1e-2
+    cfg, w, ids, want, _ = skeleton.build("first_norm_stands_on_the_branch", tmp_path)
+    assert skeleton.relative_error(torch.zeros_like(want), want) > 0.5   # a zeroed stream gives zero logits
