@@ -115,9 +115,9 @@ def serving_run(args, cfg, model, layers, full_layers) -> int:
             lens = torch.randint(128, 2049, (n,), generator=g).tolist()
             return [torch.randint(0, V, (k,), generator=g).tolist() for k in lens]
         if args.workload == "arrivals":
-            # (the same lengths in every pass, other tokens: a server that has run for a while has met
-            # the shapes of its steps before)
-            lens = torch.randint(128, 513, (n,), generator=torch.Generator().manual_seed(args.seed + 2)).tolist()
+            # (other lengths and other tokens in every pass: the timed pass meets shapes of steps that the
+            # passes before it did not, as a server does; the line reports how many steps were replayed)
+            lens = torch.randint(128, 513, (n,), generator=g).tolist()
             return [torch.randint(0, V, (k,), generator=g).tolist() for k in lens]
         prefix = torch.randint(0, V, (1024,), generator=g).tolist()
         return [prefix + torch.randint(0, V, (1024,), generator=g).tolist() for _ in range(n)]
@@ -129,19 +129,17 @@ def serving_run(args, cfg, model, layers, full_layers) -> int:
     pages = live * ((longest + P - 1) // P + 1)
     ecfg = EngineConfig(dtype="bfloat16" if args.dtype == "bf16" else "float32", block_size=P, num_blocks=pages,
                         max_num_seqs=live, max_model_len=longest, max_step_tokens=2048, prefill_chunk=512,
-                        enable_prefix_sharing=sharing, seed=args.seed)
+                        enable_prefix_sharing=sharing, seed=args.seed, record_mixed_steps=not args.eager_mixed_steps)
     engine = LLMEngine(model, None, ecfg)
-    if args.eager_mixed_steps:
-        engine.runner._mixed_graphs = False
 
-    def run_all(ps):
-        """All at once, or one request every arrive_every steps; returns the steps."""
+    def run_all(ps, phase=0):
+        """All at once, or one request every arrive_every steps (the first after ``phase`` steps); returns the steps."""
         steps, nxt, last = 0, 0, time.perf_counter()
         if not arrive_every:
             engine.submit(ps, max_new_tokens=new_tokens, ignore_eos=True)
             nxt = len(ps)
         while nxt < len(ps) or engine.scheduler.has_work():
-            if nxt < len(ps) and steps % arrive_every == 0:
+            if nxt < len(ps) and (steps + phase) % arrive_every == 0:
                 engine.submit([ps[nxt]], max_new_tokens=new_tokens, ignore_eos=True)
                 nxt += 1
             engine.step()
@@ -154,7 +152,7 @@ def serving_run(args, cfg, model, layers, full_layers) -> int:
     # Untimed passes over the same workload with other tokens: a server records its graphs
     # once and runs for long, so the timed pass should find them recorded.
     for i in range(args.warmup_passes):
-        run_all(make_prompts(args.seed + 100 + i))
+        run_all(make_prompts(args.seed + 100 + i), phase=i + 1)
         engine.run()
     before = engine.stats()
     torch.cuda.synchronize()
@@ -183,6 +181,10 @@ def serving_run(args, cfg, model, layers, full_layers) -> int:
         "warmup_unit": "passes over the workload with other tokens",
         "scheduler": {k: v - before.get(k, 0) for k, v in stats.items() if isinstance(v, (int, float))},
     }
+    # how many of the timed steps were replayed from a recorded graph (the others ran as they came: shapes
+    # not met often enough yet, or of a kind that is not recorded)
+    line["graph_hit_rate"] = round(line["scheduler"].get("graph_steps", 0) / max(1, steps), 4)
+    line["scheduler"]["graph_bytes"] = stats.get("graph_bytes", 0)
     print(json.dumps(line), flush=True)
     return 0
 
@@ -222,7 +224,10 @@ def main() -> int:
     H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     Hq, Hkv, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     layer_params = (Hq + 2 * Hkv) * D * H + Hq * D * H + 3 * H * I
-    weight_bytes = (layers * layer_params + V * H) * itemsize + (layers * (2 * H + 2 * D) + H) * 4
+    # every weight a step uses once, as the model counts its own tensors; for this architecture that is
+    # the layers' matrices and the head in the element type, and the norms' weights in 32-bit
+    weight_bytes = model.weight_bytes_read_per_step()
+    assert weight_bytes == (layers * layer_params + V * H) * itemsize + (layers * (2 * H + 2 * D) + H) * 4, weight_bytes
     kv_bytes_per_token = layers * 2 * Hkv * D * itemsize
     g = torch.Generator().manual_seed(args.seed + 1)
 
@@ -246,8 +251,8 @@ def main() -> int:
         tokens = torch.randint(0, V, (batch,), generator=g).tolist()
 
         def one_step(tokens):
-            logits = runner.step([StepEntry(r, [tokens[i]], [0]) for i, r in enumerate(ids)])
-            return ops.argmax(logits).tolist()          # the host needs the tokens to go on: a sync per step
+            # greedy: the recorded step picks the tokens itself; the host needs them to go on (a sync per step)
+            return runner.step([StepEntry(r, [tokens[i]], [0]) for i, r in enumerate(ids)], greedy=True)
 
         for _ in range(warmup):
             tokens = one_step(tokens)
@@ -276,8 +281,9 @@ def main() -> int:
             t = time.perf_counter()
             for a in range(0, T, portion):
                 part = toks[a:a + portion]
-                logits = runner.step([StepEntry("p", part, [len(part) - 1] if a + portion >= T else [])])
-            ops.argmax(logits).tolist()
+                last = a + portion >= T
+                first_token = runner.step([StepEntry("p", part, [len(part) - 1] if last else [])], greedy=last)
+            assert len(first_token) == 1
             torch.cuda.synchronize()
             dt = time.perf_counter() - t
             runner.free_request("p")
@@ -337,7 +343,8 @@ def main() -> int:
             **({"prefill_portion": args.prefill_portion} if args.prefill_portion else {}),
         },
         "prefill": {"value": round(prefill["value"], 1), "tokens": prefill["tokens"],
-                    "ms": round(prefill["ms"], 3), "frac": round(prefill["frac"], 4)},
+                    "ms": round(prefill["ms"], 3), "frac": round(prefill["frac"], 4),
+                    "timing": "best of 3 repetitions (the decode figures are means over their steps)"},
         "roofline": {"bound": "hbm", "achieved": round(main_run["gbs"], 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(main_run["gbs"] / HBM_PEAK_GBS, 4)},
         "points": points,

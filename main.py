@@ -38,6 +38,9 @@ def parse_args(argv=None):
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--num-blocks", type=int, default=None,
                     help="cache pages; default max_num_seqs * ceil(max_model_len / block_size)")
+    ap.add_argument("--gpu-memory-fraction", type=float, default=None,
+                    help="without --num-blocks: size the cache from this fraction of the device memory that is "
+                         "free once the weights are loaded")
     ap.add_argument("--model-dtype", "--dtype", dest="model_dtype", default="bfloat16",
                     choices=["bfloat16", "float32"])
     ap.add_argument("--temperature", type=float, default=0.0, help="0: greedy")
@@ -69,7 +72,7 @@ def main(argv=None) -> int:
         max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len,
         max_step_tokens=args.max_step_tokens, prefill_chunk=args.prefill_chunk,
         enable_prefix_sharing=not args.no_prefix_sharing, seed=args.seed,
-        debug_poison=args.debug_poison)
+        debug_poison=args.debug_poison, gpu_memory_fraction=args.gpu_memory_fraction)
     engine = LLMEngine.from_folder(args.model_name_or_path, engine_config)
 
     prompts = list(args.prompt) + [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]

@@ -70,17 +70,22 @@ __device__ __forceinline__ float sum_of_both_halves(float v) {
 #define QE_PREFILL_MIN_SEGMENT 512
 #define VROW 48   // bytes of a staged value row: 16 keys = 32 bytes of data + 16 of padding
 
+// The keys of a segment when ``keys`` keys are cut into ks segments: a multiple of 64, at least
+// QE_PREFILL_MIN_SEGMENT; 0 (no cut) up to QE_PREFILL_UNCUT_KEYS keys.  One formula for the host's plan
+// and for the kernels of a recorded step, which cut by a position they read on the device.
+__host__ __device__ __forceinline__ int prefill_segment_length(int keys, int ks) {
+    if (keys <= QE_PREFILL_UNCUT_KEYS || ks <= 1) return 0;
+    const int seg = ((keys + ks - 1) / ks + 63) / 64 * 64;
+    return seg < QE_PREFILL_MIN_SEGMENT ? QE_PREFILL_MIN_SEGMENT : seg;
+}
+
 // The keys of a segment when the host does not know the positions (a recorded step): seg_param < 0
 // asks for -seg_param segments of the keys that row keys_row sees, each a multiple of 64 and at least
 // QE_PREFILL_MIN_SEGMENT keys; up to QE_PREFILL_UNCUT_KEYS keys nothing is cut (0).  The same value
 // in every block of the two kernels.
 __device__ __forceinline__ int segment_keys(int seg_param, const int* __restrict__ positions, int keys_row) {
     if (seg_param >= 0) return seg_param;
-    const int keys = positions[keys_row] + 1;
-    if (keys <= QE_PREFILL_UNCUT_KEYS) return 0;
-    const int ks = -seg_param;
-    const int seg = ((keys + ks - 1) / ks + 63) / 64 * 64;
-    return seg < QE_PREFILL_MIN_SEGMENT ? QE_PREFILL_MIN_SEGMENT : seg;
+    return prefill_segment_length(positions[keys_row] + 1, -seg_param);
 }
 
 // A lane's share of its column's result: the accumulators' element 4 b + j of block db is feature
@@ -525,16 +530,15 @@ int qe_attention_prefill_tile_rows(int Hq, int Hkv) {
 int qe_attention_prefill_uncut_keys() { return QE_PREFILL_UNCUT_KEYS; }
 
 int qe_attention_prefill_segments(long blocks) {
-    if (blocks <= 0 || blocks > 128) return 1;
-    const long ks = 256 / blocks;                          // as many blocks as there are compute units, not more
+    const int units = qe_compute_units();
+    if (blocks <= 0 || blocks > units / 2) return 1;
+    const long ks = units / blocks;                        // as many blocks as there are compute units, not more
     return ks > 8 ? 8 : (int)ks;
 }
 
 int qe_attention_prefill_segment_keys(long blocks, int max_keys) {
     const int ks = qe_attention_prefill_segments(blocks);
-    if (ks <= 1 || max_keys <= QE_PREFILL_UNCUT_KEYS) return 0;
-    int seg = ((max_keys + ks - 1) / ks + 63) / 64 * 64;   // (segment_keys() computes the same on the device)
-    if (seg < QE_PREFILL_MIN_SEGMENT) seg = QE_PREFILL_MIN_SEGMENT;
+    const int seg = prefill_segment_length(max_keys, ks);
     return seg >= max_keys ? 0 : seg;
 }
 
@@ -585,7 +589,7 @@ int qe_attention_prefill(const void* q, void* out, const void* cache, const int*
     const float scale_log2 = scale * 1.4426950408889634f;
     // two groups a block where the blocks do not fill the compute units twice anyway
     // (groups: 0 = choose, 1 or 2)
-    if (groups == 0) groups = (long)grid.x * grid.z <= 256 ? 2 : 1;
+    if (groups == 0) groups = (long)grid.x * grid.z <= qe_compute_units() ? 2 : 1;
     QE_REQUIRE(groups == 1 || groups == 2, "prefill attention: %d groups a block", groups);
 #define QE_PREFILL(D_, NG_)                                                                         \
     attention_prefill_kernel<D_, NG_><<<grid, 256 * NG_, 0, stream>>>(                              \

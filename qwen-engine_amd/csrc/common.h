@@ -160,6 +160,7 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
 // the kernels do not take; qe_last_error() then holds the reason.
 extern "C" const char* qe_last_error();
 void qe_set_error(const char* fmt, ...);
+extern "C" int qe_compute_units();
 
 #define QE_REQUIRE(cond, ...)                         \
     do {                                              \

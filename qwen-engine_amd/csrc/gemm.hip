@@ -32,6 +32,20 @@ extern "C" int qe_gemm_norm_supported(int M, int N, int K, int dt_w) {
             !((long)N * K >= (16L << 20) && M > 16)) ? 1 : 0;
 }
 
+// Rows up to which a product may take the norm before it as its prologue at all.
+extern "C" int qe_gemm_norm_max_rows() { return 16; }
+
+// 1 if a product of M rows of the stream against w [N, K] should take the residual sum of n_delta partial
+// products and the norm as its prologue rather than leave them to the norm's own kernel.  Beside what
+// qe_gemm_norm_supported asks: a matrix of at most 8 M elements (a larger product is bound by the stream of
+// its weights, which stands still while the prologue runs: at the 8B sizes a decode step of one request took
+// 7 % longer with the prologue), and at most 192 KB of rows and partial products (every block reads all of
+// them for all rows; beyond that the norm's kernel, which reads them once, is quicker).
+extern "C" int qe_gemm_norm_preferred(int M, int N, int K, int dt_w, int n_delta) {
+    return (qe_gemm_norm_supported(M, N, K, dt_w) && (long)N * K <= (8L << 20) &&
+            (long)M * K * 4 * (1 + n_delta) <= 192L * 1024) ? 1 : 0;
+}
+
 // 1 if epilogue 4 (silu-mul over interleaved gate|up rows) can be used: N counts the outputs
 extern "C" int qe_gemm_silu_supported(int M, int N, int K, int dt_a, int dt_w) {
     return (N % 32 == 0 && (qe_gemm_skinny_ok(M, N, K, dt_a, dt_w) || qe_gemm_mfma_ok(M, 2 * N, K, dt_a, dt_w))) ? 1 : 0;
@@ -70,8 +84,12 @@ extern "C" int qe_gemm_partial_splits(int M, int N, int K) {
 // trips of its K loop): two to four cuts give every unit blocks to overlap (2048 x 1024 x 3072
 // with the norm behind it: 27.7 us in two cuts against 30.8; 512 rows: 15.7 against 24.7).
 extern "C" int qe_gemm_branch_splits(int M, int N, int K, int dt_a, int dt_w) {
-    if (qe_gemm_skinny_ok(M, N, K, dt_a, dt_w) || (M <= 64 && tiled_for_few_rows(M, N, K, dt_a, dt_w)))
-        return qe_gemm_partial_splits(M, N, K);
+    if (qe_gemm_skinny_ok(M, N, K, dt_a, dt_w) || (M <= 64 && tiled_for_few_rows(M, N, K, dt_a, dt_w))) {
+        const int s = qe_gemm_partial_splits(M, N, K);
+        // (rows few enough for the next product to add the parts up in its prologue: every block of that
+        // product reads all of them for all rows, so at most four)
+        return (M <= qe_gemm_norm_max_rows() && s > 4) ? 4 : s;
+    }
     if (!qe_gemm_mfma_ok(M, N, K, dt_a, dt_w) || K < 2048) return 0;
     const long tiles = (long)qe_cdiv(M, 64) * qe_cdiv(N, 128);
     if (tiles > 256) return 0;

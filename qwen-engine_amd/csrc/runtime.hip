@@ -14,7 +14,18 @@ void qe_set_error(const char* fmt, ...) {
 
 extern "C" const char* qe_last_error() { return g_error; }
 
-extern "C" int qe_abi_version() { return 1; }
+// Compute units of the current device (asked once per device; 256, an MI355X's, if the runtime does not say).
+extern "C" int qe_compute_units() {
+    static int units[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (units[dev] == 0) {
+        hipDeviceProp_t prop;
+        units[dev] = (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+                         ? prop.multiProcessorCount : 256;
+    }
+    return units[dev];
+}
 
 // The float32 mode's attention and matrix products run on the matrix units (attention_f32.hip,
 // gemm_f32.hip) unless this is switched off: then on the vector units' kernels, which sum in another

@@ -40,9 +40,20 @@ class LLMEngine:
         self.model = model
         self.tokenizer = tokenizer
         cfg = self.config
-        self.runner = ModelRunner(model, page_size=cfg.block_size, num_pages=cfg.pages_per_group(),
+        if cfg.num_blocks is None and cfg.gpu_memory_fraction is not None:
+            import torch
+            from ..parts.model import cache_plan
+            plan = cache_plan(model.spec)
+            itemsize = 2 if cfg.dtype == "bfloat16" else 4
+            per_page = max(1, plan.bytes_per_token(itemsize) * cfg.block_size)   # (every group gets the same number of pages)
+            pages = cfg.pages_per_group(torch.cuda.mem_get_info(model.rt.device)[0], per_page)
+        else:
+            pages = cfg.pages_per_group()
+        self.runner = ModelRunner(model, page_size=cfg.block_size, num_pages=pages,
                                   max_requests=cfg.max_num_seqs, prefix_sharing=cfg.enable_prefix_sharing,
-                                  keep_freed_prefixes=cfg.keep_freed_prefixes, debug_poison=cfg.debug_poison)
+                                  keep_freed_prefixes=cfg.keep_freed_prefixes, debug_poison=cfg.debug_poison,
+                                  record_mixed_steps=cfg.record_mixed_steps, graph_record_after=cfg.graph_record_after,
+                                  graph_memory_bytes=cfg.graph_memory_bytes)
         max_len = min(cfg.max_model_len, model.spec.max_positions)
         self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs, max_len, cfg.max_step_tokens,
                                    cfg.prefill_chunk, model.spec.eos_token_ids)
@@ -94,11 +105,16 @@ class LLMEngine:
             return []
         entries = [StepEntry(p.request.req_id, p.tokens, [len(p.tokens) - 1] if p.sample else [])
                    for p in planned]
-        logits = self.runner.step(entries)
         sampling = [p.request for p in planned if p.sample]
         temps = [r.params.temperature for r in sampling]
-        us = [uniform_for(r.params.seed, r.req_id, len(r.output)) if t > 0 else 0.0 for r, t in zip(sampling, temps)]
-        tokens = self.sampler.sample(logits, temps, us)
+        if all(t <= 0 for t in temps):
+            # every row is greedy: the step picks the tokens itself (inside its graph, where it is a
+            # recorded one), and no logits are copied or read again
+            tokens = self.runner.step(entries, greedy=True)
+        else:
+            logits = self.runner.step(entries)
+            us = [uniform_for(r.params.seed, r.req_id, len(r.output)) if t > 0 else 0.0 for r, t in zip(sampling, temps)]
+            tokens = self.sampler.sample(logits, temps, us)
         return self.scheduler.update(planned, tokens)
 
     def run(self) -> List[GenerationResult]:
@@ -139,6 +155,8 @@ class LLMEngine:
         for kind, n in self.runner.graph_steps_of.items():
             d[f"graph_steps_{kind}"] = n
         d["graphs_recorded"] = self.runner.graphs_recorded
+        d["graph_misses"] = self.runner.graph_misses      # steps of a recordable shape that ran as they came
+        d["graph_bytes"] = self.runner.graph_bytes()
         return d
 
 

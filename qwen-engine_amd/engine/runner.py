@@ -81,14 +81,17 @@ class ModelRunner:
     MIXED_GRAPH_STEP = 128
     MIXED_GRAPH_MAX_TOKENS = 2048
     # Recorded graphs kept; the least recently used goes first.  Each holds its own activations and
-    # workspaces (tens of MB at the small model's sizes, more for long contexts).  A server whose batch
+    # workspaces (tens of MB at the small model's sizes, a GB for a long portion at the large models'),
+    # so they are bounded by their bytes too (graph_memory_bytes).  A server whose batch
     # and contexts wander passes through 15 row counts up to 64 rows times a bucket per 1024 keys, and
     # recording a step again costs several replays of it.
     MAX_GRAPHS = 96
 
     def __init__(self, model: DecoderModel, page_size: int, num_pages, max_requests: int,
                  prefix_sharing: bool = False, use_graphs: Optional[bool] = None,
-                 keep_freed_prefixes: bool = False, debug_poison: bool = False):
+                 keep_freed_prefixes: bool = False, debug_poison: bool = False,
+                 record_mixed_steps: bool = True, graph_record_after: int = 1,
+                 graph_memory_bytes: int = 8 << 30):
         if model.rt is None:
             raise RuntimeError("the model has no weights yet")
         self.model = model
@@ -96,7 +99,7 @@ class ModelRunner:
         self.page_size = int(page_size)
         self.max_requests = int(max_requests)
         self.plan: CachePlan = cache_plan(model.spec)
-        has_state = any(s is not None for s in self.plan.entry_state)
+        has_state = any(s is not None for s in self.plan.user_state)
         self.cache = CacheManager(self.plan.groups or [], num_pages, page_size, max_requests,
                                   prefix_sharing=prefix_sharing and not has_state,
                                   keep_freed_prefixes=keep_freed_prefixes) \
@@ -109,28 +112,32 @@ class ModelRunner:
         self.cache.track_pages = self.debug_poison
         self.pages_poisoned = 0
         self.kv: List[Optional[torch.Tensor]] = []
-        for i, need in enumerate(self.plan.entry_kv):
+        for u, need in enumerate(self.plan.user_kv):         # (per cache user of the schedule, see CachePlan)
             if need is None:
                 self.kv.append(None)
                 continue
-            pages = self.cache.pools[self.plan.entry_group[i]].num_pages
+            pages = self.cache.pools[self.plan.user_group[u]].num_pages
             self.kv.append(torch.full((pages, 2, need.num_kv_heads, page_size, need.head_dim),
                                       float("nan") if self.debug_poison else 0.0, dtype=dt, device=dev))
         self.state: List[Optional[torch.Tensor]] = []
-        for need in self.plan.entry_state:
+        for need in self.plan.user_state:
             if need is None:
                 self.state.append(None)
             else:
                 # (one slot more than requests: the spare one belongs to the rows that fill a graph up)
                 self.state.append(torch.zeros((max_requests + 1, *need.shape), dtype=torch_dtype(need.dtype), device=dev))
+        # per schedule entry: one binding per cache user of its block, in the block's order
         self.bindings = []
-        for i in range(len(model.spec.schedule)):
-            src = self.plan.entry_source[i]
-            self.bindings.append(CacheBinding(
-                kv=self.kv[src] if src is not None else None,
-                group=self.plan.entry_group[i],
-                write=(src == i),
-                state=self.state[i]))
+        for users in self.plan.entry_users:
+            row = []
+            for u in users:
+                src = self.plan.user_source[u]
+                row.append(CacheBinding(
+                    kv=self.kv[src] if src is not None else None,
+                    group=self.plan.user_group[u],
+                    write=(src == u),
+                    state=self.state[u]))
+            self.bindings.append(row)
         # device copies of the block tables: [state slots, pages a request can hold]
         per_request = (model.spec.max_positions + page_size - 1) // page_size
         # (a table is indexed by position // page size: with a window the indices go on growing
@@ -150,9 +157,9 @@ class ModelRunner:
         self._spare_positions = min([w * page_size for w in self.table_width] + [model.spec.max_positions])
         # a part with per-request state is recorded into graphs only if it says that it can be
         # (``graph_safe = True`` on the class); any other part unless it says that it cannot
-        stateful_ok = all(self.plan.entry_state[i] is None or
-                          getattr(model.blocks[e.layer].mixer, "graph_safe", False) is True
-                          for i, e in enumerate(model.spec.schedule))
+        stateful_ok = all(all(self.plan.user_state[u] is None for u in users) or
+                          getattr(model.blocks[e.layer], "graph_safe_with_state", False) is True
+                          for users, e in zip(self.plan.entry_users, model.spec.schedule))
         graph_safe = stateful_ok and getattr(model, "graph_safe", True)
         self.use_graphs = (dt == torch.bfloat16 and graph_safe) if use_graphs is None else bool(use_graphs)
         # the part classes that want something prepared for every step (parts.base: step_extras)
@@ -166,7 +173,16 @@ class ModelRunner:
         # recorded portion needs (parts.base: portion_graph_extras)
         self._portion_graphs = all(hasattr(cls, "portion_graph_extras") for cls in self._step_classes)
         # ... and mixed steps only if they can say the same for those, and no part keeps state of its own
-        self._mixed_graphs = all(hasattr(cls, "mixed_graph_extras") for cls in self._step_classes) and not has_state
+        self._mixed_graphs = (all(hasattr(cls, "mixed_graph_extras") for cls in self._step_classes) and not has_state
+                              and bool(record_mixed_steps))
+        # A step of prompt tokens (a portion, or a portion beside single tokens) is recorded only when its
+        # shape has been met this many times: recording costs two runs of the step, a capture and three
+        # waits for the device, which a shape that never comes back does not earn.  Decode steps are
+        # recorded at once (their shapes are few and come back every step).
+        self.graph_record_after = max(1, int(graph_record_after))
+        self.graph_memory_bytes = int(graph_memory_bytes)
+        self._graph_seen = {}
+        self.graph_misses = 0                      # steps of a shape that is recorded, run as they came because it was not yet
         self._stage: Optional[torch.Tensor] = None     # pinned host buffer of a step's integer arrays
         self._stage_np = None
         self._stage_event = torch.cuda.Event()
@@ -183,6 +199,33 @@ class ModelRunner:
             return n
         step = 8 if n <= 64 else 32
         return -(-n // step) * step
+
+    def _graph_for(self, key, kind: str, record):
+        """The recorded step for ``key`` (most recently used last), recorded now by ``record()`` if its
+        shape has been met often enough, or None: the step then runs as it comes."""
+        rec = self._graphs.pop(key, None)
+        if rec is None:
+            if kind != "decode":
+                seen = self._graph_seen.get(key, 0) + 1
+                if seen < self.graph_record_after:
+                    if len(self._graph_seen) >= 4096:          # (shapes that never came back)
+                        self._graph_seen.clear()
+                    self._graph_seen[key] = seen
+                    self.graph_misses += 1
+                    return None
+                self._graph_seen.pop(key, None)
+            before = torch.cuda.memory_allocated(self.rt.device)
+            rec = record()
+            rec["bytes"] = max(0, torch.cuda.memory_allocated(self.rt.device) - before)
+            self.graphs_recorded += 1
+        self._graphs[key] = rec                                # dicts keep insertion order: the oldest use comes first
+        while len(self._graphs) > 1 and (len(self._graphs) > self.MAX_GRAPHS or self.graph_bytes() > self.graph_memory_bytes):
+            self._graphs.pop(next(iter(self._graphs)))
+        return rec
+
+    def graph_bytes(self) -> int:
+        """Device memory that the recorded steps hold (their buffers, activations and workspaces)."""
+        return sum(r["bytes"] for r in self._graphs.values())
 
     # ---- requests ------------------------------------------------------------------
     def add_request(self, req_id: Hashable):
@@ -214,7 +257,7 @@ class ModelRunner:
         for g, pages in by_group.items():
             idx = torch.tensor(sorted(pages), dtype=torch.long, device=self.rt.device)
             for i, kv in enumerate(self.kv):
-                if kv is not None and self.plan.entry_group[i] == g:
+                if kv is not None and self.plan.user_group[i] == g:
                     kv.index_fill_(0, idx, float("nan"))
             self.pages_poisoned += len(pages)
 
@@ -422,20 +465,25 @@ class ModelRunner:
                            logit_rows=d_rows, state_slots=d_state, max_position=int(positions.max()),
                            extras=extras)
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], greedy: bool = False):
         """Runs the entries' tokens as one batch; returns float32 logits [wanted, vocab] on the
-        device, in the order of the entries and of their ``want``."""
+        device, in the order of the entries and of their ``want``.  With ``greedy`` it returns, instead,
+        the index of the largest logit of every wanted row (the lowest on ties, src/engine/executor.py:51-54)
+        as a list of integers: a recorded step picks them inside its graph, and no logits travel."""
+        logits = None
         if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries) and entries:
-            logits = self._decode_step_with_graph(entries)
+            logits = self._decode_step_with_graph(entries, greedy)
         elif self.use_graphs and self._portion_graphs and len(entries) == 1 and len(entries[0].want) <= 1 and \
                 len(entries[0].tokens) >= self.PORTION_GRAPH_MIN and len(entries[0].tokens) % self.PORTION_GRAPH_STEP == 0:
-            logits = self._portion_step_with_graph(entries[0])
+            logits = self._portion_step_with_graph(entries[0], greedy)
         elif self.use_graphs and self._mixed_graphs and self._is_mixed_step(entries):
-            logits = self._mixed_step_with_graph(entries)
-        else:
+            logits = self._mixed_step_with_graph(entries, greedy)
+        if logits is None:                         # (also a shape that is not recorded yet)
             ctx = self.build_context(entries)
             self._clear_state_of_new_requests(ctx.seqs)
             logits = self.model.forward(ctx, self.bindings)
+            if greedy:
+                logits = ops.argmax(logits).tolist() if logits.shape[0] else []
         for e in entries:
             self.cache.commit(e.req_id, e.tokens)
         self._poison_pages()                       # (pages that a window has passed went back)
@@ -443,7 +491,17 @@ class ModelRunner:
         return logits
 
     # ---- decoding through a recorded graph ------------------------------------------------
-    def _decode_step_with_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _recorded_argmax(self, logits: torch.Tensor) -> Optional[torch.Tensor]:
+        """Inside a recording: the largest logit's index of every row, into a buffer that stays (through the
+        entry point that allocates nothing, where the rows fit its buffer)."""
+        if logits.shape[0] == 0:
+            return None
+        tokens = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+        if ops.argmax_static_takes(*logits.shape):
+            return ops.argmax_static(logits, tokens)
+        return ops.argmax(logits, out=tokens)
+
+    def _decode_step_with_graph(self, entries: Sequence[StepEntry], greedy: bool = False):
         seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._single_token_layout(entries)
         self._check_bounds(seqs, slots, upd_idx, upd_val)
         self._poison_pages()                       # (the pages just handed out, before anything is written)
@@ -473,14 +531,7 @@ class ModelRunner:
                     ops.scatter_int(self.tables[g], torch.from_numpy(upd_idx[g]).to(self.rt.device),
                                     torch.from_numpy(upd_val[g]).to(self.rt.device))
                 upd_idx[g] = upd_val[g] = np.zeros(0, dtype=i32)
-        key = (B, part_keys)
-        rec = self._graphs.pop(key, None)
-        if rec is None:
-            while len(self._graphs) >= self.MAX_GRAPHS:
-                self._graphs.pop(next(iter(self._graphs)))     # dicts keep insertion order: the oldest use
-            rec = self._record_decode_graph(B, part_keys, cap)
-            self.graphs_recorded += 1
-        self._graphs[key] = rec                                # (re)inserted last = most recently used
+        rec = self._graph_for((B, part_keys), "decode", lambda: self._record_decode_graph(B, part_keys, cap))
         iota, none, zero = rec["iota"], rec["none"], rec["zero"]       # 0 .. B - 1; cap times -1; cap zeros
         # (a row's table row is its request's state slot: tok_seq serves as both)
         parts = [token_ids, positions, tok_seq, iota, tok_seq]
@@ -494,6 +545,8 @@ class ModelRunner:
         rec["graph"].replay()
         self.graph_steps += 1
         self.graph_steps_of["decode"] += 1
+        if greedy:
+            return rec["tokens"].tolist()[:n_live]      # (one small copy to the host; waits for the step)
         return rec["logits"][:n_live].clone()          # the graph's own output is overwritten by the next replay
 
     # ---- single new tokens beside one prompt portion through a recorded graph -----------------
@@ -513,18 +566,27 @@ class ModelRunner:
                 portion = e
         return portion is not None
 
-    def _mixed_step_with_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _mixed_step_with_graph(self, entries: Sequence[StepEntry], greedy: bool = False):
         # the single tokens first, the portion last; the logits go back into the entries' order
         order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) > 1)
         ordered = [entries[i] for i in order]
-        tokens = self._check_and_reserve(ordered)
-        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(ordered, tokens)
-        self._check_bounds(seqs, slots, upd_idx, upd_val)
-        self._poison_pages()
         n_dec, n_groups, i32 = len(ordered) - 1, len(self.cache.groups), np.int32
         T1 = len(ordered[-1].tokens)
         B = self.graph_rows(n_dec)
         T = -(-T1 // self.MIXED_GRAPH_STEP) * self.MIXED_GRAPH_STEP
+        cap = 2 * B + 2 * (T // self.page_size + 2)
+        # which recorded step this is, from the requests' lengths alone (nothing is reserved yet: a shape
+        # that is not recorded runs as it comes)
+        max_dec_position = max([self.cache.get(e.req_id).num_tokens for e in ordered[:-1]], default=0)
+        portion_keys = self.cache.get(ordered[-1].req_id).num_tokens + T1
+        part_keys = tuple(cls.mixed_graph_key(max_dec_position, portion_keys) for cls in self._step_classes)
+        rec = self._graph_for(("mixed", B, T, part_keys), "mixed", lambda: self._record_mixed_graph(B, T, part_keys, cap))
+        if rec is None:
+            return None
+        tokens = self._check_and_reserve(ordered)
+        seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(ordered, tokens)
+        self._check_bounds(seqs, slots, upd_idx, upd_val)
+        self._poison_pages()
         fill, pad = B - n_dec, T - T1
         spare = self.spare_row
 
@@ -536,24 +598,12 @@ class ModelRunner:
         positions_all = padded(positions, 0, np.arange(pad, dtype=i32))
         tok_seq = padded(tok_seq, spare, np.full(pad, spare, dtype=i32))
         slots = [padded(x, -1, np.full(pad, -1, dtype=i32)) for x in slots]
-        cap = 2 * B + 2 * (T // self.page_size + 2)
         if any(len(u) > cap for u in upd_idx):
             for g in range(n_groups):
                 if len(upd_idx[g]):
                     ops.scatter_int(self.tables[g], torch.from_numpy(upd_idx[g]).to(self.rt.device),
                                     torch.from_numpy(upd_val[g]).to(self.rt.device))
                 upd_idx[g] = upd_val[g] = np.zeros(0, dtype=i32)
-        max_dec_position = int(positions[:n_dec].max()) if n_dec else 0
-        portion_keys = seqs[-1].kv_before + T1
-        part_keys = tuple(cls.mixed_graph_key(max_dec_position, portion_keys) for cls in self._step_classes)
-        key = ("mixed", B, T, part_keys)
-        rec = self._graphs.pop(key, None)
-        if rec is None:
-            while len(self._graphs) >= self.MAX_GRAPHS:
-                self._graphs.pop(next(iter(self._graphs)))
-            rec = self._record_mixed_graph(B, T, part_keys, cap)
-            self.graphs_recorded += 1
-        self._graphs[key] = rec
         none, zero = rec["none"], rec["zero"]
         parts = [token_ids, positions_all, tok_seq]
         for g in range(n_groups):
@@ -576,6 +626,9 @@ class ModelRunner:
                 picked.append(at)
             elif entries[i].want:
                 picked.append(B)
+        if greedy:
+            toks = rec["tokens"].tolist()
+            return [toks[i] for i in picked]
         logits = rec["logits"]
         if picked == list(range(n_dec)) + [B]:            # the usual order: no index has to travel
             return torch.cat([logits[:n_dec], logits[B:B + 1]]) if n_dec < B else logits[:B + 1].clone()
@@ -625,7 +678,8 @@ class ModelRunner:
         def run():
             for g in range(n_groups):
                 ops.scatter_int(self.tables[g], d_upd[g][0], d_upd[g][1])
-            return self.model.forward(ctx, self.bindings)
+            logits = self.model.forward(ctx, self.bindings)
+            return logits, self._recorded_argmax(logits)
 
         torch.cuda.synchronize()
         stream = torch.cuda.Stream()
@@ -636,39 +690,36 @@ class ModelRunner:
         ctx.memo.clear()                          # (what the parts made for the first run is made again inside the graph)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
-            logits = run()
+            logits, tokens = run()
         torch.cuda.synchronize()
         event = torch.cuda.Event()
         event.record()
-        return {"graph": graph, "ctx": ctx, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits,
+        return {"graph": graph, "ctx": ctx, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits, "tokens": tokens,
                 "event": event, "none": np.full(cap, -1, dtype=np.int32), "zero": np.zeros(cap, dtype=np.int32)}
 
     # ---- one prompt portion through a recorded graph ----------------------------------------
-    def _portion_step_with_graph(self, entry: StepEntry) -> torch.Tensor:
+    def _portion_step_with_graph(self, entry: StepEntry, greedy: bool = False):
+        T, n_want, n_groups = len(entry.tokens), len(entry.want), len(self.cache.groups)
+        cap = 2 * (T // self.page_size + 2)
+        i32 = np.int32
+        keys = self.cache.get(entry.req_id).num_tokens + T
+        part_keys = tuple(cls.portion_graph_key(T, keys) if hasattr(cls, "portion_graph_key") else None
+                          for cls in self._step_classes)
+        rec = self._graph_for(("portion", T, n_want, part_keys), "portion",
+                              lambda: self._record_portion_graph(T, n_want, cap, part_keys))
+        if rec is None:
+            return None
         tokens = self._check_and_reserve([entry])
         seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout([entry], tokens)
         self._check_bounds(seqs, slots, upd_idx, upd_val)
         self._poison_pages()
         self._clear_state_of_new_requests(seqs)
-        T, n_want, n_groups = len(token_ids), len(rows), len(self.cache.groups)
-        cap = 2 * (T // self.page_size + 2)
-        i32 = np.int32
         if any(len(u) > cap for u in upd_idx):
             for g in range(n_groups):
                 if len(upd_idx[g]):
                     ops.scatter_int(self.tables[g], torch.from_numpy(upd_idx[g]).to(self.rt.device),
                                     torch.from_numpy(upd_val[g]).to(self.rt.device))
                 upd_idx[g] = upd_val[g] = np.zeros(0, dtype=i32)
-        part_keys = tuple(cls.portion_graph_key(T, seqs[0].kv_before + T) if hasattr(cls, "portion_graph_key") else None
-                          for cls in self._step_classes)
-        key = ("portion", T, n_want, part_keys)
-        rec = self._graphs.pop(key, None)
-        if rec is None:
-            while len(self._graphs) >= self.MAX_GRAPHS:
-                self._graphs.pop(next(iter(self._graphs)))
-            rec = self._record_portion_graph(T, n_want, cap, part_keys)
-            self.graphs_recorded += 1
-        self._graphs[key] = rec
         none, zero = rec["none"], rec["zero"]
         parts = [token_ids, positions, tok_seq, rows, np.asarray([seqs[0].state_slot], dtype=i32)]
         for g in range(n_groups):
@@ -681,6 +732,8 @@ class ModelRunner:
         rec["graph"].replay()
         self.graph_steps += 1
         self.graph_steps_of["portion"] += 1
+        if greedy:
+            return rec["tokens"].tolist() if rec["tokens"] is not None else []
         return rec["logits"].clone()
 
     def _record_portion_graph(self, T: int, n_want: int, cap: int, part_keys: tuple):
@@ -720,7 +773,8 @@ class ModelRunner:
         def run():
             for g in range(n_groups):
                 ops.scatter_int(self.tables[g], d_upd[g][0], d_upd[g][1])
-            return self.model.forward(ctx, self.bindings)
+            logits = self.model.forward(ctx, self.bindings)
+            return logits, self._recorded_argmax(logits)
 
         torch.cuda.synchronize()
         stream = torch.cuda.Stream()
@@ -730,11 +784,11 @@ class ModelRunner:
         stream.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
-            logits = run()
+            logits, tokens = run()
         torch.cuda.synchronize()
         event = torch.cuda.Event()
         event.record()
-        return {"graph": graph, "ctx": ctx, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits,
+        return {"graph": graph, "ctx": ctx, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits, "tokens": tokens,
                 "event": event, "none": np.full(cap, -1, dtype=np.int32), "zero": np.zeros(cap, dtype=np.int32)}
 
     def _record_decode_graph(self, B: int, part_keys: tuple, cap: int):
@@ -774,7 +828,8 @@ class ModelRunner:
         def run():
             for g in range(n_groups):
                 ops.scatter_int(self.tables[g], d_upd[g][0], d_upd[g][1])
-            return self.model.forward(ctx, self.bindings)
+            logits = self.model.forward(ctx, self.bindings)
+            return logits, self._recorded_argmax(logits)
 
         torch.cuda.synchronize()
         stream = torch.cuda.Stream()
@@ -784,12 +839,12 @@ class ModelRunner:
         stream.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
-            logits = run()
+            logits, tokens = run()
         torch.cuda.synchronize()
         event = torch.cuda.Event()
         event.record()
         # (the context is kept with the graph: what the parts made for the recorded step, their
         # graph_extras, is read by every replay)
-        return {"graph": graph, "ctx": ctx, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits,
+        return {"graph": graph, "ctx": ctx, "host": host, "host_np": host.numpy(), "meta": meta, "logits": logits, "tokens": tokens,
                 "event": event, "iota": np.arange(B, dtype=np.int32), "none": np.full(cap, -1, dtype=np.int32),
                 "zero": np.zeros(cap, dtype=np.int32)}

@@ -184,8 +184,12 @@ class Scheduler:
             # The portion limit keeps a step short for the requests that decode in it.  While none
             # does, a prompt may take the whole budget: a long prompt in an idle engine then runs in
             # few large steps (8192 tokens: four steps instead of sixteen, 1.7 times sooner).
+            # Several prompts at once share the budget in equal parts of at least the portion limit, so that a
+            # long prompt does not hold a short one that arrived with it back until it is through.
+            with_prompt = sum(1 for r in self.running if r.num_known - r.num_computed > 1) + len(self.waiting)
+            shares = max(1, min(with_prompt, self.max_step_tokens // self.prefill_chunk))
             chunk = self.prefill_chunk if any(r.num_known - r.num_computed == 1 for r in self.running) \
-                else max(self.prefill_chunk, self.max_step_tokens)
+                else max(self.prefill_chunk, self.max_step_tokens // shares)
             # pages the entries planned so far need, per group: an entry fits if its own pages fit
             # beside them (the same answer as cache.can_reserve on the whole list, without going
             # through the list again for every candidate)

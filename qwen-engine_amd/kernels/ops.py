@@ -50,6 +50,8 @@ def load_library():
         "qe_gemm_silu_supported": [i32, i32, i32, i32, i32],
         "qe_gemm": [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp, f32, vp, i32, vp, vp],
         "qe_gemm_norm_supported": [i32, i32, i32, i32],
+        "qe_gemm_norm_preferred": [i32, i32, i32, i32, i32],
+        "qe_gemm_norm_max_rows": [],
         "qe_gemm_partial_splits": [i32, i32, i32],
         "qe_gemm_qkv_supported": [i32, i32, i32, i32, i32, i32, i32, i32],
         "qe_gemm_qkv_run": [vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, vp, f32, vp, vp, vp, i32, vp],
@@ -75,6 +77,7 @@ def load_library():
         "qe_gemm_branch_splits": [i32, i32, i32, i32, i32],
         "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
         "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
+        "qe_argmax_static": [vp, vp, i32, i32, vp],
         "qe_sample": [vp, vp, vp, vp, i32, i32, vp],
     }
     for name, args in sigs.items():
@@ -87,6 +90,8 @@ def load_library():
     lib.qe_mfma_probe.restype = ctypes.c_int
     lib.qe_argmax_workspace_bytes.argtypes = [i32, i32]
     lib.qe_argmax_workspace_bytes.restype = ctypes.c_long
+    lib.qe_argmax_static_max_bytes.argtypes = []
+    lib.qe_argmax_static_max_bytes.restype = ctypes.c_long
     lib.qe_attention_decode_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]
     lib.qe_attention_decode_workspace_bytes.restype = ctypes.c_long
     lib.qe_attention_prefill_workspace_bytes.restype = ctypes.c_long
@@ -266,6 +271,19 @@ def gemm_norm_supported(M: int, w: torch.Tensor) -> bool:
     for M rows of the stream against w: up to 16 rows, bfloat16 weights."""
     lib = load_library()
     return w.dtype in _DT and bool(lib.qe_gemm_norm_supported(int(M), w.shape[0], w.shape[1], _DT[w.dtype]))
+
+
+def gemm_norm_preferred(M: int, w: torch.Tensor, n_delta: int) -> bool:
+    """True if the product of M rows of the stream against w should do the residual sum of ``n_delta``
+    partial products and the norm before it in its prologue (gemm with ``norm_weight``) rather than leave
+    them to the norm's own kernel: gemm_norm_supported, and the sizes up to which that pays."""
+    lib = load_library()
+    return w.dtype in _DT and bool(lib.qe_gemm_norm_preferred(int(M), w.shape[0], w.shape[1], _DT[w.dtype], int(n_delta)))
+
+
+def gemm_norm_max_rows() -> int:
+    """No product takes the norm before it as its prologue with more rows than this."""
+    return load_library().qe_gemm_norm_max_rows()
 
 
 def gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -726,6 +744,25 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     nbytes = lib.qe_argmax_workspace_bytes(R, V)
     ws = torch.empty((nbytes,), dtype=torch.uint8, device=logits.device) if nbytes else None
     _check(lib.qe_argmax(logits.data_ptr(), out.data_ptr(), R, V, _ptr(ws), nbytes, _stream()), "argmax")
+    return out
+
+
+def argmax_static_takes(rows: int, vocab: int) -> bool:
+    """True if argmax_static takes logits of this shape (what lies between its two stages fits the
+    library's fixed buffer)."""
+    lib = load_library()
+    return lib.qe_argmax_workspace_bytes(int(rows), int(vocab)) <= lib.qe_argmax_static_max_bytes()
+
+
+def argmax_static(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """argmax into ``out`` (int32 [R]) without any allocation: what lies between the two stages is kept
+    in a buffer inside the library (one per GPU, shared by all calls on it: calls on one stream only).
+    For code that is recorded into a graph; needs argmax_static_takes(R, V)."""
+    lib = load_library()
+    _need(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    _need(out, "out", torch.int32, (R,), logits.device)
+    _check(lib.qe_argmax_static(logits.data_ptr(), out.data_ptr(), R, V, _stream()), "argmax (static)")
     return out
 
 

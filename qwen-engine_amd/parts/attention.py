@@ -16,7 +16,6 @@ import torch
 from ..cache.plan import KVNeed
 from ..kernels import ops
 from .base import CacheBinding, Runtime, StreamInput, TensorInfo
-from .block_sizes import FEW_ROWS, FEW_ROWS_MAX_WEIGHT, FEW_ROWS_PARTS
 from .registry import build_part, register_part
 
 
@@ -57,12 +56,12 @@ class PagedAttention:
 
     GRAPH_SPLIT_BUCKET = 8      # a recorded decode step serves positions up to the next multiple of this many key splits
 
-    @staticmethod
-    def graph_key(max_position: int) -> int:
+    @classmethod
+    def graph_key(cls, max_position: int) -> int:
         """The decode kernel's grid and workspace follow the number of key splits: recorded steps are
         kept per bucket of splits."""
         splits = int(max_position) // ops.DECODE_SPLIT_KEYS + 1
-        b = PagedAttention.GRAPH_SPLIT_BUCKET
+        b = cls.GRAPH_SPLIT_BUCKET
         return (splits + b - 1) // b * b
 
     @staticmethod
@@ -89,9 +88,9 @@ class PagedAttention:
     # tables' spare row that writes nowhere), then the portion, whose last row is the step's last.
     mixed_graph_dynamic_size = 4
 
-    @staticmethod
-    def mixed_graph_key(max_dec_position: int, portion_keys: int):
-        return PagedAttention.graph_key(max_dec_position), portion_keys > ops.prefill_uncut_keys()
+    @classmethod
+    def mixed_graph_key(cls, max_dec_position: int, portion_keys: int):
+        return cls.graph_key(max_dec_position), portion_keys > ops.prefill_uncut_keys()
 
     @staticmethod
     def mixed_graph_dynamic(rows: int, pad: int, tokens: int) -> List[int]:
@@ -109,8 +108,12 @@ class PagedAttention:
                 "portions": dynamic.view(2, 2), "portion_rows": int(tokens)}
 
     def _extras(self, ctx) -> dict:
-        return ctx.extras.get(PagedAttention) or {"dec_tokens": None, "other_tokens": None, "max_dec_position": 0,
-                                                  "max_other_keys": 0}
+        """What the step function prepared for this part's class (a class derived from this one finds
+        its own entry: the step function files them under the class of the part it met)."""
+        for cls in type(self).__mro__:
+            if cls in ctx.extras:
+                return ctx.extras[cls]
+        return {"dec_tokens": None, "other_tokens": None, "max_dec_position": 0, "max_other_keys": 0}
 
     def _other_tiles(self, ctx) -> Optional[torch.Tensor]:
         """The rows of requests that bring several tokens, cut into tiles for the prefill kernel: built
@@ -197,7 +200,7 @@ class PagedAttention:
             raise RuntimeError("attention was given no cache")
         lazy = None
         if isinstance(x, StreamInput):
-            if ctx.rt.dtype == torch.bfloat16 and self.w_qkv.numel() <= FEW_ROWS_MAX_WEIGHT and ops.gemm_norm_supported(x.rows, self.w_qkv):
+            if x.prefers_prologue(ops, self.w_qkv):
                 lazy, x = x, x.stream.h
             else:
                 x = x.materialize()
@@ -266,8 +269,6 @@ class PagedAttention:
 
     def _project_out(self, o: torch.Tensor) -> torch.Tensor:
         splits = ops.gemm_branch_splits(o, self.w_o)
-        if o.shape[0] <= FEW_ROWS and splits > FEW_ROWS_PARTS and ops.gemm_fused_supported(o, self.w_o):
-            splits = FEW_ROWS_PARTS
         if splits:
             # the product is cut along K (few rows: to fill the chip; a narrow matrix: to give every
             # compute unit blocks to overlap); the norm that follows adds the parts

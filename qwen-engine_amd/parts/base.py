@@ -125,18 +125,17 @@ class StreamInput:
     def rows(self) -> int:
         return self.stream.h.shape[0]
 
-    # Every block of the product reads the rows and all partial products of all rows: beyond this
-    # many bytes a block the norm's own kernel, which reads them once, is quicker.
-    FUSED_BYTES_PER_BLOCK = 192 * 1024
-
     def fusable(self) -> bool:
-        """True if a product should take the residual sum and the norm as its prologue: nothing to
-        add, or float32 partial products and a second buffer for the sums; and little enough to read."""
+        """True if a product can take the residual sum and the norm as its prologue at all: nothing to
+        add, or float32 partial products and a second buffer for the sums."""
         d = self.delta
-        if d is not None and not (d.dim() == 3 and d.dtype == torch.float32 and self.stream.spare is not None):
-            return False
-        parts = 1 + (d.shape[0] if d is not None else 0)
-        return self.stream.h.numel() * 4 * parts <= self.FUSED_BYTES_PER_BLOCK
+        return d is None or (d.dim() == 3 and d.dtype == torch.float32 and self.stream.spare is not None)
+
+    def prefers_prologue(self, ops, w: torch.Tensor) -> bool:
+        """True if the product against w should do the sum and the norm itself (the kernel library knows up
+        to which sizes that is quicker than the norm's own kernel); else the part calls materialize()."""
+        parts = 0 if self.delta is None else self.delta.shape[0]
+        return self.rt.dtype == torch.bfloat16 and ops.gemm_norm_preferred(self.rows, w, parts)
 
     def gemm(self, ops, w: torch.Tensor, bias=None, **kw) -> torch.Tensor:
         """The product of the normed rows with w, the residual sum and the norm inside it."""

@@ -9,7 +9,7 @@ from typing import Dict, Optional
 import torch
 
 from .base import CacheBinding, Runtime, Stream, StreamInput, TensorInfo, sub_tensors
-from .block_sizes import FEW_ROWS as FUSED_NORM_MAX_ROWS
+from ..kernels import ops
 from .registry import build_part, part_class, register_part
 
 def _names(spec):
@@ -31,8 +31,22 @@ class PreNormBlock:
         """False if any part of the block says that its forward cannot be recorded into a graph."""
         return all(getattr(p, "graph_safe", True) for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
 
+    @property
+    def graph_safe_with_state(self) -> bool:
+        """A part with per-request state is recorded into graphs only if it says itself that it can be."""
+        return getattr(self.mixer, "graph_safe", False) is True
+
     def parts(self):
         return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+
+    @staticmethod
+    def cache_needs(spec, hidden: int):
+        """What the block's parts keep per request, one (keys and values, fixed-size state) per cache
+        user, in the order in which forward gets their bindings: this block has one, its mixer."""
+        cls = part_class(spec.mixer.kind)
+        kv = cls.cache_need(spec.mixer) if hasattr(cls, "cache_need") else None
+        state = cls.state_need(spec.mixer, hidden) if hasattr(cls, "state_need") else None
+        return [(kv, state)]
 
     @staticmethod
     def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
@@ -46,23 +60,25 @@ class PreNormBlock:
         for name, part in zip(_names(self.spec), (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)):
             part.load(sub_tensors(tensors, name + "."), rt)
 
-    def forward(self, h, pending: Optional[torch.Tensor], ctx, binding: CacheBinding) -> torch.Tensor:
+    def forward(self, h, pending: Optional[torch.Tensor], ctx, bindings) -> torch.Tensor:
         """h: the 32-bit residual stream, a tensor (updated in place) or a Stream (whose buffers may
-        change places).  pending: branch output not yet added to the stream, or None.  Returns the
+        change places).  pending: branch output not yet added to the stream, or None.  bindings: one
+        CacheBinding per cache user of the block (cache_needs), here the mixer's.  Returns the
         feed-forward output, to be added by whoever norms next.  A branch output is [T, H] in the
         activation type, or float32 [S, T, H]: partial products that the norm adds in the order of S."""
         stream = h if isinstance(h, Stream) else Stream(h)
         x = self._input(self.mixer_norm, self.mixer, stream, pending, ctx)
-        a = self.mixer.forward(x, ctx, binding)
+        a = self.mixer.forward(x, ctx, bindings[0])
         x = self._input(self.ffn_norm, self.ffn, stream, a, ctx)
         return self.ffn.forward(x, ctx)
 
     @staticmethod
     def _input(norm, part, stream: Stream, delta, ctx):
-        """The part's input: the normed rows, or, with few rows and where both the norm and the part
-        can do it, the stream, what is to be added, and the norm, for the part's first product."""
+        """The part's input: the normed rows, or, with few rows (the model then gave the stream a second
+        buffer) and where both the norm and the part can do it, the stream, what is to be added, and
+        the norm, for the part's first product."""
         if (getattr(part, "takes_stream", False) and hasattr(norm, "fusable_weight") and
-                stream.h.shape[0] <= FUSED_NORM_MAX_ROWS):
+                stream.spare is not None):
             fw = norm.fusable_weight()
             si = StreamInput(stream, delta, norm, fw[0], fw[1], ctx.rt) if fw is not None else None
             if si is not None and si.fusable():

@@ -10,7 +10,6 @@ import torch
 
 from ..kernels import ops
 from .base import Runtime, StreamInput, TensorInfo
-from .block_sizes import FEW_ROWS, FEW_ROWS_MAX_WEIGHT, FEW_ROWS_PARTS
 from .registry import register_part
 
 
@@ -47,7 +46,7 @@ class SwiGLU:
         x: the normed rows, or a StreamInput."""
         a = None
         if isinstance(x, StreamInput):
-            if ctx.rt.dtype == torch.bfloat16 and self.w_gu.numel() <= FEW_ROWS_MAX_WEIGHT and ops.gemm_norm_supported(x.rows, self.w_gu):
+            if x.prefers_prologue(ops, self.w_gu):
                 a = x.gemm(ops, self.w_gu, epilogue=ops.EPI_SILU_MUL_IL if self.interleaved else ops.EPI_SILU_MUL)
             else:
                 x = x.materialize()
@@ -60,8 +59,6 @@ class SwiGLU:
         else:
             a = ops.silu_mul(ops.gemm(x, self.w_gu), interleaved=self.interleaved)
         splits = ops.gemm_branch_splits(a, self.w_down)
-        if a.shape[0] <= FEW_ROWS and splits > FEW_ROWS_PARTS and ops.gemm_fused_supported(a, self.w_down):
-            splits = FEW_ROWS_PARTS
         if splits:   # partial products along K, added by the norm that follows
             return ops.gemm(a, self.w_down, epilogue=ops.EPI_PARTIAL, splits=splits)
         return ops.gemm(a, self.w_down)

@@ -11,7 +11,6 @@ from ..cache.plan import CachePlan, plan_cache
 from ..config.spec import ModelSpec
 from ..kernels import ops
 from .base import CacheBinding, Runtime, Stream, TensorInfo, sub_tensors
-from .block import FUSED_NORM_MAX_ROWS
 from .registry import build_part, part_class
 
 
@@ -39,13 +38,14 @@ def _join(prefix: str, rel: str) -> str:
 
 
 def cache_plan(spec: ModelSpec) -> CachePlan:
+    """Every block kind says itself what its parts keep per request (``cache_needs(spec, hidden)``: a list
+    of (keys and values, fixed-size state), one per cache user of the block; none if it has no such method)."""
     needs = []
     for entry in spec.schedule:
-        mixer_spec = spec.layers[entry.layer].mixer
-        cls = part_class(mixer_spec.kind)
-        kv = cls.cache_need(mixer_spec) if hasattr(cls, "cache_need") else None
-        state = cls.state_need(mixer_spec, spec.hidden_size) if hasattr(cls, "state_need") else None
-        needs.append((kv, state, entry.cache_from))
+        layer = spec.layers[entry.layer]
+        cls = part_class(layer.kind)
+        users = list(cls.cache_needs(layer, spec.hidden_size)) if hasattr(cls, "cache_needs") else []
+        needs.append((users, entry.cache_from))
     return plan_cache(needs)
 
 
@@ -97,29 +97,35 @@ class DecoderModel:
                 part.load({rel: tensors[pre + rel] for rel in names}, rt)
 
     def weight_bytes_read_per_step(self) -> int:
-        """Bytes of every weight a step uses once (the embedding table only where it is the head)."""
-        seen, total = set(), 0
+        """Bytes of every weight a step uses once: all tensors that the parts hold (the parts inside the
+        parts included), a layer that the schedule runs n times n times; the embedding table only where
+        it is the head.  Tables that a step reads a few rows of (a position encoding's) are the parts'
+        to leave out: they keep them under a name that begins with an underscore."""
+        seen = set()
 
-        def add(t):
-            nonlocal total
-            if isinstance(t, torch.Tensor) and t.data_ptr() not in seen:
-                seen.add(t.data_ptr())
-                total += t.numel() * t.element_size()
+        def held(part) -> int:
+            total = 0
+            for name, v in vars(part).items():
+                if name.startswith("_"):
+                    continue
+                if isinstance(v, torch.Tensor):
+                    if v.data_ptr() not in seen:
+                        seen.add(v.data_ptr())
+                        total += v.numel() * v.element_size()
+                elif hasattr(v, "load") and hasattr(v, "expected_tensors"):     # a part inside the part
+                    total += held(v)
+            return total
 
         counts: Dict[int, int] = {}
         for e in self.spec.schedule:
             counts[e.layer] = counts.get(e.layer, 0) + 1
+        total = 0
         for idx, n in counts.items():
-            b = self.blocks[idx]
-            before = total
-            for part in (b.mixer_norm, b.mixer, b.ffn_norm, b.ffn):
-                for v in vars(part).values():
-                    add(v)
-            total += (n - 1) * (total - before)
+            total += n * held(self.blocks[idx])
         for part in self._around():
-            for v in vars(part).values():
-                add(v)
-        add(self.head)
+            total += held(part)
+        if self.head is not None and self.head.data_ptr() not in seen:
+            total += self.head.numel() * self.head.element_size()
         return total
 
     def forward(self, ctx, bindings: List[CacheBinding]) -> torch.Tensor:
@@ -129,10 +135,10 @@ class DecoderModel:
             if self.prologue is not None:
                 self.prologue.forward(h, ctx)
             # (few rows: a second buffer, so that a product can do the residual sum before it, see Stream)
-            stream = Stream(h, torch.empty_like(h) if h.shape[0] <= FUSED_NORM_MAX_ROWS else None)
+            stream = Stream(h, torch.empty_like(h) if h.shape[0] <= ops.gemm_norm_max_rows() else None)
             pending = None
             for i, entry in enumerate(self.spec.schedule):
-                pending = self.blocks[entry.layer].forward(stream, pending, ctx, bindings[i])
+                pending = self.blocks[entry.layer].forward(stream, pending, ctx, bindings[i])   # (the entry's users' bindings)
             h = stream.h
             R = ctx.logit_rows.shape[0]
             if R == 0:

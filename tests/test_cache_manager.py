@@ -229,9 +229,9 @@ def test_plan_groups_entries_by_need_and_lets_an_entry_read_another():
     plan = plan_cache([(full, None, None), (win, None, None), (full, None, 0), (None, StateNeed((4,)), None),
                        (win, None, None)])
     assert plan.groups == [GroupSpec(None), GroupSpec(8)]
-    assert plan.entry_group == [0, 1, 0, None, 1]
-    assert plan.entry_source == [0, 1, 0, None, 4]
-    assert plan.entry_kv[2] is None and plan.entry_state[3] == StateNeed((4,))
+    assert plan.user_group == [0, 1, 0, None, 1]
+    assert plan.user_source == [0, 1, 0, None, 4]
+    assert plan.user_kv[2] is None and plan.user_state[3] == StateNeed((4,))
     assert plan.bytes_per_token(2) == 3 * 2 * 2 * 16 * 2
     with pytest.raises(ValueError):
         plan_cache([(full, None, None), (KVNeed(1, 16, None), None, 0)])
@@ -277,3 +277,22 @@ def test_pages_handed_out_and_given_back_are_noted_and_kept_pages_are_not():
     ev = k.take_page_events()
     assert sorted(set(ev)) == [(0, 0), (0, 1), (0, 2)] and k.num_kept == 0
     k.check_invariants()
+
+
+def test_plan_with_blocks_of_several_cache_users_and_of_none():
+    """A block says how many of its parts keep something per request: two mixers side by side are two
+    users of one schedule entry, a block without a mixer has none; an entry that reads another entry's
+    cache pairs its users with that entry's."""
+    full, win = KVNeed(2, 16, None), KVNeed(2, 16, 8)
+    plan = plan_cache([([(full, None), (win, StateNeed((3,)))], None),     # entry 0: users 0 and 1
+                       ([], None),                                           # entry 1: no user
+                       ([(full, None), (win, None)], 0),                     # entry 2: reads entry 0's two caches
+                       (full, None, None)])                                  # entry 3: the short form, one user
+    assert plan.entry_users == [[0, 1], [], [2, 3], [4]]
+    assert plan.groups == [GroupSpec(None), GroupSpec(8)]
+    assert plan.user_group == [0, 1, 0, 1, 0]
+    assert plan.user_source == [0, 1, 0, 1, 4]
+    assert plan.user_kv == [full, win, None, None, full]
+    assert plan.user_state == [None, StateNeed((3,)), None, None, None]
+    with pytest.raises(ValueError):
+        plan_cache([([(full, None), (win, None)], None), ([(full, None)], 0)])   # one user cannot pair with two

@@ -152,7 +152,7 @@ def test_block_part_defers_its_last_residual_sum(dtype):
     cache = torch.zeros(8, 2, cfg.num_key_value_heads, page, cfg.head_dim, dtype=dtype, device=DEV)
     ctx = one_request_context(rt, list(range(T)), page, 8)
     hd = h.to(DEV)
-    out = block.forward(hd, pending.to(DEV), ctx, CacheBinding(cache, 0, True, None))
+    out = block.forward(hd, pending.to(DEV), ctx, [CacheBinding(cache, 0, True, None)])
     act = None if dtype == torch.float32 else dtype
     table = P.rope_table(cfg.rope_theta, cfg.head_dim, cfg.max_position_embeddings)
     h_in = h + pending.float()

@@ -132,6 +132,27 @@ def test_a_prompt_takes_the_whole_budget_while_nothing_decodes():
     assert short.output == expected_output(short.prompt, 20) and long.output == expected_output(long.prompt, 2)
 
 
+def test_prompts_that_arrive_together_share_the_budget():
+    """A long and a short prompt arrive in an idle engine: the long one does not take the whole budget step
+    after step; the short one's first token comes from the first step."""
+    sched, cache = make(num_pages=200, budget=32, chunk=8, max_model_len=400)
+    long = Request(0, list(range(3, 103)), SamplingParams(max_new_tokens=2))        # 100 tokens
+    short = Request(1, [5, 6, 7, 8, 9], SamplingParams(max_new_tokens=2))
+    sched.add(long)
+    sched.add(short)
+    log = []
+    drive(sched, cache, log)
+    assert log[0] == [(0, 16, False), (1, 5, True)]          # two prompts: half the budget each at most
+    assert log[1][0] == (0, 8, False)                          # the short one decodes now: portions of the limit
+    assert long.output == expected_output(long.prompt, 2) and short.output == expected_output(short.prompt, 2)
+    # three prompts and a budget of four portions: a third of the budget each, rounded down, at least a portion
+    sched, cache = make(num_pages=400, budget=32, chunk=8, max_model_len=400, max_num_seqs=4)
+    for i in range(3):
+        sched.add(Request(i, list(range(3, 103)), SamplingParams(max_new_tokens=1)))
+    planned = sched.plan()
+    assert [(p.request.req_id, len(p.tokens)) for p in planned] == [(0, 10), (1, 10), (2, 10)]
+
+
 def test_a_first_portion_of_the_whole_budget_that_does_not_fit_is_made_smaller():
     """12 pages of 4 tokens: a prompt of 40 tokens cannot take a first portion of the whole budget (64
     tokens would be the limit, 40 tokens are 10 pages, and 5 pages are held by another request), but a

@@ -141,3 +141,45 @@ def test_head_product_at_the_large_widths_against_the_whole_vocabulary(K):
         want = x.double() @ w_cols.t()
         err = float((got[:, cols].double() - want).abs().max()) / float(want.abs().max())
         assert err < 2e-5, (rows, err)
+
+
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_greedy_steps_give_the_argmax_of_the_logits(model_and_refs, use_graphs):
+    """step(..., greedy=True) returns the index of the largest logit of every wanted row (a recorded step
+    picks it inside its graph): the same steps on a second runner that returns logits, for decode steps that
+    are filled up to a recorded size, a portion of a round length, a portion beside single tokens in any
+    order of the entries, and a step without wanted rows."""
+    cfg, w, _ = model_and_refs
+    model = DecoderModel(cfg.to_model_spec())
+    model.load(w, Runtime(torch.device("cuda:0"), torch.bfloat16))
+    runners = [ModelRunner(model, page_size=16, num_pages=200, max_requests=12, use_graphs=use_graphs, debug_poison=True)
+               for _ in range(2)]
+    prompts = [tokens(30 + 17 * i, 7000 + i) for i in range(11)]
+    long = tokens(900, 7100)
+
+    def both(entries):
+        got = runners[0].step(entries, greedy=True)
+        logits = runners[1].step(entries)
+        assert isinstance(got, list) and got == logits.argmax(dim=1).tolist()
+        return got
+
+    for r in runners:
+        for i in range(11):
+            r.add_request(i)
+        r.add_request("p")
+    for i, p in enumerate(prompts):
+        assert len(both([StepEntry(i, p, [len(p) - 1])])) == 1                      # a lone ragged portion
+    last = [p[-1] for p in prompts]
+    for step in range(3):                                                           # 11 rows: filled up to 16
+        last = both([StepEntry(i, [last[i]], [0]) for i in range(11)])
+    assert both([StepEntry("p", long[:256], [])]) == []                             # a portion of a round length, nothing wanted
+    assert len(both([StepEntry("p", long[256:512], [255])])) == 1
+    singles = [StepEntry(i, [last[i]], [0]) for i in range(11)]
+    got = both(singles[:4] + [StepEntry("p", long[512:700], [187])] + singles[4:])  # the portion among the single tokens
+    assert len(got) == 12
+    got = both([StepEntry("p", long[700:830], [])] + [StepEntry(i, [got[i if i < 4 else i + 1]], [0]) for i in range(11)])
+    assert len(got) == 11
+    if use_graphs:
+        assert runners[0].graph_steps_of == runners[1].graph_steps_of
+        assert runners[0].graph_steps_of["decode"] == 3 and runners[0].graph_steps_of["portion"] == 2
+        assert runners[0].graph_steps_of["mixed"] == 11 + 2

@@ -153,9 +153,9 @@ def test_cache_plan_of_the_toy(toy):
     from qwen_engine_amd.parts import cache_plan
     plan = cache_plan(config_from_folder(toy).to_model_spec())
     assert [g.window for g in plan.groups] == [None, WINDOW]
-    assert plan.entry_group == [0, None, 1, 0, 0, None]
-    assert plan.entry_source == [0, None, 2, 3, 0, None]       # entry 4 reads entry 0's cache
-    assert [s is not None for s in plan.entry_state] == [False, True, False, False, False, True]
+    assert plan.user_group == [0, None, 1, 0, 0, None]
+    assert plan.user_source == [0, None, 2, 3, 0, None]       # entry 4 reads entry 0's cache
+    assert [s is not None for s in plan.user_state] == [False, True, False, False, False, True]
 
 
 @pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])

@@ -199,7 +199,7 @@ def test_the_toy_uses_both_new_parts(toy):
     assert kinds == [("WaveScale", "RoutedFeedForward"), ("RotaryHalf", "SwiGLU")]
     assert [b.graph_safe for b in model.blocks] == [False, True] and not model.graph_safe
     plan = cache_plan(config_from_folder(toy).to_model_spec())
-    assert len(plan.groups) == 1 and plan.entry_state == [None, None]
+    assert len(plan.groups) == 1 and plan.user_state == [None, None]
     # the router spreads the tokens over the experts (else the test would show little)
     _, w = P.read_folder(toy)
     x = torch.randn(200, H, generator=torch.Generator().manual_seed(1))

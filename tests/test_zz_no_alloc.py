@@ -43,15 +43,23 @@ def test_argmax_without_allocation_equals_argmax_with_a_workspace():
         inputs.append((logits, torch.full((R,), -7, dtype=torch.int32, device=dev),
                        torch.full((R,), -7, dtype=torch.int32, device=dev),
                        torch.empty(nbytes, dtype=torch.uint8, device=dev), nbytes))
+    # one call before the counts are taken: it asks for the address of this device's copy of the buffer,
+    # once per process (whatever the runtime sets up for that is not the entry point's own allocation)
+    warm = torch.zeros(2, 5000, device=dev)
+    assert lib.qe_argmax_static(warm.data_ptr(), torch.empty(2, dtype=torch.int32, device=dev).data_ptr(), 2, 5000, stream) == 0
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated(dev)
+    free_before = torch.cuda.mem_get_info(dev)[0]        # the driver's count of free bytes: sees a hipMalloc that torch's count cannot
     for (R, V), (logits, got, want, ws, nbytes) in zip(cases, inputs):
         rc = lib.qe_argmax_static(logits.data_ptr(), got.data_ptr(), R, V, stream)
         assert rc == 0, lib.qe_last_error().decode()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
+    assert torch.cuda.memory_allocated(dev) == before
+    for (R, V), (logits, got, want, ws, nbytes) in zip(cases, inputs):
         rc = lib.qe_argmax(logits.data_ptr(), want.data_ptr(), R, V, ws.data_ptr(), nbytes, stream)
         assert rc == 0, lib.qe_last_error().decode()
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated(dev) == before
     for (R, V), (logits, got, want, _, _) in zip(cases, inputs):
         assert got.tolist() == want.tolist()
         assert got.tolist() == logits.argmax(dim=1).tolist()
@@ -78,3 +86,30 @@ def test_sizes_beyond_the_fixed_buffer_are_refused():
     assert "static buffer" in msg and "437" in msg
     torch.cuda.synchronize()
     assert out.tolist() == [-7] * R
+
+
+def test_argmax_without_allocation_inside_a_graph_capture():
+    """Under stream capture an allocation is an error of the capture; the entry point records its two
+    kernels and nothing else.  Replayed three times with other logits and the program's own work between
+    the replays, each replay against the eager result."""
+    lib = _library()
+    dev = torch.device("cuda:0")
+    R, V = 8, 151936
+    g = torch.Generator().manual_seed(13)
+    logits = torch.randn(R, V, generator=g).to(dev)
+    out = torch.full((R,), -7, dtype=torch.int32, device=dev)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        assert lib.qe_argmax_static(logits.data_ptr(), out.data_ptr(), R, V, stream.cuda_stream) == 0   # (the address is known now)
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        rc = lib.qe_argmax_static(logits.data_ptr(), out.data_ptr(), R, V, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.qe_last_error().decode()
+    for rep in range(3):
+        logits.copy_(torch.randn(R, V, generator=g))
+        out.fill_(-7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert out.tolist() == logits.argmax(dim=1).tolist(), rep
