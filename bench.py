@@ -30,6 +30,11 @@ Other sizes and workloads (not what the default line reports):
                             arrive one every --arrive-every steps (default 8: some 16 alive at a time), so that
                             most steps are single new tokens beside one prompt portion
   --eager-mixed-steps       all three: run such steps as they come instead of replaying a recorded graph
+  --kernels                 no model step: each kernel of a layer alone, at 1, 8, 64, 512 and 2048 rows (the four
+                            products, the head's, decode and prefill attention at --context), its time from a
+                            recorded graph of repetitions over weights that do not fit the caches, and its rate
+                            against the nominal and the measured peaks (the counterpart of the reference's
+                            per-operator benchmarks, src/layers/ops/linear.py:204-249)
   --warmup-passes N         both: untimed passes over the workload with other tokens before the timed
                             one (default 1: the decode graphs are recorded there, as in a server that
                             has run for a while; 0 times the recording too)
@@ -83,6 +88,7 @@ def parse():
     ap.add_argument("--eager-mixed-steps", action="store_true",
                     help="run steps of single new tokens beside a prompt portion as they come, not from a recorded graph")
     ap.add_argument("--requests", type=int, default=None, help="requests of the serving workloads")
+    ap.add_argument("--kernels", action="store_true", help="time each kernel of a layer alone over a range of rows")
     ap.add_argument("--warmup-passes", type=int, default=1,
                     help="serving workloads: untimed passes before the timed one (they record the decode graphs)")
     return ap.parse_args()
@@ -189,6 +195,138 @@ def serving_run(args, cfg, model, layers, full_layers) -> int:
     return 0
 
 
+def kernel_sweep(args, cfg) -> int:
+    """Each kernel of a layer alone.  A kernel's time is that of a recorded graph of ``reps`` launches, each on
+    another copy of its weights (or cache), the copies together larger than the 256 MB memory-side cache: as in
+    a model step, where a layer's weights come from HBM.  Products are asked for as the parts ask for them."""
+    import torch
+    from qwen_engine_amd.kernels import ops
+
+    dev = torch.device("cuda:0")
+    bf = torch.bfloat16
+    H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    Hq, Hkv, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    P, ctx_len = args.block_size, args.context
+    copy_gbs = None
+    probe = ops.mfma_probe() / 1e12
+    g = torch.Generator(device="cpu").manual_seed(args.seed)
+
+    def timed(launch, reps):
+        """launch(i): the i-th launch.  Microseconds a launch, the best of three replays."""
+        for i in range(min(reps, 3)):
+            launch(i)
+        torch.cuda.synchronize()
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            with ops.one_stream():
+                for i in range(reps):
+                    launch(i)
+        best = None
+        for _ in range(3):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            graph.replay()
+            b.record()
+            b.synchronize()
+            t = a.elapsed_time(b) * 1e3 / reps
+            best = t if best is None else min(best, t)
+        return best
+
+    def copies_of(nbytes):
+        return max(2, min(48, -(-(640 << 20) // max(1, nbytes))))
+
+    rows_all = (1, 8, 64, 512, 2048)
+    out = []
+
+    def record(name, rows, us, nbytes, flops, note=""):
+        gbs, tf = nbytes / us / 1e3, flops / us / 1e6
+        out.append({"kernel": name, "rows": rows, "us": round(us, 2), "gbs": round(gbs, 1), "tflops": round(tf, 1),
+                    "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "frac_mfma": round(tf * 1e12 / PEAK_FLOPS["bf16"], 4),
+                    "frac_mfma_measured": round(tf / probe, 4), **({"note": note} if note else {})})
+        print(f"[bench] {name:28s} rows {rows:5d}  {us:9.2f} us  {gbs:8.1f} GB/s  {tf:8.1f} TFLOP/s  {note}",
+              file=sys.stderr, flush=True)
+
+    products = [("q|k|v product", (Hq + 2 * Hkv) * D, H, "store"), ("o product", H, Hq * D, "branch"),
+                ("gate|up product + silu.mul", 2 * I, H, "silu"), ("down product", H, I, "branch"),
+                ("head product (32-bit logits)", V, H, "head")]
+    for name, N, K, kind in products:
+        n = copies_of(N * K * 2)
+        ws = [(torch.randn(N, K, generator=g) * 0.02).to(bf).to(dev) for _ in range(2)]
+        ws = ws + [ws[i % 2].clone() for i in range(n - 2)]
+        if kind == "silu":
+            ws = [ops.interleave_gate_up(w[:N // 2], w[N // 2:]) for w in ws]
+        for rows in rows_all:
+            if kind == "head" and rows > 64:
+                continue                                   # (logits are asked for at a step's wanted rows only)
+            x = torch.randn(rows, K, generator=g).to(bf).to(dev)
+            if kind == "silu":
+                f = (lambda i: ops.gemm(x, ws[i % n], epilogue=ops.EPI_SILU_MUL_IL)) if ops.gemm_silu_supported(x, ws[0]) \
+                    else (lambda i: ops.silu_mul(ops.gemm(x, ws[i % n]), interleaved=True))
+            elif kind == "branch":
+                splits = ops.gemm_branch_splits(x, ws[0])
+                f = (lambda i: ops.gemm(x, ws[i % n], epilogue=ops.EPI_PARTIAL, splits=splits)) if splits \
+                    else (lambda i: ops.gemm(x, ws[i % n]))
+            elif kind == "head":
+                f = lambda i: ops.gemm(x, ws[i % n], out_dtype=torch.float32)
+            else:
+                f = lambda i: ops.gemm(x, ws[i % n])
+            us = timed(f, 2 * n)
+            record(name, rows, us, N * K * 2 + rows * K * 2, 2.0 * rows * N * K,
+                   f"{splits} partial products" if kind == "branch" and splits else "")
+        del ws
+        torch.cuda.empty_cache()
+
+    # attention over the cache: decode (rows requests, one new token each, at the context), and one prompt portion
+    scale = 1.0 / D ** 0.5
+    pages_per_req = -(-ctx_len // P)
+    for rows in (1, 8, 64):
+        kv_bytes = rows * ctx_len * 2 * Hkv * D * 2
+        n = max(2, min(8, -(-(640 << 20) // kv_bytes)))
+        caches = [torch.randn(rows * pages_per_req, 2, Hkv, P, D, device=dev).to(bf) for _ in range(n)]
+        table = torch.arange(rows * pages_per_req, dtype=torch.int32, device=dev).view(rows, pages_per_req)
+        pos = torch.full((rows,), ctx_len - 1, dtype=torch.int32, device=dev)
+        seq = torch.arange(rows, dtype=torch.int32, device=dev)
+        q = torch.randn(rows, Hq, D, device=dev).to(bf)
+        f = lambda i: ops.attention(q, caches[i % n], pos, seq, table, scale, dec_tokens=seq, max_dec_position=ctx_len - 1,
+                                    other_tokens=None)
+        us = timed(f, 4 * n)
+        record("decode attention (split + merge)", rows, us, kv_bytes, 4.0 * rows * Hq * D * ctx_len, f"context {ctx_len}")
+        del caches
+        torch.cuda.empty_cache()
+    from qwen_engine_amd.parts.attention import prefill_tiles
+    for rows in (64, 512, 2048):
+        for before in (0, max(0, ctx_len - rows)):
+            if before == 0 and rows > ctx_len:
+                continue
+            keys = before + rows
+            pages = -(-keys // P)
+            cache = torch.randn(pages, 2, Hkv, P, D, device=dev).to(bf)
+            table = torch.arange(pages, dtype=torch.int32, device=dev).view(1, pages)
+            pos = torch.arange(before, keys, dtype=torch.int32, device=dev)
+            seq = torch.zeros(rows, dtype=torch.int32, device=dev)
+            q = torch.randn(rows, Hq, D, device=dev).to(bf)
+            other = torch.arange(rows, dtype=torch.int32, device=dev)
+            tiles = torch.tensor(prefill_tiles([(0, rows)], ops.prefill_tile_rows(Hq, Hkv)), dtype=torch.int32).view(-1, 2).to(dev)
+            f = lambda i: ops.attention(q, cache, pos, seq, table, scale, dec_tokens=None, other_tokens=other,
+                                        other_tiles=tiles, max_other_keys=keys)
+            us = timed(f, 8)
+            flops = 4.0 * Hq * D * (rows * before + rows * (rows + 1) / 2.0)
+            record("prefill attention", rows, us, keys * 2 * Hkv * D * 2, flops, f"after {before} cached tokens")
+            del cache
+            if before == max(0, ctx_len - rows):
+                break
+    line = {"metric": f"per-kernel sweep (Qwen3-{args.model.upper()} sizes)", "unit": "us", "n_gpus": 1, "dtype": "bf16",
+            "data": "synthetic: random operands", "config": {"model": f"Qwen3-{args.model.upper()} sizes", "hidden_size": H,
+            "num_attention_heads": Hq, "num_key_value_heads": Hkv, "head_dim": D, "intermediate_size": I, "vocab_size": V,
+            "context": ctx_len, "page_size": P},
+            "peaks": {"hbm_gbs": HBM_PEAK_GBS, "mfma_tflops": PEAK_FLOPS["bf16"] / 1e12, "measured_mfma_tflops": round(probe, 1)},
+            "kernels": out}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     args = parse()
     if args.gpus != 1:
@@ -210,6 +348,9 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     ops.load_library()
+
+    if args.kernels:
+        return kernel_sweep(args, cfg)
 
     t0 = time.time()
     model = DecoderModel(cfg.to_model_spec())
