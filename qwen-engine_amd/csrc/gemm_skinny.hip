@@ -397,10 +397,15 @@ bool qe_gemm_skinny_ok(int M, int N, int K, int dt_a, int dt_w) {
 }
 
 // How many partial products a [M, N] = [M, K] . [N, K]^T product is best cut into along K so that
-// the launch has some 512 blocks, each wave still summing at least two chunks.
+// the launch has some 512 blocks (1024 against a matrix of 16 M elements or more: a wave has one round of
+// loads in flight, and a large matrix is read at the memory's rate only with four waves a SIMD: the o and
+// down products of eight rows at the 32B sizes take 22 and 64 us in four cuts where they took 31 and 98 in
+// one), each wave still summing at least two chunks.
 int qe_gemm_skinny_splits(int N, int K) {
     const int blocks = qe_cdiv(N, 16);
-    int s = 512 / (blocks > 0 ? blocks : 1);
+    const int want = (long)N * K >= (16L << 20) ? 1024 : 512;
+    int s = qe_cdiv(want, blocks > 0 ? blocks : 1);
+    if (want == 512) s = 512 / (blocks > 0 ? blocks : 1);
     const int most = (K / 32) / 8;
     if (s > most) s = most;
     if (s > 16) s = 16;
