@@ -101,3 +101,21 @@ def test_engine_config_page_count_follows_the_reference():
     assert EngineConfig(num_blocks=7).pages_per_group() == 7
     with pytest.raises(ValueError):
         EngineConfig(dtype="float16").validate()
+
+
+def test_pool_sized_from_free_memory():
+    """Without num_blocks and with gpu_memory_fraction the pool takes that fraction of the memory that is free
+    after the weights, less what recorded steps may hold; the reference's formula (main.py:23) otherwise."""
+    from qwen_engine_amd.config import EngineConfig
+    cfg = EngineConfig(max_num_seqs=4, max_model_len=256, block_size=16)
+    assert cfg.pages_per_group() == 4 * 16                                     # main.py:23
+    assert EngineConfig(num_blocks=7, gpu_memory_fraction=0.5).pages_per_group(1 << 40, 4096) == 7   # an explicit number wins
+    cfg = EngineConfig(max_model_len=256, block_size=16, gpu_memory_fraction=0.5, graph_memory_bytes=1 << 30)
+    per_page = 28 * 2 * 8 * 128 * 2 * 16                                        # bytes of a page through 28 layers
+    assert cfg.pages_per_group(10 << 30, per_page) == ((10 << 30) // 2 - (1 << 30)) // per_page
+    with pytest.raises(ValueError):
+        cfg.pages_per_group()                                                   # needs the two numbers
+    with pytest.raises(ValueError):
+        cfg.pages_per_group(2 << 30, per_page)                                  # half of 2 GiB less 1 GiB: nothing left
+    with pytest.raises(ValueError):
+        EngineConfig(gpu_memory_fraction=1.5).validate()

@@ -367,3 +367,20 @@ def test_random_engine_sizes_and_prompt_sets(folders, which):
                 e2.runner.cache.check_invariants()
             assert both[0] == both[1], (seed, sizes)
     assert preempted >= 2 and shared >= 5          # the draws reach both
+
+
+def test_pool_sized_from_the_free_memory(folders):
+    """EngineConfig.gpu_memory_fraction: the pool gets what that fraction of the free device memory holds,
+    and generation runs in it as in a pool of a given size."""
+    folder = folders["A"]
+    cfg, w = P.read_folder(folder)
+    prompt = prompts_for(cfg, [9], 77)[0]
+    want = P.greedy_generate(cfg, w, prompt, 5)
+    ecfg = EngineConfig(dtype="float32", block_size=4, max_model_len=64, gpu_memory_fraction=0.001, graph_memory_bytes=0)
+    engine = LLMEngine.from_folder(folder, ecfg)
+    free = torch.cuda.mem_get_info()[0]
+    pages = engine.runner.cache.pools[0].num_pages
+    per_page = cfg["num_hidden_layers"] * 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * 4 * 4
+    assert pages >= 16 and abs(pages * per_page - 0.001 * (free + pages * per_page)) < 0.0002 * free
+    engine.submit([prompt], max_new_tokens=5, ignore_eos=True)
+    assert engine.run()[0].token_ids == want
