@@ -36,8 +36,9 @@ Other sizes and workloads (not what the default line reports):
                             against the nominal and the measured peaks (the counterpart of the reference's
                             per-operator benchmarks, src/layers/ops/linear.py:204-249)
   --warmup-passes N         both: untimed passes over the workload with other tokens before the timed
-                            one (default 1: the decode graphs are recorded there, as in a server that
-                            has run for a while; 0 times the recording too)
+                            one (default 2: the graphs are recorded there, a shape of steps when it is met
+                            the second time, as in a server that has run for a while; 0 times the
+                            recording too)
 """
 import argparse
 import json
@@ -89,7 +90,7 @@ def parse():
                     help="run steps of single new tokens beside a prompt portion as they come, not from a recorded graph")
     ap.add_argument("--requests", type=int, default=None, help="requests of the serving workloads")
     ap.add_argument("--kernels", action="store_true", help="time each kernel of a layer alone over a range of rows")
-    ap.add_argument("--warmup-passes", type=int, default=1,
+    ap.add_argument("--warmup-passes", type=int, default=2,
                     help="serving workloads: untimed passes before the timed one (they record the decode graphs)")
     return ap.parse_args()
 

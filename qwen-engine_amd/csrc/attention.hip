@@ -15,7 +15,7 @@ bool qe_attention_decode_ok(int Hq, int Hkv, int D, int P, int dt_a);
 size_t qe_attention_decode_workspace(int n_dec, int Hq, int D, int num_splits);
 int qe_attention_decode(const void* q, void* out, const void* cache, const int* dec_tokens, int n_dec,
                         const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
-                        int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
+                        const int* shared_keys, int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
                         int split_keys, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 int qe_attention_prefill(const void* q, void* out, const void* cache, const int* tiles, int num_tiles,
@@ -123,35 +123,38 @@ extern "C" long qe_attention_decode_workspace_bytes(int n_dec, int Hq, int D, in
 
 int qe_attention_decode_fused(const void* qkv, void* out, void* cache, const int* dec_tokens, int n_dec,
                               const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
-                              const int* slots, const float* q_w, const float* k_w, float eps, const float* table,
-                              int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
+                              const int* shared_keys, const int* slots, const float* q_w, const float* k_w, float eps,
+                              const float* table, int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
                               int split_keys, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 // Decode attention with the q/k norm, the rotation and the cache write of the new tokens inside:
 // qkv [T, (Hq + 2 Hkv) D] bfloat16 as the projection left it; q_w, k_w [D] float or null; table
 // [positions, D] float rows [cos | sin] (a rotation over the whole head) or null; slots [T]: where
-// each row's own key and value go in the cache (negative: nowhere).  Takes what
-// qe_attention_decode_supported takes.
+// each row's own key and value go in the cache (negative: nowhere).  shared_keys: null, or per row of the
+// block table how many of the request's first keys other requests read too (a hint for the caches: those
+// keys are left in them, the others stream past).  Takes what qe_attention_decode_supported takes.
 extern "C" int qe_attention_decode_fused_run(const void* qkv, void* out, void* cache, const int* dec_tokens,
                                              int n_dec, const int* positions, const int* tok_seq,
-                                             const int* block_table, int max_blocks, const int* slots,
+                                             const int* block_table, int max_blocks, const int* shared_keys,
+                                             const int* slots,
                                              const float* q_w, const float* k_w, float eps, const float* table,
                                              int Hq, int Hkv, int D, int P, float scale, int window,
                                              int max_position, int split_keys, void* workspace,
                                              long workspace_bytes, hipStream_t stream) {
     QE_REQUIRE(Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && max_position >= 0, "decode attention: bad sizes");
     return qe_attention_decode_fused(qkv, out, cache, dec_tokens, n_dec, positions, tok_seq, block_table,
-                                     max_blocks, slots, q_w, k_w, eps, table, Hq, Hkv, D, P, scale, window,
+                                     max_blocks, shared_keys, slots, q_w, k_w, eps, table, Hq, Hkv, D, P, scale, window,
                                      max_position, split_keys, workspace, (size_t)workspace_bytes, stream);
 }
 
 extern "C" int qe_attention_decode_run(const void* q, void* out, const void* cache, const int* dec_tokens,
                                        int n_dec, const int* positions, const int* tok_seq,
-                                       const int* block_table, int max_blocks, int Hq, int Hkv, int D, int P,
-                                       float scale, int window, int max_position, int split_keys,
-                                       void* workspace, long workspace_bytes, hipStream_t stream) {
+                                       const int* block_table, int max_blocks, const int* shared_keys,
+                                       int Hq, int Hkv, int D, int P, float scale, int window,
+                                       int max_position, int split_keys, void* workspace, long workspace_bytes,
+                                       hipStream_t stream) {
     QE_REQUIRE(Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && max_position >= 0, "decode attention: bad sizes");
     return qe_attention_decode(q, out, cache, dec_tokens, n_dec, positions, tok_seq, block_table, max_blocks,
-                               Hq, Hkv, D, P, scale, window, max_position, split_keys, workspace,
+                               shared_keys, Hq, Hkv, D, P, scale, window, max_position, split_keys, workspace,
                                (size_t)workspace_bytes, stream);
 }

@@ -16,7 +16,7 @@ template <int D, int SPLIT>
 __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
     const int* __restrict__ dec_tokens, const int* __restrict__ positions, const int* __restrict__ tok_seq,
-    const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ shared_keys,
     float* __restrict__ part_acc, float* __restrict__ part_ml,
     int Hq, int Hkv, int P, float scale, int window, int num_splits) {
     constexpr int TILES = SPLIT / 16;
@@ -36,7 +36,10 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
         if (head_ok && g == 0) { pml[0] = -INFINITY; pml[1] = 0.f; }
         return;
     }
-    const int* bt = block_table + (long)tok_seq[t] * max_blocks;
+    const int row = tok_seq[t];
+    const int* bt = block_table + (long)row * max_blocks;
+    // (keys that other requests read too are left in the caches, the others stream: see load_tile)
+    const bool stream = !(shared_keys && split * SPLIT < shared_keys[row]);
     const long page_stride = 2L * Hkv * P * D;
     const int tile0 = (k_begin - split * SPLIT) / 16;                 // first and one-past-last tile of the split
     const int tile1 = (k_end - split * SPLIT + 15) / 16;
@@ -57,7 +60,7 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     // Two tile buffers used in turn: the loads of the next tile are issued before the current
     // one is computed, and nothing is copied from one buffer to the other.
 #define LOAD(buf_, i_) load_tile<D>(buf_, cache, __builtin_amdgcn_readlane(my_page, (i_)), page_stride, kvh, Hkv, P, \
-                                    (split * SPLIT + (i_) * 16) % P, g, n)
+                                    (split * SPLIT + (i_) * 16) % P, g, n, stream)
 #define STEP(buf_, i_) attn_tile_step<D>(st, buf_, qreg, scale, split * SPLIT + (i_) * 16, g, k_begin, k_end, k_begin, k_end)
     KVTile<D> ta, tb;
     int i = tile0;
@@ -178,8 +181,8 @@ template <int D, int SPLIT, int AHEAD>
 __global__ __launch_bounds__(64) void attention_decode_fused_split_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* cache,
     const int* __restrict__ dec_tokens, const int* __restrict__ positions, const int* __restrict__ tok_seq,
-    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ slots,
-    const float* __restrict__ q_w, const float* __restrict__ k_w, float eps, const float* __restrict__ table,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ shared_keys,
+    const int* __restrict__ slots, const float* __restrict__ q_w, const float* __restrict__ k_w, float eps, const float* __restrict__ table,
     float* __restrict__ part_acc, float* __restrict__ part_ml,
     int Hq, int Hkv, int P, float scale, int window, int num_splits) {
     constexpr int TILES = SPLIT / 16;
@@ -208,13 +211,15 @@ __global__ __launch_bounds__(64) void attention_decode_fused_split_kernel(
     st.init();
     bf16x8 qreg[D / 32];
     if (k_begin < k_end) {
-        const int* bt = block_table + (long)tok_seq[t] * max_blocks;
+        const int row = tok_seq[t];
+        const int* bt = block_table + (long)row * max_blocks;
+        const bool stream = !(shared_keys && split * SPLIT < shared_keys[row]);
         const int tile0 = (k_begin - split * SPLIT) / 16;
         const int tile1 = (k_end - split * SPLIT + 15) / 16;
         int my_page = 0;
         if (lane >= tile0 && lane < tile1) my_page = bt[(split * SPLIT + lane * 16) / P];
 #define LOAD(buf_, i_) load_tile<D>(buf_, cache, __builtin_amdgcn_readlane(my_page, (i_)), page_stride, kvh, Hkv, P, \
-                                    (split * SPLIT + (i_) * 16) % P, g, n)
+                                    (split * SPLIT + (i_) * 16) % P, g, n, stream)
 #define STEP(buf_, i_) attn_tile_step<D>(st, buf_, qreg, scale, split * SPLIT + (i_) * 16, g, k_begin, k_end, k_begin, k_end)
         NormRotate<D> nq;
         nq.fetch(qkv + t * width + (long)head * D, head_ok, q_w, cs, g);
@@ -394,10 +399,12 @@ size_t qe_attention_decode_workspace(int n_dec, int Hq, int D, int num_splits) {
 // dec_tokens: the rows of q that are single new tokens of their requests (null: the rows
 // 0 .. n_dec - 1, which saves every wave a dependent load).  max_position: the
 // largest of their positions (fixes the number of splits).  workspace: at least
-// qe_attention_decode_workspace(...) bytes.
+// qe_attention_decode_workspace(...) bytes.  shared_keys: null, or for every row of the block table
+// the number of the request's first keys that other requests of the step may read as well (pages they
+// hold together): a hint for the caches, results do not depend on it.
 int qe_attention_decode(const void* q, void* out, const void* cache, const int* dec_tokens, int n_dec,
                         const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
-                        int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
+                        const int* shared_keys, int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
                         int split_keys, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     QE_REQUIRE(qe_attention_decode_ok(Hq, Hkv, D, P, QE_BF16), "decode attention: sizes not taken");
     QE_REQUIRE(split_keys == 128 || split_keys == 256, "decode attention: splits of 128 or 256 keys, not %d", split_keys);
@@ -415,7 +422,7 @@ int qe_attention_decode(const void* q, void* out, const void* cache, const int* 
     do {                                                                                                \
         attention_decode_split_kernel<D_, S_><<<grid, 64, 0, stream>>>(                                 \
             (const bf16_t*)q, (const bf16_t*)cache, dec_tokens, positions, tok_seq, block_table,        \
-            max_blocks, part_acc, part_ml, Hq, Hkv, P, scale, window, num_splits);                      \
+            max_blocks, shared_keys, part_acc, part_ml, Hq, Hkv, P, scale, window, num_splits);         \
         attention_decode_merge_kernel<D_><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, dec_tokens,     \
                                                                      (bf16_t*)out, Hq, num_splits);     \
     } while (0)
@@ -434,7 +441,7 @@ int qe_attention_decode(const void* q, void* out, const void* cache, const int* 
 // its own new key; the cache holds the keys before it.
 int qe_attention_decode_fused(const void* qkv, void* out, void* cache, const int* dec_tokens, int n_dec,
                               const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
-                              const int* slots, const float* q_w, const float* k_w, float eps, const float* table,
+                              const int* shared_keys, const int* slots, const float* q_w, const float* k_w, float eps, const float* table,
                               int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
                               int split_keys, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     QE_REQUIRE(qe_attention_decode_ok(Hq, Hkv, D, P, QE_BF16), "decode attention: sizes not taken");
@@ -454,11 +461,13 @@ int qe_attention_decode_fused(const void* qkv, void* out, void* cache, const int
         if (few)                                                                                        \
             attention_decode_fused_split_kernel<D_, S_, 3><<<grid, 64, 0, stream>>>(                    \
                 (const bf16_t*)qkv, (bf16_t*)cache, dec_tokens, positions, tok_seq, block_table, max_blocks, \
-                slots, q_w, k_w, eps, table, part_acc, part_ml, Hq, Hkv, P, scale, window, num_splits); \
+                shared_keys, slots, q_w, k_w, eps, table, part_acc, part_ml, Hq, Hkv, P, scale, window, \
+                num_splits);                                                                            \
         else                                                                                            \
         attention_decode_fused_split_kernel<D_, S_, 1><<<grid, 64, 0, stream>>>(                        \
             (const bf16_t*)qkv, (bf16_t*)cache, dec_tokens, positions, tok_seq, block_table, max_blocks, \
-            slots, q_w, k_w, eps, table, part_acc, part_ml, Hq, Hkv, P, scale, window, num_splits);     \
+            shared_keys, slots, q_w, k_w, eps, table, part_acc, part_ml, Hq, Hkv, P, scale, window,     \
+            num_splits);                                                                                \
         attention_decode_merge_kernel<D_><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, dec_tokens,     \
                                                                      (bf16_t*)out, Hq, num_splits);     \
     } while (0)

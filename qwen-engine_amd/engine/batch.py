@@ -35,6 +35,10 @@ class StepContext:
     logit_rows: torch.Tensor           # int32 [R] rows whose logits are wanted
     state_slots: torch.Tensor          # int32 [B]
     max_position: int = 0              # largest position in the batch (host)
+    # int32, an entry per row of the block tables, or None: how many of the request's first keys lie in
+    # pages that other requests read as well (a shared prefix).  A hint for kernels that choose between
+    # loads that leave a line in the caches and loads that stream past them; no result depends on it.
+    shared_keys: Optional[torch.Tensor] = None
     # What single parts asked to have prepared for this step, by part class (see
     # ``parts.base``: step_extras / graph_extras), and a place where a part may keep what it
     # builds once per step and shares between its layers.

@@ -153,6 +153,9 @@ class ModelRunner:
         for t in self.tables:
             t[max_requests].zero_()            # (every entry: the stand-in of a recorded prompt portion reads them all)
         self.spare_row = max_requests
+        # per table row: the request's first keys that other requests read too (StepContext.shared_keys)
+        self.shared_keys = torch.zeros(max_requests + 1, dtype=torch.int32, device=dev)
+        self._shared_keys_host = [0] * (max_requests + 1)
         # positions that a row standing on the spare row may have: inside every group's table row, and the model's
         self._spare_positions = min([w * page_size for w in self.table_width] + [model.spec.max_positions])
         # a part with per-request state is recorded into graphs only if it says that it can be
@@ -235,13 +238,19 @@ class ModelRunner:
         self.cache.free_request(req_id)
         self._poison_pages()
 
-    def _clear_state_of_new_requests(self, seqs: Sequence[SeqInfo]) -> None:
-        """The fixed-size state of a request that runs its first step begins at zero."""
+    def _begin_new_requests(self, seqs: Sequence[SeqInfo]) -> None:
+        """For a request that runs its first step: its fixed-size state begins at zero, and its entry of
+        ``shared_keys`` says how many of its first keys lie in pages that it took over from other requests
+        (the request that computed them first is not told: one reader of many)."""
         for s in seqs:
             if s.new_request:
                 for st in self.state:
                     if st is not None:
                         st[s.state_slot].zero_()
+                shared = self.cache.get(s.req_id).shared_len
+                if self._shared_keys_host[s.state_slot] != shared:
+                    self._shared_keys_host[s.state_slot] = shared
+                    self.shared_keys[s.state_slot:s.state_slot + 1].fill_(shared)
 
     def _poison_pages(self) -> None:
         """With debug_poison: NaN into every page that was handed out or went back since the last
@@ -461,7 +470,8 @@ class ModelRunner:
         for (cls, name), t in zip(wanted, dev[n_fixed + 3 * n_groups:]):
             extras[cls][name] = t
         return StepContext(rt=self.rt, page_size=self.page_size, num_tokens=T, seqs=seqs, token_ids=d_tok,
-                           positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
+                           positions=d_pos, tok_seq=d_seq, block_tables=self.tables,
+                           shared_keys=self.shared_keys, slots=d_slots,
                            logit_rows=d_rows, state_slots=d_state, max_position=int(positions.max()),
                            extras=extras)
 
@@ -480,7 +490,7 @@ class ModelRunner:
             logits = self._mixed_step_with_graph(entries, greedy)
         if logits is None:                         # (also a shape that is not recorded yet)
             ctx = self.build_context(entries)
-            self._clear_state_of_new_requests(ctx.seqs)
+            self._begin_new_requests(ctx.seqs)
             logits = self.model.forward(ctx, self.bindings)
             if greedy:
                 logits = ops.argmax(logits).tolist() if logits.shape[0] else []
@@ -505,7 +515,7 @@ class ModelRunner:
         seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._single_token_layout(entries)
         self._check_bounds(seqs, slots, upd_idx, upd_val)
         self._poison_pages()                       # (the pages just handed out, before anything is written)
-        self._clear_state_of_new_requests(seqs)
+        self._begin_new_requests(seqs)
         n_live, n_groups = len(seqs), len(self.cache.groups)
         i32 = np.int32
         # Graphs are recorded for 1 to 8 rows, for multiples of 8 and, beyond 64, of 32: a batch in between is filled up
@@ -587,6 +597,7 @@ class ModelRunner:
         seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout(ordered, tokens)
         self._check_bounds(seqs, slots, upd_idx, upd_val)
         self._poison_pages()
+        self._begin_new_requests(seqs)
         fill, pad = B - n_dec, T - T1
         spare = self.spare_row
 
@@ -670,7 +681,8 @@ class ModelRunner:
         seqs = [SeqInfo(None, i, 1, 0, self.spare_row, False) for i in range(B)] + \
             [SeqInfo(None, B, T, 0, self.spare_row, False)]
         ctx = StepContext(rt=self.rt, page_size=self.page_size, num_tokens=B + T, seqs=seqs, token_ids=d_tok,
-                          positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
+                          positions=d_pos, tok_seq=d_seq, block_tables=self.tables,
+                          shared_keys=self.shared_keys, slots=d_slots,
                           logit_rows=d_rows, state_slots=d_state, max_position=0,
                           extras={cls: dict(cls.mixed_graph_extras(B, T, k, dev, dyn))
                                   for cls, k, dyn in zip(self._step_classes, part_keys, d_dyn)})
@@ -713,7 +725,7 @@ class ModelRunner:
         seqs, token_ids, positions, tok_seq, rows, slots, upd_idx, upd_val = self._layout([entry], tokens)
         self._check_bounds(seqs, slots, upd_idx, upd_val)
         self._poison_pages()
-        self._clear_state_of_new_requests(seqs)
+        self._begin_new_requests(seqs)
         if any(len(u) > cap for u in upd_idx):
             for g in range(n_groups):
                 if len(upd_idx[g]):
@@ -764,7 +776,8 @@ class ModelRunner:
             d_upd.append((take(cap), take(cap)))
         seqs = [SeqInfo(None, 0, T, 0, self.spare_row, False)]
         ctx = StepContext(rt=self.rt, page_size=self.page_size, num_tokens=T, seqs=seqs, token_ids=d_tok,
-                          positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
+                          positions=d_pos, tok_seq=d_seq, block_tables=self.tables,
+                          shared_keys=self.shared_keys, slots=d_slots,
                           logit_rows=d_rows, state_slots=d_state, max_position=0,
                           extras={cls: dict(cls.portion_graph_extras(T, dev) if k is None
                                             else cls.portion_graph_extras(T, dev, k))
@@ -820,7 +833,8 @@ class ModelRunner:
             d_upd.append((take(cap), take(cap)))
         seqs = [SeqInfo(None, i, 1, 0, 0, False) for i in range(B)]
         ctx = StepContext(rt=self.rt, page_size=self.page_size, num_tokens=B, seqs=seqs, token_ids=d_tok,
-                          positions=d_pos, tok_seq=d_seq, block_tables=self.tables, slots=d_slots,
+                          positions=d_pos, tok_seq=d_seq, block_tables=self.tables,
+                          shared_keys=self.shared_keys, slots=d_slots,
                           logit_rows=d_rows, state_slots=d_state, max_position=0,
                           extras={cls: dict(cls.graph_extras(B, k, dev)) if hasattr(cls, "graph_extras") else {}
                                   for cls, k in zip(self._step_classes, part_keys)})

@@ -186,10 +186,12 @@ class Scheduler:
             # few large steps (8192 tokens: four steps instead of sixteen, 1.7 times sooner).
             # Several prompts at once share the budget in equal parts of at least the portion limit, so that a
             # long prompt does not hold a short one that arrived with it back until it is through.
+            # What the shares leave over (a prompt shorter than its share, a request that waits for pages which
+            # another is still computing) goes to the planned prompts that can use it, oldest first.
             with_prompt = sum(1 for r in self.running if r.num_known - r.num_computed > 1) + len(self.waiting)
             shares = max(1, min(with_prompt, self.max_step_tokens // self.prefill_chunk))
-            chunk = self.prefill_chunk if any(r.num_known - r.num_computed == 1 for r in self.running) \
-                else max(self.prefill_chunk, self.max_step_tokens // shares)
+            decoding = any(r.num_known - r.num_computed == 1 for r in self.running)
+            chunk = self.prefill_chunk if decoding else max(self.prefill_chunk, self.max_step_tokens // shares)
             # pages the entries planned so far need, per group: an entry fits if its own pages fit
             # beside them (the same answer as cache.can_reserve on the whole list, without going
             # through the list again for every candidate)
@@ -264,6 +266,22 @@ class Scheduler:
                 planned.append(Planned(r, r.known_span(start, n), sample=(start + n == r.num_known)))
                 budget -= n
             self.waiting.extendleft(reversed(held))            # back to the front, in their order
+            if budget > 0 and not decoding:
+                for i, p in enumerate(planned):
+                    r = p.request
+                    end = r.num_computed + len(p.tokens)
+                    more = min(r.num_known - end, budget)
+                    if more <= 0:
+                        continue
+                    had = self.cache.pages_needed(r.req_id, end)
+                    need = self.cache.pages_needed(r.req_id, end + more)
+                    if any(taken[g] + need[g] - had[g] > self.cache.available(g) for g in groups):
+                        continue
+                    for g in groups:
+                        taken[g] += need[g] - had[g]
+                    planned[i] = Planned(r, r.known_span(r.num_computed, len(p.tokens) + more),
+                                         sample=(end + more == r.num_known))
+                    budget -= more
             if not planned and self.waiting and not self.running:
                 # nothing runs and the first waiting request cannot start: it can never start
                 r = self.waiting.popleft()

@@ -67,8 +67,8 @@ def load_library():
         "qe_attention_prefill_plan": [i32, i32, i32, i32],
         "qe_attention_prefill_plan_uncut_keys": [],
         "qe_attention_prefill_workspace_bytes": [i32, i32, i32, i32, i32, i32],
-        "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
-        "qe_attention_decode_fused_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, f32, vp,
+        "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
+        "qe_attention_decode_fused_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, vp, f32, vp,
                                           i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
         "qe_qk_rope_store": [vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_qk_rope_store_parts": [vp, i32, vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, vp],
@@ -578,7 +578,7 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
               other_tokens: Optional[torch.Tensor] = None,
               other_tiles: Optional[torch.Tensor] = None, prefill_groups: int = 0,
               max_other_keys: int = 0, prefill_segment_keys: int = -1,
-              other_keys_row: Optional[int] = None) -> torch.Tensor:
+              other_keys_row: Optional[int] = None, shared_keys: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [T, Hq, D]; cache [pages, 2, Hkv, P, D] (key tiles [P][D], value tiles transposed [D][P]);
     positions, tok_seq int32 [T]; block_table int32 [B, max_blocks].  Token t sees the keys at
     positions max(0, p - window + 1) .. p of request tok_seq[t] (window 0: all).  The caller
@@ -594,7 +594,10 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
     their length, a multiple of 64; 0 for none; -1 to let it choose).  A caller that does not know
     the positions (a recorded step) names the row of q that sees the most keys instead
     (other_keys_row): the kernel then cuts by that row's position.
-    Without the lists every row is treated alike."""
+    Without the lists every row is treated alike.
+
+    shared_keys (int32, an entry per row of block_table, or None): how many of a request's first keys
+    other requests read too.  A hint for the decode kernel's loads; results do not depend on it."""
     lib = load_library()
     _need(q, "q", _ACT, (None, None, None))
     T, Hq, D = q.shape
@@ -610,6 +613,8 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
     if Hq % Hkv:
         raise KernelError(f"attention: {Hq} query heads are no multiple of {Hkv} key/value heads")
     max_blocks = block_table.shape[1]
+    if shared_keys is not None:
+        _need(shared_keys, "shared_keys", torch.int32, (block_table.shape[0],), dev)
 
     def generic(tokens):
         n = T if tokens is None else tokens.shape[0]
@@ -628,7 +633,8 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
             ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
             _check(lib.qe_attention_decode_run(q.data_ptr(), out.data_ptr(), cache.data_ptr(),
                                                dec_tokens.data_ptr(), n_dec, positions.data_ptr(),
-                                               tok_seq.data_ptr(), block_table.data_ptr(), max_blocks, Hq, Hkv,
+                                               tok_seq.data_ptr(), block_table.data_ptr(), max_blocks,
+                                               _ptr(shared_keys), Hq, Hkv,
                                                D, P, float(scale), int(window), int(max_dec_position),
                                                DECODE_SPLIT_KEYS, ws.data_ptr(), nbytes, _stream()),
                    "attention (decode)")
@@ -686,13 +692,14 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, cache: torch.Tenso
                            dec_tokens: Optional[torch.Tensor], max_dec_position: int,
                            q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                            table: Optional[torch.Tensor], slots: Optional[torch.Tensor],
-                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           out: Optional[torch.Tensor] = None,
+                           shared_keys: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of single new tokens with the step before it inside: per-head q/k RMSNorm
     (weights or None), half-split rotation from ``table`` (rows [cos | sin] of the head size, or
     None) and the write of each token's key and value to cache slot ``slots[t]`` (negative or no
     slots: not written).  qkv [T, (Hq + 2 Hkv) D] bfloat16; the rows ``dec_tokens`` (None: all
     rows) are computed into out [T, Hq, D]; the cache holds each request's keys before the
-    token's own position."""
+    token's own position.  shared_keys: as for attention()."""
     lib = load_library()
     _need(qkv, "qkv", torch.bfloat16, (None, None))
     T, dev = qkv.shape[0], qkv.device
@@ -716,6 +723,8 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, cache: torch.Tenso
         _need(table, "table", torch.float32, (None, D), dev)
     if slots is not None:
         _need(slots, "slots", torch.int32, (T,), dev)
+    if shared_keys is not None:
+        _need(shared_keys, "shared_keys", torch.int32, (block_table.shape[0],), dev)
     if out is None:
         out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=dev)
     _need(out, "out", torch.bfloat16, (T, Hq, D), dev)
@@ -726,7 +735,8 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, cache: torch.Tenso
     ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
     _check(lib.qe_attention_decode_fused_run(qkv.data_ptr(), out.data_ptr(), cache.data_ptr(), _ptr(dec_tokens),
                                              n_dec, positions.data_ptr(), tok_seq.data_ptr(), block_table.data_ptr(),
-                                             block_table.shape[1], _ptr(slots), _ptr(q_weight), _ptr(k_weight),
+                                             block_table.shape[1], _ptr(shared_keys), _ptr(slots), _ptr(q_weight),
+                                             _ptr(k_weight),
                                              float(eps), _ptr(table), Hq, Hkv, D, P, float(scale), int(window),
                                              int(max_dec_position), DECODE_SPLIT_KEYS, ws.data_ptr(), nbytes,
                                              _stream()), "attention (decode, fused)")

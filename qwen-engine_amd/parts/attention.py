@@ -244,7 +244,8 @@ class PagedAttention:
                 # happen inside the attention kernel
                 o = ops.attention_decode_fused(qkv, self.hq, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g],
                                                self.scale, self.window, None, ex["max_dec_position"],
-                                               self.q_norm, self.k_norm, eps, table, slots)
+                                               self.q_norm, self.k_norm, eps, table, slots,
+                                               shared_keys=ctx.shared_keys)
                 return self._project_out(o.view(T, self.hq * self.d))
             q = ops.qk_rope_store(qkv, self.hq, self.hkv, self.d, ctx.positions, self.q_norm, self.k_norm,
                                   eps, table, slots, cache, ctx.page_size)
@@ -264,7 +265,8 @@ class PagedAttention:
                           dec_tokens=ex["dec_tokens"], max_dec_position=ex["max_dec_position"],
                           other_tokens=ex["other_tokens"],
                           other_tiles=self._other_tiles(ctx) if ex["other_tokens"] is not None else None,
-                          max_other_keys=ex.get("max_other_keys", 0), other_keys_row=ex.get("other_keys_row"))
+                          max_other_keys=ex.get("max_other_keys", 0), other_keys_row=ex.get("other_keys_row"),
+                          shared_keys=ctx.shared_keys)
         return self._project_out(o.view(T, self.hq * self.d))
 
     def _project_out(self, o: torch.Tensor) -> torch.Tensor:

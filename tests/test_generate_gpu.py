@@ -122,6 +122,12 @@ def test_shared_prefix_pages_are_taken_over(folders):
     assert eng.stats()["shared_prefix_tokens"] == 32
     assert res[0].token_ids == P.greedy_generate(cfg, w, a, 4)
     assert res[1].token_ids == P.greedy_generate(cfg, w, b, 4)
+    # the kernels were told which request read keys of another's pages (its row of the device tables)
+    assert sorted(eng.runner.shared_keys.tolist()) == [0, 0, 32]
+    # a request without a shared prefix that takes the same row over is told so as well
+    eng.submit([[1, 2, 3]] * 2, max_new_tokens=2, ignore_eos=True)
+    eng.run()
+    assert eng.runner.shared_keys.tolist() == [0, 0, 0]
 
 
 def test_temperature_sampling_equals_the_plain_draw(folders):

@@ -552,6 +552,14 @@ def test_decode_attention_kernel(ops, hq, hkv, d, page, window):
     out2 = ops.attention(qd, cd, i32(positions), i32(list(range(B))), table.to(DEV), scale, window=window,
                          dec_tokens=i32([5, 1, 3]), max_dec_position=700, other_tokens=i32([0, 2, 4]))
     close(out2, torch.cat(want), bf)
+    # the hint that some requests' first keys are read by others chooses between two kinds of loads: the same bits
+    out3 = ops.attention(qd, cd, i32(positions), i32(list(range(B))), table.to(DEV), scale, window=window,
+                         dec_tokens=i32(list(range(B))), max_dec_position=max(positions),
+                         shared_keys=i32([0, 16, 0, 64, 129, 300]))
+    assert torch.equal(out3, out)
+    with pytest.raises(ops.KernelError):                      # an entry per row of the table
+        ops.attention(qd, cd, i32(positions), i32(list(range(B))), table.to(DEV), scale, window=window,
+                      dec_tokens=i32(list(range(B))), max_dec_position=max(positions), shared_keys=i32([0, 16]))
 
 
 @pytest.mark.parametrize("hq,hkv,d,page", [(16, 8, 128, 16), (4, 4, 64, 16), (8, 1, 128, 32), (6, 2, 64, 48), (16, 1, 64, 16)])
@@ -641,6 +649,11 @@ def test_decode_attention_with_norm_rotation_and_cache_write_inside(ops, hq, hkv
     out3 = ops.attention_decode_fused(qkv.to(DEV), hq, cache.to(DEV), i32(positions), i32(list(range(B))), tab.to(DEV),
                                       scale, window, None, max(positions), dev(qw), dev(kw), eps, dev(table), i32(slots))
     assert torch.equal(out3, out)
+    # ... and with the hint that other requests read some requests' first keys too (another kind of load there)
+    out4 = ops.attention_decode_fused(qkv.to(DEV), hq, cache.to(DEV), i32(positions), i32(list(range(B))), tab.to(DEV),
+                                      scale, window, None, max(positions), dev(qw), dev(kw), eps, dev(table), i32(slots),
+                                      shared_keys=i32([(64 * b) % 200 for b in range(B)]))
+    assert torch.equal(out4, out)
 
 
 @pytest.mark.parametrize("key_pos", [0, 15, 16, 127, 128, 255, 256, 1000, 1023])

@@ -142,7 +142,8 @@ def test_prompts_that_arrive_together_share_the_budget():
     sched.add(short)
     log = []
     drive(sched, cache, log)
-    assert log[0] == [(0, 16, False), (1, 5, True)]          # two prompts: half the budget each at most
+    # two prompts: half the budget each; what the short one leaves of its half goes to the long one
+    assert log[0] == [(0, 16 + 11, False), (1, 5, True)]
     assert log[1][0] == (0, 8, False)                          # the short one decodes now: portions of the limit
     assert long.output == expected_output(long.prompt, 2) and short.output == expected_output(short.prompt, 2)
     # three prompts and a budget of four portions: a third of the budget each, rounded down, at least a portion
@@ -150,7 +151,23 @@ def test_prompts_that_arrive_together_share_the_budget():
     for i in range(3):
         sched.add(Request(i, list(range(3, 103)), SamplingParams(max_new_tokens=1)))
     planned = sched.plan()
-    assert [(p.request.req_id, len(p.tokens)) for p in planned] == [(0, 10), (1, 10), (2, 10)]
+    assert [(p.request.req_id, len(p.tokens)) for p in planned] == [(0, 10 + 2), (1, 10), (2, 10)]
+    # requests that wait for pages which the first is still computing take no share: the first gets the budget
+    common = list(range(3, 43))
+    sched, cache = make(num_pages=400, budget=32, chunk=8, max_model_len=400, max_num_seqs=4, sharing=True)
+    for i in range(4):
+        sched.add(Request(i, common + [50 + i], SamplingParams(max_new_tokens=1)))
+    planned = sched.plan()
+    assert [(p.request.req_id, len(p.tokens)) for p in planned] == [(0, 32)]
+    assert sched.stats["held_back_for_prefix"] == 3
+    # a top-up that has no pages is left out: 10 pages of 4 tokens, two prompts of 36 and shares of 24 (the
+    # second's made smaller until it fits: 6 + 3 pages), 12 tokens of the budget left and one page
+    sched, cache = make(num_pages=10, budget=48, chunk=8, max_model_len=64, max_num_seqs=2)
+    for i in range(2):
+        sched.add(Request(i, list(range(3, 39)), SamplingParams(max_new_tokens=1)))
+    planned = sched.plan()
+    assert [(p.request.req_id, len(p.tokens)) for p in planned] == [(0, 24), (1, 12)]
+    assert cache.can_reserve([(p.request.req_id, p.request.num_computed + len(p.tokens)) for p in planned])
 
 
 def test_a_first_portion_of_the_whole_budget_that_does_not_fit_is_made_smaller():
