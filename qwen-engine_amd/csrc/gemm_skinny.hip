@@ -205,14 +205,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     const bf16_t* x = (const bf16_t*)x_in;
     const int KP = K + 8;                                            // padded row of the normed copy
 
-    floatx4 acc[NT][NW][MT];
-#pragma unroll
-    for (int q = 0; q < NT; ++q)
-#pragma unroll
-        for (int a = 0; a < NW; ++a)
-#pragma unroll
-            for (int j = 0; j < MT; ++j) acc[q][a][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-
     bool row_ok[NT];
     const bf16_t* wrow0[NT];
     const bf16_t* wrow1[NT];
@@ -235,54 +227,155 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     }
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-    // The weights of the first round are asked for before the prologue: they come from HBM and do
-    // not depend on it, so the norm runs while they travel.
-    bf16x8 a0[U][NT], a1[U][NT];
-    int c = c_begin + wave;
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    // How the chunks of K are dealt to the waves: in pairs (wave w takes the chunks 2 w and 2 w + 1, then those
+    // 2 WAVES further on), so that a wave's two loads of a row are one line of 128 bytes: the q|k|v and down
+    // products of the large models go 8 % faster than with single chunks dealt round the waves, where two
+    // waves fetch a line's halves at different times.  With silu.mul (eight waves, two matrices) single chunks
+    // are faster.  A wave's chunks do not depend on how many it takes a round or on the rows of x: a row's sums
+    // are added in the same order whatever else is in the batch.
+    constexpr bool PAIRS = !SILU;
+    static_assert(!PAIRS || U % 2 == 0, "chunks are dealt in pairs");
+#define QE_CHUNK(c_, u) (PAIRS ? (c_) + 2 * WAVES * ((u) >> 1) + ((u) & 1) : (c_) + WAVES * (u))
+#define QE_MFMA(acc_, a0_, a1_, b_)                                                                    \
+    _Pragma("unroll") for (int q = 0; q < NT; ++q) {                                                   \
+        acc_[q][0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0_[u][q], b_, acc_[q][0][j], 0, 0, 0); \
+        if (SILU) acc_[q][1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1_[u][q], b_, acc_[q][1][j], 0, 0, 0); \
+    }
+#define QE_KEEP(acc_)                                                                                  \
+    _Pragma("unroll") for (int q = 0; q < NT; ++q)                                                     \
+        _Pragma("unroll") for (int a = 0; a < NW; ++a)                                                 \
+            _Pragma("unroll") for (int j = 0; j < MT; ++j)                                             \
+                _Pragma("unroll") for (int i = 0; i < 4; ++i) red[wave][q][a][j][lane][i] = acc_[q][a][j][i];
+#define QE_NORM_PROLOGUE()                                                                             \
+    norm_rows_into_lds<WAVES>((const float*)x_in, delta, n_delta, (blockIdx.x == 0 && blockIdx.y == 0) ? h_out : nullptr, \
+                              norm_w, norm_eps, (bf16_t*)dyn_lds, M, K, KP);
+    const int last = c_end - 1;
+    // Three forms of the main part: with the norm as prologue, for a block whose waves have one round of
+    // chunks at most, and for several rounds.  Each leaves its sums in shared memory itself: the
+    // accumulators of two forms never meet in one register.
+#define QE_ZERO(acc_)                                                                                  \
+    _Pragma("unroll") for (int q = 0; q < NT; ++q)                                                     \
+        _Pragma("unroll") for (int a = 0; a < NW; ++a)                                                 \
+            _Pragma("unroll") for (int j = 0; j < MT; ++j) acc_[q][a][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // (loads that stand under their own conditions: a wave with few chunks asks for no more than it has)
 #define QE_LOAD_W()                                                                                    \
     _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                    \
-        const int cc = c + WAVES * u;                                                                  \
-        const bool ok = cc < c_end;                                                                    \
+        const int cc = QE_CHUNK(c, u);                                                                 \
+        const bool ok = cc <= last;                                                                    \
         _Pragma("unroll") for (int q = 0; q < NT; ++q) {                                               \
             a0[u][q] = (ok && row_ok[q]) ? *(const bf16x8*)(wrow0[q] + cc * 32) : zero;                \
             if (SILU) a1[u][q] = (ok && row_ok[q]) ? *(const bf16x8*)(wrow1[q] + cc * 32) : zero;      \
         }                                                                                              \
     }
-    if (c < c_end) { QE_LOAD_W() }
-    if (NORM)
-        norm_rows_into_lds<WAVES>((const float*)x_in, delta, n_delta, (blockIdx.x == 0 && blockIdx.y == 0) ? h_out : nullptr,
-                                  norm_w, norm_eps, (bf16_t*)dyn_lds, M, K, KP);
-    while (c < c_end) {
-        bf16x8 b[U][MT];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int cc = c + WAVES * u;
-            const bool ok = cc < c_end;
-#pragma unroll
-            for (int j = 0; j < MT; ++j) b[u][j] = (ok && tok_ok[j]) ? *(const bf16x8*)(xrow[j] + cc * 32) : zero;
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int q = 0; q < NT; ++q)
-#pragma unroll
-                for (int j = 0; j < MT; ++j) {
-                    acc[q][0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[u][q], b[u][j], acc[q][0][j], 0, 0, 0);
-                    if (SILU)
-                        acc[q][1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[u][q], b[u][j], acc[q][1][j], 0, 0, 0);
-                }
-        c += WAVES * U;
-        if (c < c_end) { QE_LOAD_W() }
+#define QE_ROUND()                                                                                     \
+    {                                                                                                  \
+        bf16x8 b[U][MT];                                                                               \
+        _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                \
+            const int cc = QE_CHUNK(c, u);                                                             \
+            const bool ok = cc <= last;                                                                \
+            _Pragma("unroll") for (int j = 0; j < MT; ++j)                                             \
+                b[u][j] = (ok && tok_ok[j]) ? *(const bf16x8*)(xrow[j] + cc * 32) : zero;              \
+        }                                                                                              \
+        _Pragma("unroll") for (int u = 0; u < U; ++u)                                                  \
+            _Pragma("unroll") for (int j = 0; j < MT; ++j) { QE_MFMA(acc, a0, a1, b[u][j]) }           \
     }
+    if (NORM) {
+        // The norm as prologue (small matrices): the first round's weights travel while the rows are normed;
+        // further rounds, if any, one after the other.
+        floatx4 acc[NT][NW][MT];
+        QE_ZERO(acc)
+        bf16x8 a0[U][NT], a1[U][NT];
+        int c = c_begin + (PAIRS ? 2 : 1) * wave_s;
+        if (c <= last) { QE_LOAD_W() }
+        QE_NORM_PROLOGUE()
+        while (c <= last) {
+            QE_ROUND()
+            c += WAVES * U;
+            if (c <= last) { QE_LOAD_W() }
+        }
+        QE_KEEP(acc)
+    } else if (c_end - c_begin <= WAVES * U) {
+        // One round at most a wave (the small model's products).
+        floatx4 acc[NT][NW][MT];
+        QE_ZERO(acc)
+        bf16x8 a0[U][NT], a1[U][NT];
+        const int c = c_begin + (PAIRS ? 2 : 1) * wave_s;
+        QE_LOAD_W()
+        QE_ROUND()
+        QE_KEEP(acc)
+        asm volatile("" ::: "memory");             // (so that this way does not end like the next: see there)
+    } else {
+        // Several rounds: the next round's weights and rows are asked for before the current round is
+        // multiplied (two sets of registers used in turn), so a wave always has a round on its way.  No load
+        // stands under a condition here (the compiler would wait for every load in flight behind one): a
+        // chunk beyond the wave's last reads the last chunk's place instead, and its rows of x count as
+        // zeros.
+        floatx4 acc[NT][NW][MT];
+        QE_ZERO(acc)
+        bf16x8 a0[2][U][NT], a1[2][U][NT], b[2][U][MT];
+        int c = c_begin + (PAIRS ? 2 : 1) * wave_s;
+#define QE_LOAD(s_, c_)                                                                                \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                    \
+        const int cc = min(QE_CHUNK(c_, u), last);                                                     \
+        _Pragma("unroll") for (int q = 0; q < NT; ++q) {                                               \
+            a0[s_][u][q] = *(const bf16x8*)(wrow0[q] + cc * 32);                                       \
+            if (SILU) a1[s_][u][q] = *(const bf16x8*)(wrow1[q] + cc * 32);                             \
+        }                                                                                              \
+    }
+#define QE_LOAD_X(s_, c_)                                                                              \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                    \
+        const int cc = min(QE_CHUNK(c_, u), last);                                                     \
+        _Pragma("unroll") for (int j = 0; j < MT; ++j) b[s_][u][j] = *(const bf16x8*)(xrow[j] + cc * 32); \
+    }
+#define QE_MULTIPLY(s_, c_)                                                                            \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                    \
+        const bool ok = QE_CHUNK(c_, u) <= last;                                                       \
+        _Pragma("unroll") for (int j = 0; j < MT; ++j) {                                               \
+            const bf16x8 bb = ok ? b[s_][u][j] : zero;                                                 \
+            QE_MFMA(acc, a0[s_], a1[s_], bb)                                                           \
+        }                                                                                              \
+    }
+        const int rounds = c <= last ? (last - c) / (WAVES * U) + 1 : 1;     // of this wave: the same in all its lanes
+        QE_LOAD(0, c)
+        QE_LOAD_X(0, c)
+        for (int p = (rounds - 1) >> 1; p > 0; --p) {          // while three rounds or more are left: two of them
+            QE_LOAD(1, c + WAVES * U)
+            QE_LOAD_X(1, c + WAVES * U)
+            QE_MULTIPLY(0, c)
+            c += WAVES * U;
+            QE_LOAD(0, c + WAVES * U)
+            QE_LOAD_X(0, c + WAVES * U)
+            QE_MULTIPLY(1, c)
+            c += WAVES * U;
+        }
+        // one round or two are left.  Each way leaves its sums in shared memory itself, and the two ways do not
+        // end alike (the empty statement), so that the compiler does not join them behind the branch: joined,
+        // the accumulators of the two ways would meet in one register, and this compiler's copies for that have
+        // overwritten operands that were still to be multiplied (seen with two tiles of rows).
+        if (rounds & 1) {
+            QE_MULTIPLY(0, c)
+            QE_KEEP(acc)
+        } else {
+            QE_LOAD(1, c + WAVES * U)
+            QE_LOAD_X(1, c + WAVES * U)
+            QE_MULTIPLY(0, c)
+            c += WAVES * U;
+            QE_MULTIPLY(1, c)
+            QE_KEEP(acc)
+            asm volatile("" ::: "memory");
+        }
+#undef QE_LOAD
+#undef QE_LOAD_X
+#undef QE_MULTIPLY
+    }
+#undef QE_MFMA
+#undef QE_KEEP
+#undef QE_ZERO
 #undef QE_LOAD_W
-#pragma unroll
-    for (int q = 0; q < NT; ++q)
-#pragma unroll
-        for (int a = 0; a < NW; ++a)
-#pragma unroll
-            for (int j = 0; j < MT; ++j)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) red[wave][q][a][j][lane][i] = acc[q][a][j][i];
+#undef QE_ROUND
+#undef QE_NORM_PROLOGUE
+#undef QE_CHUNK
     __syncthreads();
     // wave w finishes the (output tile, token tile) pairs w, w + WAVES, ...: the waves' sums in their order
     for (int qj = wave; qj < NT * MT; qj += WAVES) {

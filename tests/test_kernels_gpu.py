@@ -492,6 +492,40 @@ def test_gemm_for_few_rows(ops, M, N, K):
     close(normed, P.rms_norm(total.float(), nw, 1e-6), bf)
 
 
+@pytest.mark.parametrize("N", [48, 8192])
+@pytest.mark.parametrize("K", [512, 1536, 2048, 2560, 5120])
+def test_gemm_for_few_rows_over_rounds_of_chunks(ops, N, K):
+    """The kernel for few rows has a form for blocks whose waves read their chunks of K in one round and a form
+    that runs several rounds with the next round's loads in flight (pairs of rounds, then one or two): K from
+    one round to five or more, with and without a cut along K, for one to four tiles of 16 rows of x and for
+    one and two tiles of outputs a block; silu.mul in both layouts of gate and up.  In 64-bit on drawn columns."""
+    bf = torch.bfloat16
+    g = torch.Generator().manual_seed(1000 * N + K)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(bf)
+    wd = w.to(DEV)
+    cols = torch.randint(0, N, (192,), generator=g) if N > 192 else torch.arange(N)
+    wc, cd = w[cols].double(), cols.to(DEV)
+    half = N // 2
+    w_il = ops.interleave_gate_up(wd[:half], wd[half:]) if half % 32 == 0 else None
+    for M in (1, 8, 16, 17, 32, 33, 49, 64):
+        x = torch.randn(M, K, generator=g).to(bf)
+        xd = x.to(DEV)
+        want = x.double() @ wc.t()
+        scale = float(want.abs().max())
+        got = ops.gemm(xd, wd, out_dtype=torch.float32, algo=ops.ALGO_FAST)[:, cd]
+        assert float((got.double().cpu() - want).abs().max()) <= 3e-6 * scale, ("store", M)
+        for splits in (2, 3):
+            parts = ops.gemm(xd, wd, epilogue=ops.EPI_PARTIAL, splits=splits)
+            assert float((parts.sum(0)[:, cd].double().cpu() - want).abs().max()) <= 3e-6 * scale, ("partial", splits, M)
+        gu = x.double() @ w.double().t()
+        want_g = P.silu_mul(gu[:, :half], gu[:, half:])
+        got = ops.gemm(xd, wd, epilogue=ops.EPI_SILU_MUL, out_dtype=torch.float32)
+        assert float((got.double().cpu() - want_g).abs().max()) <= 1e-5 * float(want_g.abs().max()), ("silu", M)
+        if w_il is not None and ops.gemm_silu_supported(xd, w_il):
+            got = ops.gemm(xd, w_il, epilogue=ops.EPI_SILU_MUL_IL, out_dtype=torch.float32)
+            assert float((got.double().cpu() - want_g).abs().max()) <= 1e-5 * float(want_g.abs().max()), ("silu, interleaved", M)
+
+
 @pytest.mark.parametrize("M", [1, 8, 40, 64])
 @pytest.mark.parametrize("I,K", [(160, 96), (112, 64), (3072, 1024)])
 def test_gemm_with_silu_mul(ops, M, I, K):
