@@ -280,15 +280,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
         _Pragma("unroll") for (int u = 0; u < U; ++u)                                                  \
             _Pragma("unroll") for (int j = 0; j < MT; ++j) { QE_MFMA(acc, a0, a1, b[u][j]) }           \
     }
-    if (NORM) {
+    if (NORM || NT == 4) {
         // The norm as prologue (small matrices): the first round's weights travel while the rows are normed;
-        // further rounds, if any, one after the other.
+        // further rounds, if any, one after the other.  Four tiles of outputs a block (the logits' matrix) run
+        // this way too: a round is 16 KB of weights a wave already, and the second set of registers only cost
+        // (eight rows against the 8B sizes' logits: 241 us this way, 255 with two rounds in flight).
         floatx4 acc[NT][NW][MT];
         QE_ZERO(acc)
         bf16x8 a0[U][NT], a1[U][NT];
         int c = c_begin + (PAIRS ? 2 : 1) * wave_s;
         if (c <= last) { QE_LOAD_W() }
-        QE_NORM_PROLOGUE()
+        if (NORM) { QE_NORM_PROLOGUE() }
         while (c <= last) {
             QE_ROUND()
             c += WAVES * U;
@@ -435,9 +437,11 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
     // two tiles of outputs a block where the activations have more than 16 rows and there are blocks
     // enough all the same (with silu.mul a tile of outputs is two tiles of W already: only up to 32 rows)
     const bool two = mt >= 2 && (!SILU || mt <= 2) && (long)qe_cdiv(N, 32) * splits >= 256;
-    // ... and four where 2 to 16 rows meet a matrix of very many rows (the logits'): with 8 rows the
-    // activations are then an eighth of what a block reads instead of a third
-    const bool four = !SILU && mt == 1 && M > 1 && (long)qe_cdiv(N, 64) * splits >= 2048;
+    // ... and four where 9 to 16 rows meet a matrix of very many rows (the logits'): the activations are
+    // then a ninth of what a block reads instead of a third (16 rows against the 8B sizes' logits: 266 us
+    // against 289; up to 8 rows one tile a block with two rounds in flight is as fast or faster: 236
+    // against 245 us with eight rows, 200 against 239 with two)
+    const bool four = !SILU && mt == 1 && M > 8 && (long)qe_cdiv(N, 64) * splits >= 2048;
     const dim3 grid(qe_cdiv(N, four ? 64 : (two ? 32 : 16)), splits);
 #define QE_SKINNY_W(MT_, NT_, WAVES_, NORM_)                                                           \
     do {                                                                                               \

@@ -122,10 +122,10 @@ def test_single_tokens_beside_a_portion_deep_in_a_context(model_and_refs, n_dec,
 
 @pytest.mark.parametrize("K", [4096, 5120])
 def test_head_product_at_the_large_widths_against_the_whole_vocabulary(K):
-    """logits = x . W^T with W [151 936, K] (src/models/qwen3/model.py:369-373,422), float32 out, for 1, 8
-    and 64 rows of a decode step at the 8B and 32B widths (2 to 16 rows: four tiles of outputs a block of
-    the kernel for few rows; 17 to 64: the tiled kernel): compared in 64-bit on 3000 drawn columns and the
-    last 100."""
+    """logits = x . W^T with W [151 936, K] (src/models/qwen3/model.py:369-373,422), float32 out, for 1, 8, 16
+    and 64 rows of a decode step at the 8B and 32B widths (up to 8 rows: one tile of outputs a block of the
+    kernel for few rows, several rounds of chunks with the next in flight; 9 to 16: four tiles a block; 17 to
+    64: the tiled kernel): compared in 64-bit on 3000 drawn columns and the last 100."""
     V = 151936
     g = torch.Generator().manual_seed(K)
     w = torch.empty(V, K, dtype=torch.bfloat16)
@@ -134,7 +134,7 @@ def test_head_product_at_the_large_widths_against_the_whole_vocabulary(K):
     w_dev = w.cuda()
     cols = torch.cat([torch.randint(0, V, (3000,), generator=g), torch.arange(V - 100, V)])
     w_cols = w[cols].double()
-    for rows in (1, 8, 64):
+    for rows in (1, 8, 16, 64):
         x = torch.randn(rows, K, generator=g).to(torch.bfloat16)
         got = ops.gemm(x.cuda(), w_dev, out_dtype=torch.float32).cpu()
         assert got.shape == (rows, V) and torch.isfinite(got).all()
