@@ -185,7 +185,7 @@ __device__ __forceinline__ void norm_rows_into_lds(const float* __restrict__ hs,
 // (M rows against the block's 16 NT rows of W), so with more than 16 rows of activations most of
 // what a block reads is activations, from the L2; two tiles a block halve that, four quarter it
 // (8 rows against the logits' matrix: 4.15 TB/s of weights with one tile a block, 6.07 with one row).
-template <int MT, int NT, int EPI, typename TO, int WAVES, bool NORM>
+template <int MT, int NT, int EPI, typename TO, int WAVES, bool NORM, bool LN = false, bool XH = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     const void* __restrict__ x_in, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TO* __restrict__ out, int M, int N, int K, int cps, const float* __restrict__ norm_w, float norm_eps,
@@ -231,12 +231,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     // How the chunks of K are dealt to the waves: in pairs (wave w takes the chunks 2 w and 2 w + 1, then those
     // 2 WAVES further on), so that a wave's two loads of a row are one line of 128 bytes: the q|k|v and down
     // products of the large models go 8 % faster than with single chunks dealt round the waves, where two
-    // waves fetch a line's halves at different times.  With silu.mul (eight waves, two matrices) single chunks
-    // are faster.  A wave's chunks do not depend on how many it takes a round or on the rows of x: a row's sums
-    // are added in the same order whatever else is in the batch.
-    constexpr bool PAIRS = !SILU;
-    static_assert(!PAIRS || U % 2 == 0, "chunks are dealt in pairs");
-#define QE_CHUNK(c_, u) (PAIRS ? (c_) + 2 * WAVES * ((u) >> 1) + ((u) & 1) : (c_) + WAVES * (u))
+    // waves fetch a line's halves at different times.  With silu.mul (eight waves, two matrices) a block whose
+    // waves have one round of chunks at most (the small model's) is faster with single chunks.  A wave's chunks
+    // depend on the matrix and the cut of K alone, not on the rows of x or on the form of the loop below: a
+    // row's sums are added in the same order whatever else is in the batch.
+    static_assert(U % 2 == 0, "chunks are dealt in pairs");
+    const bool pairs = !SILU || c_end - c_begin > WAVES * U;
+#define QE_CHUNK(c_, u) (pairs ? (c_) + 2 * WAVES * ((u) >> 1) + ((u) & 1) : (c_) + WAVES * (u))
 #define QE_MFMA(acc_, a0_, a1_, b_)                                                                    \
     _Pragma("unroll") for (int q = 0; q < NT; ++q) {                                                   \
         acc_[q][0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0_[u][q], b_, acc_[q][0][j], 0, 0, 0); \
@@ -288,7 +289,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
         floatx4 acc[NT][NW][MT];
         QE_ZERO(acc)
         bf16x8 a0[U][NT], a1[U][NT];
-        int c = c_begin + (PAIRS ? 2 : 1) * wave_s;
+        int c = c_begin + (pairs ? 2 : 1) * wave_s;
         if (c <= last) { QE_LOAD_W() }
         if (NORM) { QE_NORM_PROLOGUE() }
         while (c <= last) {
@@ -302,7 +303,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
         floatx4 acc[NT][NW][MT];
         QE_ZERO(acc)
         bf16x8 a0[U][NT], a1[U][NT];
-        const int c = c_begin + (PAIRS ? 2 : 1) * wave_s;
+        const int c = c_begin + (pairs ? 2 : 1) * wave_s;
         QE_LOAD_W()
         QE_ROUND()
         QE_KEEP(acc)
@@ -313,29 +314,102 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
         // stands under a condition here (the compiler would wait for every load in flight behind one): a
         // chunk beyond the wave's last reads the last chunk's place instead, and its rows of x count as
         // zeros.
+        //
+        // LN (one tile of rows of x, one of outputs; K in whole lines of 128 bytes): a load instruction takes whole
+        // lines, 8 lanes a row and 8 rows, of the weights and of x alike, instead of the 64 bytes a row that the
+        // MFMA operand layout would have 4 lanes take: the L1 then serves half as many requests, and the weights
+        // stream as fast beside 8 rows of x as beside one (a matrix of 1.2 GB: 6.3 TB/s where 64-byte pieces reach
+        // 5.5 with 8 rows and 4.6 with 16).  The registers go through a piece of shared memory of the wave's own to
+        // come out in the operand layout (written in the lanes' order, read by row and segment; the segments of a
+        // row stand swapped about by the row, so that neither side meets a bank twice).  Chunk by chunk the same
+        // products in the same order as without.
         floatx4 acc[NT][NW][MT];
         QE_ZERO(acc)
-        bf16x8 a0[2][U][NT], a1[2][U][NT], b[2][U][MT];
-        int c = c_begin + (PAIRS ? 2 : 1) * wave_s;
+        bf16x8 a0[LN ? 1 : 2][LN ? 1 : U][NT], a1[LN ? 1 : 2][LN ? 1 : U][NT], b[LN ? 1 : 2][LN ? 1 : U][MT];
+        constexpr int L = U / 2, XR = XH ? 2 : 1;                     // lines a round; load instructions a line of x
+        constexpr int LINE_BYTES = NW * 2048 + XR * 1024;
+        typedef __attribute__((ext_vector_type(4))) unsigned int u4;
+        u4 wreg[LN ? 2 : 1][LN ? L : 1][NW][2], xreg[LN ? 2 : 1][LN ? L : 1][XR];
+        unsigned char* scratch = dyn_lds + wave_s * LINE_BYTES;
+        const bf16_t* wl[NW][2];
+        const bf16_t* xlp[XR];
+        if (LN) {
+            static_assert(!LN || (MT == 1 && NT == 1 && !NORM), "whole lines: one tile of rows, one of outputs");
+            const int row8 = lane >> 3, pos = lane & 7;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int row = h * 8 + row8;
+                const int nrow = n0 + row < N ? n0 + row : 0;
+                const long wr = (EPI == EPI_SILU_MUL_IL) ? (long)(nrow >> 5) * 64 + (nrow & 31) : nrow;
+                wl[0][h] = w + wr * K + (pos ^ ((row >> 1) & 7)) * 8;
+                if (SILU) wl[NW - 1][h] = (EPI == EPI_SILU_MUL_IL) ? wl[0][h] + 32L * K : wl[0][h] + (long)N * K;
+            }
+#pragma unroll
+            for (int h = 0; h < XR; ++h) {
+                const int row = h * 8 + row8;
+                xlp[h] = x + (long)(row < M ? row : 0) * K + (pos ^ ((row >> 1) & 7)) * 8;
+            }
+        }
+        int c = c_begin + 2 * wave_s;                                 // (several rounds: always pairs)
 #define QE_LOAD(s_, c_)                                                                                \
-    _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                    \
-        const int cc = min(QE_CHUNK(c_, u), last);                                                     \
-        _Pragma("unroll") for (int q = 0; q < NT; ++q) {                                               \
-            a0[s_][u][q] = *(const bf16x8*)(wrow0[q] + cc * 32);                                       \
-            if (SILU) a1[s_][u][q] = *(const bf16x8*)(wrow1[q] + cc * 32);                             \
+    if (LN) {                                                                                          \
+        _Pragma("unroll") for (int i = 0; i < L; ++i) {                                                \
+            const int cc = min((c_) + 2 * WAVES * i, last & ~1);                                       \
+            _Pragma("unroll") for (int a = 0; a < NW; ++a)                                             \
+                _Pragma("unroll") for (int h = 0; h < 2; ++h)                                          \
+                    wreg[s_][i][a][h] = *(const u4*)(wl[a][h] + cc * 32);                              \
+        }                                                                                              \
+    } else {                                                                                           \
+        _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                \
+            const int cc = min(QE_CHUNK(c_, u), last);                                                 \
+            _Pragma("unroll") for (int q = 0; q < NT; ++q) {                                           \
+                a0[s_][u][q] = *(const bf16x8*)(wrow0[q] + cc * 32);                                   \
+                if (SILU) a1[s_][u][q] = *(const bf16x8*)(wrow1[q] + cc * 32);                         \
+            }                                                                                          \
         }                                                                                              \
     }
 #define QE_LOAD_X(s_, c_)                                                                              \
-    _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                    \
-        const int cc = min(QE_CHUNK(c_, u), last);                                                     \
-        _Pragma("unroll") for (int j = 0; j < MT; ++j) b[s_][u][j] = *(const bf16x8*)(xrow[j] + cc * 32); \
+    if (LN) {                                                                                          \
+        _Pragma("unroll") for (int i = 0; i < L; ++i) {                                                \
+            const int cc = min((c_) + 2 * WAVES * i, last & ~1);                                       \
+            _Pragma("unroll") for (int h = 0; h < XR; ++h) xreg[s_][i][h] = *(const u4*)(xlp[h] + cc * 32); \
+        }                                                                                              \
+    } else {                                                                                           \
+        _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                \
+            const int cc = min(QE_CHUNK(c_, u), last);                                                 \
+            _Pragma("unroll") for (int j = 0; j < MT; ++j) b[s_][u][j] = *(const bf16x8*)(xrow[j] + cc * 32); \
+        }                                                                                              \
     }
 #define QE_MULTIPLY(s_, c_)                                                                            \
-    _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                    \
-        const bool ok = QE_CHUNK(c_, u) <= last;                                                       \
-        _Pragma("unroll") for (int j = 0; j < MT; ++j) {                                               \
-            const bf16x8 bb = ok ? b[s_][u][j] : zero;                                                 \
-            QE_MFMA(acc, a0[s_], a1[s_], bb)                                                           \
+    if (LN) {                                                                                          \
+        _Pragma("unroll") for (int i = 0; i < L; ++i) {                                                \
+            const int cc = (c_) + 2 * WAVES * i;                                                       \
+            _Pragma("unroll") for (int a = 0; a < NW; ++a)                                             \
+                _Pragma("unroll") for (int h = 0; h < 2; ++h)                                          \
+                    *(u4*)(scratch + (a * 2 + h) * 1024 + lane * 16) = wreg[s_][i][a][h];              \
+            _Pragma("unroll") for (int h = 0; h < XR; ++h)                                             \
+                *(u4*)(scratch + NW * 2048 + h * 1024 + lane * 16) = xreg[s_][i][h];                   \
+            const int fr = (r >> 1) & 7, xr_ = XH ? r : (r & 7), fx = (xr_ >> 1) & 7;                  \
+            const unsigned char* xs = scratch + NW * 2048 + xr_ * 128;                                 \
+            const bf16x8 x0 = *(const bf16x8*)(xs + ((g ^ fx) * 16));                                  \
+            const bf16x8 x1 = *(const bf16x8*)(xs + (((g + 4) ^ fx) * 16));                            \
+            const bf16x8 b0 = cc <= last ? x0 : zero, b1 = cc + 1 <= last ? x1 : zero;                 \
+            _Pragma("unroll") for (int a = 0; a < NW; ++a) {                                           \
+                const bf16x8 w0 = *(const bf16x8*)(scratch + a * 2048 + r * 128 + ((g ^ fr) * 16));    \
+                acc[0][a][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, b0, acc[0][a][0], 0, 0, 0); \
+            }                                                                                          \
+            _Pragma("unroll") for (int a = 0; a < NW; ++a) {                                           \
+                const bf16x8 w1 = *(const bf16x8*)(scratch + a * 2048 + r * 128 + (((g + 4) ^ fr) * 16)); \
+                acc[0][a][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, b1, acc[0][a][0], 0, 0, 0); \
+            }                                                                                          \
+        }                                                                                              \
+    } else {                                                                                           \
+        _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                \
+            const bool ok = QE_CHUNK(c_, u) <= last;                                                   \
+            _Pragma("unroll") for (int j = 0; j < MT; ++j) {                                           \
+                const bf16x8 bb = ok ? b[s_][u][j] : zero;                                             \
+                QE_MFMA(acc, a0[s_], a1[s_], bb)                                                       \
+            }                                                                                          \
         }                                                                                              \
     }
         const int rounds = c <= last ? (last - c) / (WAVES * U) + 1 : 1;     // of this wave: the same in all its lanes
@@ -443,10 +517,12 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
     // against 245 us with eight rows, 200 against 239 with two)
     const bool four = !SILU && mt == 1 && M > 8 && (long)qe_cdiv(N, 64) * splits >= 2048;
     const dim3 grid(qe_cdiv(N, four ? 64 : (two ? 32 : 16)), splits);
-#define QE_SKINNY_W(MT_, NT_, WAVES_, NORM_)                                                           \
+#define QE_SKINNY_W(MT_, NT_, WAVES_, NORM_) QE_SKINNY_K(MT_, NT_, WAVES_, NORM_, false, false)
+#define QE_SKINNY_K(MT_, NT_, WAVES_, NORM_, LN_, XH_)                                                 \
     do {                                                                                               \
-        auto kern = gemm_skinny_kernel<MT_, NT_, EPI, TO, WAVES_, NORM_>;                              \
-        const size_t dyn = NORM_ ? norm_lds_bytes(M, K) : 0;                                           \
+        auto kern = gemm_skinny_kernel<MT_, NT_, EPI, TO, WAVES_, NORM_, LN_, XH_>;                    \
+        const size_t dyn = NORM_ ? norm_lds_bytes(M, K)                                                \
+                                 : (LN_ ? (size_t)WAVES_ * ((SILU ? 2 : 1) * 2048 + ((XH_) ? 2 : 1) * 1024) : 0); \
         if (dyn > 32 * 1024) {                                                                         \
             static bool raised = false;   /* (once per kernel: the limit of dynamic shared memory) */ \
             if (!raised) {                                                                             \
@@ -460,13 +536,23 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
                                                  delta, n_delta, h_out);                               \
     } while (0)
 #define QE_SKINNY(MT_, NT_) QE_SKINNY_W(MT_, NT_, 4, false)
+    // whole lines of K a load (see the kernel): up to 16 rows, one tile of outputs a block, several rounds of
+    // chunks a wave (blocks of fewer chunks run the form for one round), every block's chunks beginning at a line
+    const bool lines = !getenv("QE_NOLN") && !norm_w && mt == 1 && K % 64 == 0 && (splits == 1 || cps % 2 == 0);
     if (norm_w) {
         QE_REQUIRE(qe_gemm_skinny_norm_ok(M, N, K) && splits == 1, "skinny gemm: the norm prologue takes up to 16 rows, K <= 8192");
         if constexpr (SILU) QE_SKINNY_W(1, 1, 8, true);
         else if constexpr (EPI == EPI_STORE) QE_SKINNY_W(1, 1, 4, true);
         else QE_REQUIRE(false, "skinny gemm: the norm prologue goes with the store and silu-mul epilogues");
     } else if (mt == 1 && SILU) {
-        if constexpr (SILU) QE_SKINNY_W(1, 1, 8, false);
+        if constexpr (SILU) {
+            if (lines && cps > 8 * 4) {
+                if (M > 8) QE_SKINNY_K(1, 1, 8, false, true, true);
+                else QE_SKINNY_K(1, 1, 8, false, true, false);
+            } else {
+                QE_SKINNY_W(1, 1, 8, false);
+            }
+        }
     } else if (four) {
         if constexpr (!SILU) QE_SKINNY(1, 4);
     } else if (two) {
@@ -477,7 +563,14 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
         }
     } else {
         switch (mt) {
-            case 1: QE_SKINNY(1, 1); break;
+            case 1:
+                if (lines && cps > 4 * 8) {
+                    if (M > 8) QE_SKINNY_K(1, 1, 4, false, true, true);
+                    else QE_SKINNY_K(1, 1, 4, false, true, false);
+                } else {
+                    QE_SKINNY(1, 1);
+                }
+                break;
             case 2: QE_SKINNY(2, 1); break;
             case 3: QE_SKINNY(3, 1); break;
             default: QE_SKINNY(4, 1); break;
@@ -485,6 +578,7 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
     }
 #undef QE_SKINNY
 #undef QE_SKINNY_W
+#undef QE_SKINNY_K
     QE_LAUNCH_CHECK();
     return 0;
 }
