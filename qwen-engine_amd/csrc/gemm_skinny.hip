@@ -298,7 +298,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
             if (c <= last) { QE_LOAD_W() }
         }
         QE_KEEP(acc)
-    } else if (c_end - c_begin <= WAVES * U) {
+    } else if (!LN && c_end - c_begin <= WAVES * U) {
         // One round at most a wave (the small model's products).
         floatx4 acc[NT][NW][MT];
         QE_ZERO(acc)
@@ -511,11 +511,14 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
     // two tiles of outputs a block where the activations have more than 16 rows and there are blocks
     // enough all the same (with silu.mul a tile of outputs is two tiles of W already: only up to 32 rows)
     const bool two = mt >= 2 && (!SILU || mt <= 2) && (long)qe_cdiv(N, 32) * splits >= 256;
-    // ... and four where 9 to 16 rows meet a matrix of very many rows (the logits'): the activations are
-    // then a ninth of what a block reads instead of a third (16 rows against the 8B sizes' logits: 266 us
-    // against 289; up to 8 rows one tile a block with two rounds in flight is as fast or faster: 236
-    // against 245 us with eight rows, 200 against 239 with two)
-    const bool four = !SILU && mt == 1 && M > 8 && (long)qe_cdiv(N, 64) * splits >= 2048;
+    // whole lines of K a load (see the kernel): up to 16 rows, one tile of outputs a block, several rounds of
+    // chunks a wave (blocks of fewer chunks run the form for one round, but against a large matrix), every
+    // block's chunks beginning at a line
+    const bool lines = !norm_w && mt == 1 && K % 64 == 0 && (splits == 1 || cps % 2 == 0);
+    // ... and four where 9 to 16 rows meet a matrix of very many rows (the logits') whose K is not in whole
+    // lines: the activations are then a ninth of what a block reads instead of a third (16 rows against the 8B
+    // sizes' logits: 266 us against 289; with whole lines a load, one tile a block: 234)
+    const bool four = !lines && !SILU && mt == 1 && M > 8 && (long)qe_cdiv(N, 64) * splits >= 2048;
     const dim3 grid(qe_cdiv(N, four ? 64 : (two ? 32 : 16)), splits);
 #define QE_SKINNY_W(MT_, NT_, WAVES_, NORM_) QE_SKINNY_K(MT_, NT_, WAVES_, NORM_, false, false)
 #define QE_SKINNY_K(MT_, NT_, WAVES_, NORM_, LN_, XH_)                                                 \
@@ -536,9 +539,6 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
                                                  delta, n_delta, h_out);                               \
     } while (0)
 #define QE_SKINNY(MT_, NT_) QE_SKINNY_W(MT_, NT_, 4, false)
-    // whole lines of K a load (see the kernel): up to 16 rows, one tile of outputs a block, several rounds of
-    // chunks a wave (blocks of fewer chunks run the form for one round), every block's chunks beginning at a line
-    const bool lines = !getenv("QE_NOLN") && !norm_w && mt == 1 && K % 64 == 0 && (splits == 1 || cps % 2 == 0);
     if (norm_w) {
         QE_REQUIRE(qe_gemm_skinny_norm_ok(M, N, K) && splits == 1, "skinny gemm: the norm prologue takes up to 16 rows, K <= 8192");
         if constexpr (SILU) QE_SKINNY_W(1, 1, 8, true);
@@ -564,7 +564,7 @@ static int launch_skinny(const void* x, const void* w, const float* bias, void* 
     } else {
         switch (mt) {
             case 1:
-                if (lines && cps > 4 * 8) {
+                if (lines && (cps > 4 * 8 || (long)N * K >= (16L << 20))) {      // (one round too, against a large matrix)
                     if (M > 8) QE_SKINNY_K(1, 1, 4, false, true, true);
                     else QE_SKINNY_K(1, 1, 4, false, true, false);
                 } else {

@@ -983,13 +983,15 @@ def test_decode_kernel_with_more_than_32_splits(ops, L):
 
 
 @pytest.mark.parametrize("M", [1, 2, 5, 8, 16, 64])
-def test_gemm_for_few_rows_against_the_whole_vocabulary(ops, M):
-    """The head's product at the family's vocabulary: [M, 1024] against [151936, 1024], 32-bit logits,
+@pytest.mark.parametrize("K", [1024, 1056])
+def test_gemm_for_few_rows_against_the_whole_vocabulary(ops, M, K):
+    """The head's product at the family's vocabulary: [M, K] against [151936, K], 32-bit logits,
     compared in 64-bit on the first and last columns and on 3000 drawn ones.  Up to 16 rows (one tile
-    of rows, whether a block owns one tile of outputs or four) a row's logits are the same bits
-    whatever else is in the batch."""
+    of rows; K = 1024: whole lines of 128 bytes a load, one tile of outputs a block; K = 1056, an odd
+    number of chunks of 32: one tile a block up to 8 rows, four from 9 on) a row's logits are the same
+    bits whatever else is in the batch."""
     bf = torch.bfloat16
-    N, K = 151936, 1024
+    N = 151936
     x, w = rand(M, K, seed=520, dtype=bf), rand(N, K, seed=521, dtype=bf, scale=0.02)
     got = ops.gemm(x.to(DEV), w.to(DEV), out_dtype=torch.float32).cpu()
     assert got.shape == (M, N) and torch.isfinite(got).all()
