@@ -4,10 +4,15 @@
 //
 // A block of 4 waves owns 16 rows of W (or two such tiles).  The rows are the M side of v_mfma_f32_16x16x32_bf16
 // (lane (g, r), g = lane / 16, r = lane % 16, holds W[n0 + r][c * 32 + g * 8 .. + 8]: one 16-byte
-// load), the tokens are the N side (lane (g, r) holds x[j * 16 + r][the same k]).  Wave w takes
-// the 32-wide chunks c = w, w + 4, ... of K, so the four waves read neighbouring 64-byte pieces
-// of the same rows at the same time; their partial tiles are summed through shared memory.
+// load), the tokens are the N side (lane (g, r) holds x[j * 16 + r][the same k]).  The waves split
+// the 32-wide chunks of K between them (in pairs: wave w takes the chunks 2 w, 2 w + 1, 2 w + 8, ...;
+// see the kernel); their partial tiles are summed through shared memory.
 // The result tile has, per lane, 4 consecutive n for one token: one 8- or 16-byte store.
+//
+// Against a large matrix with up to 16 rows of x the loads do not follow the operand layout (4 lanes
+// and 64 bytes a row) but take whole 128-byte lines, 8 lanes a row, and the registers are turned into
+// the operand layout through shared memory: the L1 serves half as many requests, which is what bounds
+// the stream once rows of x are read beside the weights (see LN in the kernel).
 //
 // Epilogues: store (+ bias); add into a 32-bit residual stream; silu(gate) * up, where W holds
 // the gate rows followed by the up rows and a block owns 16 of each; 32-bit partial products
@@ -183,8 +188,8 @@ __device__ __forceinline__ void norm_rows_into_lds(const float* __restrict__ hs,
 // order of s (the fused residual-add + norm kernel does), so the sum has one fixed order.
 // NT: tiles of 16 rows of W a block owns.  Every wave reads the activations of its chunks itself
 // (M rows against the block's 16 NT rows of W), so with more than 16 rows of activations most of
-// what a block reads is activations, from the L2; two tiles a block halve that, four quarter it
-// (8 rows against the logits' matrix: 4.15 TB/s of weights with one tile a block, 6.07 with one row).
+// what a block reads is activations, from the L2; two tiles a block halve that, four quarter it.
+// LN: whole lines a load (up to 16 rows, one tile a block); XH: more than 8 rows of x then.
 template <int MT, int NT, int EPI, typename TO, int WAVES, bool NORM, bool LN = false, bool XH = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     const void* __restrict__ x_in, const bf16_t* __restrict__ w, const float* __restrict__ bias,
