@@ -586,20 +586,27 @@ template <typename TO, bool SILU>
 static int pick_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                      int tile, int splits, hipStream_t stream) {
     if (tile == 0) tile = choose_tile(M, N, splits);
+    // Up to 64 rows against a gate|up matrix of at most one tile column a compute unit (its K cannot be
+    // cut): a block streams its weights alone on its unit, and what it has in flight bounds it.  A k step of
+    // 128 doubles that (24576 x 4096 against 64 rows: 44.4 us against 49.2; with two blocks a unit, 51200 x
+    // 5120, it gains nothing).
+    if (tile == 0 && SILU && M <= 64 && qe_cdiv(N, 128) <= 256) tile = 65;
+    if (tile == 65) return launch_mfma<TO, 64, 128, 128, 4, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 512) return launch_mfma<TO, 256, 256, 64, 4, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 256) return launch_mfma<TO, 256, 128, 64, 8, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 128) return launch_mfma<TO, 128, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, splits, stream);
     return launch_mfma<TO, 64, 128, 64, 4, 2, SILU>(x, w, bias, out, M, N, K, splits, stream);
 }
 
-// tile: rows of the output tile (256, 128 or 64; 512 stands for 256 x 256), 0 to choose by the shape.  silu: w is [N, K] with
+// tile: rows of the output tile (256, 128 or 64; 512 stands for 256 x 256, 65 for 64 x 128 with a k step of 128), 0 to choose
+// by the shape.  silu: w is [N, K] with
 // gate and up rows interleaved in blocks of 32, out is [M, N / 2] = silu(gate) * up.
 // splits > 1: out is float [splits, M, N], partial products along K (no silu then).
 int qe_gemm_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int dt_o,
                  int tile, bool silu, int splits, hipStream_t stream) {
     QE_REQUIRE(splits >= 1 && (splits == 1 || (!silu && dt_o == QE_F32)), "mfma gemm: partial products are 32-bit and plain");
     QE_REQUIRE(K % 8 == 0 && K >= 64 && K < (1 << 22), "mfma gemm: K=%d is no multiple of 8 in [64, 2^22)", K);
-    QE_REQUIRE(tile == 0 || tile == 512 || tile == 256 || tile == 128 || tile == 64, "mfma gemm: tile of %d rows", tile);
+    QE_REQUIRE(tile == 0 || tile == 512 || tile == 256 || tile == 128 || tile == 64 || tile == 65, "mfma gemm: tile of %d rows", tile);
     if (silu) {
         QE_REQUIRE(!bias && N % 64 == 0, "mfma gemm: silu-mul takes no bias and gate|up rows in blocks of 32");
         if (dt_o == QE_BF16) return pick_mfma<bf16_t, true>(x, w, bias, out, M, N, K, tile, splits, stream);

@@ -18,7 +18,7 @@ F32, BF16 = 0, 1
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
 
 ALGO_AUTO, ALGO_GENERIC, ALGO_FAST = 0, 1, 2
-ALGO_TILE = 1000   # ALGO_TILE + 256, 128 or 64: the tiled MFMA gemm with tiles of that many rows
+ALGO_TILE = 1000   # ALGO_TILE + 256, 128 or 64: the tiled MFMA gemm with tiles of that many rows (+ 512: 256 x 256; + 65: 64 rows, k step 128)
 EPI_STORE, EPI_RESIDUAL, EPI_SILU_MUL, EPI_PARTIAL, EPI_SILU_MUL_IL = 0, 1, 2, 3, 4
 DECODE_SPLIT_KEYS = 128   # keys per split of the decode attention kernel
 

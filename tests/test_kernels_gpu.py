@@ -717,7 +717,7 @@ def test_gemm_tiled_mfma(ops, M, N, K):
     want = P.linear(x.double(), w.double())
     got = ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_FAST)
     close(got, want, bf)
-    for rows in (64, 128, 256, 512):                         # every tile shape on every size (512: 256 x 256)
+    for rows in (64, 65, 128, 256, 512):                     # every tile shape on every size (512: 256 x 256; 65: 64 rows, k step 128)
         close(ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_TILE + rows), want, bf)
         close(ops.gemm(x.to(DEV), w.to(DEV), bias.to(DEV), out_dtype=torch.float32, algo=ops.ALGO_TILE + rows),
               want + bias.double(), torch.float32, scale=float(want.abs().max()))
@@ -943,10 +943,31 @@ def test_gemm_with_silu_mul_over_interleaved_rows(ops, M, I, K):
     if ops.gemm_silu_supported(x.to(DEV), w.to(DEV)):
         close(ops.gemm(x.to(DEV), w.to(DEV), epilogue=ops.EPI_SILU_MUL_IL), want, bf)
         if M > 64:
-            for rows in (64, 128, 256, 512):
+            for rows in (64, 65, 128, 256, 512):
                 close(ops.gemm(x.to(DEV), w.to(DEV), epilogue=ops.EPI_SILU_MUL_IL, algo=ops.ALGO_TILE + rows), want, bf)
     gu = ops.gemm(x.to(DEV), w.to(DEV), algo=ops.ALGO_GENERIC)
     close(ops.silu_mul(gu, interleaved=True), want, bf)
+
+
+@pytest.mark.parametrize("M", [17, 40, 64])
+def test_gemm_of_few_rows_against_a_large_matrix(ops, M):
+    """17 to 64 rows against 16 M weights and more go through the tiled kernel: gate|up with silu.mul in a
+    tile shape of its own, the others as partial products in as many cuts of K as the kernel asks for."""
+    bf = torch.bfloat16
+    I, K = 4096, 2048
+    g, u = rand(I, K, seed=180, dtype=bf, scale=0.2), rand(I, K, seed=181, dtype=bf, scale=0.2)
+    x = rand(M, K, seed=182, dtype=bf)
+    w = ops.interleave_gate_up(g, u).to(DEV)
+    want = P.silu_mul(P.linear(x.double(), g.double()), P.linear(x.double(), u.double()))
+    close(ops.gemm(x.to(DEV), w, epilogue=ops.EPI_SILU_MUL_IL), want, bf)
+    close(ops.gemm(x.to(DEV), w, epilogue=ops.EPI_SILU_MUL_IL, algo=ops.ALGO_TILE + 64), want, bf)
+    wd = torch.cat([g, u]).to(DEV)                           # [8192, 2048]: 64 tile columns, so 4 cuts
+    cuts = ops.gemm_branch_splits(x.to(DEV), wd)
+    assert cuts == 4
+    parts = ops.gemm(x.to(DEV), wd, epilogue=ops.EPI_PARTIAL, splits=cuts)
+    assert parts.shape == (cuts, M, 2 * I) and parts.dtype == torch.float32
+    want = P.linear(x.double(), torch.cat([g, u]).double())
+    close(parts.sum(0), want, torch.float32, scale=float(want.abs().max()))
 
 
 @pytest.mark.parametrize("L", [4096, 4097, 8300])
