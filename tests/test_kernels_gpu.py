@@ -526,6 +526,26 @@ def test_gemm_for_few_rows_over_rounds_of_chunks(ops, N, K):
             assert float((got.double().cpu() - want_g).abs().max()) <= 1e-5 * float(want_g.abs().max()), ("silu, interleaved", M)
 
 
+@pytest.mark.parametrize("N,K", [(8201, 2112), (9000, 2080), (8200, 4160)])
+def test_gemm_for_few_rows_whose_sizes_are_no_multiples_of_the_tiles(ops, N, K):
+    """A matrix large enough for the whole-line loads whose last tile of rows is partly beyond the matrix, with
+    a K of 33 and 65 lines and with one that is no whole number of lines (which takes the other form), for
+    row counts inside the first and the third tile of 16: every output, in 64-bit."""
+    bf = torch.bfloat16
+    g = torch.Generator().manual_seed(N + K)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(bf)
+    wd = w.to(DEV)
+    for M in (1, 3, 11, 16, 40):
+        x = torch.randn(M, K, generator=g).to(bf)
+        want = x.double() @ w.double().t()
+        scale = float(want.abs().max())
+        got = ops.gemm(x.to(DEV), wd, out_dtype=torch.float32)
+        assert float((got.double().cpu() - want).abs().max()) <= 3e-6 * scale, ("store", M)
+        for splits in (2, 4):
+            parts = ops.gemm(x.to(DEV), wd, epilogue=ops.EPI_PARTIAL, splits=splits)
+            assert float((parts.sum(0).double().cpu() - want).abs().max()) <= 3e-6 * scale, ("partial", splits, M)
+
+
 @pytest.mark.parametrize("M", [1, 8, 40, 64])
 @pytest.mark.parametrize("I,K", [(160, 96), (112, 64), (3072, 1024)])
 def test_gemm_with_silu_mul(ops, M, I, K):
