@@ -585,12 +585,12 @@ static int choose_tile(int M, int N, int splits, bool with_256x256 = true) {
 template <typename TO, bool SILU>
 static int pick_mfma(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                      int tile, int splits, hipStream_t stream) {
-    if (tile == 0) tile = choose_tile(M, N, splits);
     // Up to 64 rows against a gate|up matrix of at most one tile column a compute unit (its K cannot be
     // cut): a block streams its weights alone on its unit, and what it has in flight bounds it.  A k step of
     // 128 doubles that (24576 x 4096 against 64 rows: 44.4 us against 49.2; with two blocks a unit, 51200 x
     // 5120, it gains nothing).
     if (tile == 0 && SILU && M <= 64 && qe_cdiv(N, 128) <= 256) tile = 65;
+    if (tile == 0) tile = choose_tile(M, N, splits);
     if (tile == 65) return launch_mfma<TO, 64, 128, 128, 4, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 512) return launch_mfma<TO, 256, 256, 64, 4, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
     if (tile == 256) return launch_mfma<TO, 256, 128, 64, 8, 1, SILU>(x, w, bias, out, M, N, K, splits, stream);
