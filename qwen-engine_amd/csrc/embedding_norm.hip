@@ -64,57 +64,71 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ del
 }
 
 // The same for rows of up to NV * 4 * blockDim.x elements with H % 4 == 0: the row is read once
-// (16-byte loads, all in flight together) and kept in registers.  This is the kernel of decode
-// steps, where a launch has few rows and its time is the latency of its memory accesses.
-template <typename TA, typename TD, int NV>
-__global__ void rmsnorm_regs_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_delta, long delta_stride,
+// (16-byte loads) and kept in registers.  This is the kernel of decode steps, where a launch has few
+// rows and its time is the latency of its memory accesses: the row's pieces and the parts to add are
+// asked for together, SB parts of all pieces at a time, before the first is added, from addresses that
+// are always valid (a piece beyond the row or a part beyond the last reads another again and is not
+// used), so that no branch stands between the loads and a trip to memory serves them all.  (With a
+// trip per piece, a row of 4096 with eight parts took 6.8 us.)  The parts are added in ascending order.
+// FEW: few rows, SB = 8 (or 4) parts at a time; many rows fill the chip anyway and are bound by the
+// memory's rate, which more waves a compute unit (fewer registers: two parts at a time) serve better.
+template <typename TA, typename TD, int NV, bool FEW>
+__global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_delta, long delta_stride,
                                     const int* __restrict__ rows, const float* __restrict__ w,
                                     TA* __restrict__ out, int H, float eps) {
+    constexpr int SB = !FEW ? 2 : (NV <= 4 ? 8 : 4);
     __shared__ float red[16];
     const long r = blockIdx.x;
     const long src = rows ? (long)rows[r] : r;
     float* hr = h + src * H;
     const TD* dr = delta ? delta + src * H : nullptr;
-    float v[NV][4];
-    float ss = 0.f;
+    int cs[NV];
+    bool ok[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int c = (threadIdx.x + i * blockDim.x) * 4;
-        if (c < H) {
-            Vec4<float>::load(hr + c, v[i]);
-            if (dr) {
-                // the parts are asked for eight at a time, all before the first is added (one trip
-                // to memory for eight), and added in ascending order
-                for (int s0 = 0; s0 < n_delta; s0 += 8) {
-                    float d[8][4];
+        ok[i] = c < H;
+        cs[i] = ok[i] ? c : 0;
+    }
+    float v[NV][4];
 #pragma unroll
-                    for (int s = 0; s < 8; ++s)
-                        if (s0 + s < n_delta) Vec4<TD>::load(dr + (s0 + s) * delta_stride + c, d[s]);
+    for (int i = 0; i < NV; ++i) Vec4<float>::load(hr + cs[i], v[i]);
+    if (dr) {
+        for (int s0 = 0; s0 < n_delta; s0 += SB) {
+            float d[SB][NV][4];
 #pragma unroll
-                    for (int s = 0; s < 8; ++s)
-                        if (s0 + s < n_delta) {
+            for (int s = 0; s < SB; ++s) {
+                const TD* part = dr + (long)min(s0 + s, n_delta - 1) * delta_stride;
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[i][e] += d[s][e];
-                        }
-                }
+                for (int i = 0; i < NV; ++i) Vec4<TD>::load(part + cs[i], d[s][i]);
             }
 #pragma unroll
-            for (int e = 0; e < 4; ++e) ss += v[i][e] * v[i][e];
+            for (int s = 0; s < SB; ++s)
+                if (s0 + s < n_delta) {
+#pragma unroll
+                    for (int i = 0; i < NV; ++i)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[i][e] += d[s][i][e];
+                }
         }
     }
     float wv[NV][4];                       // the weights are asked for before the sum is waited for
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-        const int c = (threadIdx.x + i * blockDim.x) * 4;
-        if (c < H) Vec4<float>::load(w + c, wv[i]);
-    }
+    for (int i = 0; i < NV; ++i) Vec4<float>::load(w + cs[i], wv[i]);
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+        if (ok[i]) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ss += v[i][e] * v[i][e];
+        }
     ss = block_sum(ss, red);
     const float rstd = rsqrtf(ss / (float)H + eps);
     const bool write_back = dr && !rows;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int c = (threadIdx.x + i * blockDim.x) * 4;
-        if (c < H) {
+        if (ok[i]) {
+            const int c = cs[i];
             if (write_back) Vec4<float>::store(hr + c, v[i]);
             float o[4];
 #pragma unroll
@@ -131,8 +145,15 @@ static void launch_rmsnorm(float* h, const void* delta, int n_delta, long stride
         int threads = ((H / 4 + 63) / 64) * 64;
         if (threads > 256) threads = 256;
         const int nv = (H / 4 + threads - 1) / threads;
-#define QE_NORM(NV_) rmsnorm_regs_kernel<TA, TD, NV_><<<n_out_rows, threads, 0, stream>>>( \
-        h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps)
+#define QE_NORM(NV_)                                                                                         \
+    do {                                                                                                     \
+        if (n_out_rows <= 512)                                                                               \
+            rmsnorm_regs_kernel<TA, TD, NV_, true><<<n_out_rows, threads, 0, stream>>>(                      \
+                h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps);                            \
+        else                                                                                                 \
+            rmsnorm_regs_kernel<TA, TD, NV_, false><<<n_out_rows, threads, 0, stream>>>(                     \
+                h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps);                            \
+    } while (0)
         if (nv <= 1) QE_NORM(1);
         else if (nv <= 2) QE_NORM(2);
         else if (nv <= 4) QE_NORM(4);
