@@ -138,6 +138,45 @@ struct QkvSource {
 #pragma unroll
         for (int e = 0; e < 4; ++e) { Elem<TA>::store(r + e, v[e]); v[e] = Elem<TA>::load(r + e); }
     }
+    // The same for two places of four elements at once (the two halves of a head that rotate together): the
+    // parts of both are asked for together, and a part beyond the last is skipped by a select, not by a
+    // branch, so that one trip to memory serves all of them.
+    __device__ __forceinline__ void load4x2(long idx_a, int col_a, long idx_b, int col_b, float (&a)[4], float (&b)[4]) const {
+        if (qkv) {
+            Vec4<TA>::load(qkv + idx_a, a);
+            Vec4<TA>::load(qkv + idx_b, b);
+            return;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[e] = b[e] = 0.f;
+        for (int s0 = 0; s0 < S; s0 += 8) {
+            float pa[8][4], pb[8][4];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int sk = s0 + k < S ? s0 + k : S - 1;
+                Vec4<float>::load(parts + sk * stride + idx_a, pa[k]);
+                Vec4<float>::load(parts + sk * stride + idx_b, pb[k]);
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const bool on = s0 + k < S;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    a[e] = on ? a[e] + pa[k][e] : a[e];
+                    b[e] = on ? b[e] + pb[k][e] : b[e];
+                }
+            }
+        }
+        if (bias) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { a[e] += bias[col_a + e]; b[e] += bias[col_b + e]; }
+        }
+        TA r[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { Elem<TA>::store(r + e, a[e]); a[e] = Elem<TA>::load(r + e); }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { Elem<TA>::store(r + e, b[e]); b[e] = Elem<TA>::load(r + e); }
+    }
     __device__ __forceinline__ float load1(long idx, int col) const {
         if (qkv) return Elem<TA>::load(qkv + idx);
         float v = parts[idx];
@@ -154,7 +193,7 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
     const QkvSource<TA> in, const int* __restrict__ positions,
     const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
     const float* __restrict__ table, const int* __restrict__ slot, TA* __restrict__ cache,
-    TA* __restrict__ q_out, TA* __restrict__ packed_out, int Hq, int Hkv, int D, int P) {
+    TA* __restrict__ q_out, TA* __restrict__ packed_out, int Hq, int Hkv, int D, int P, int value_blocks) {
     const long t = blockIdx.x;
     const int lph = D / 8;                     // lanes per head
     const int half = D / 2;
@@ -165,14 +204,28 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
     const int s = slot ? slot[t] : -1;
     const float* cs = table ? table + (long)positions[t] * D : nullptr;
     const int nloop = packed_out ? nheads : Hq + Hkv;   // (values go to the cache by tiles, further down)
-    // (the blocks (t, 0 .. gridDim.y - 1) share the token's heads: more blocks where the tokens are few)
-    for (int head = threadIdx.x / lph + blockIdx.y * heads_per_pass; head < nloop; head += heads_per_pass * gridDim.y) {
+    // (the blocks (t, 0 .. ny - 1) share the token's heads: more blocks where the tokens are few; with
+    // value_blocks = 1 the last block of a token takes no heads but the values, further down, which block 0
+    // does after its heads otherwise: a kernel for few tokens lasts as long as its longest chain of loads)
+    const int ny = (int)gridDim.y - value_blocks;
+    const int first = (int)blockIdx.y < ny ? (int)(threadIdx.x / lph + blockIdx.y * heads_per_pass) : nloop;
+    for (int head = first; head < nloop; head += heads_per_pass * ny) {
         const bool is_q = head < Hq;
         const bool is_k = !is_q && head < Hq + Hkv;
         const long src = t * width + (long)head * D;   // element index of the head's first feature
+        // the norm's weights and the table's row are asked for before the head, not after it has arrived
+        const float* w = is_q ? q_w : k_w;
+        float wa[4], wb[4], c[4], sn[4];
+        if (w) {
+            Vec4<float>::load(w + 4 * j, wa);
+            Vec4<float>::load(w + half + 4 * j, wb);
+        }
+        if (cs) {
+            Vec4<float>::load(cs + 4 * j, c);
+            Vec4<float>::load(cs + half + 4 * j, sn);
+        }
         float a[4], b[4];                      // features 4 j .. 4 j + 3 and half + 4 j .. half + 4 j + 3
-        in.load4(src + 4 * j, head * D + 4 * j, a);
-        in.load4(src + half + 4 * j, head * D + half + 4 * j, b);
+        in.load4x2(src + 4 * j, head * D + 4 * j, src + half + 4 * j, head * D + half + 4 * j, a, b);
         TA* dst = nullptr;
         if (packed_out) {
             dst = packed_out + t * width + (long)head * D;
@@ -193,7 +246,6 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
             }
             continue;
         }
-        const float* w = is_q ? q_w : k_w;
         if (w) {
             float ss = 0.f;
 #pragma unroll
@@ -201,16 +253,10 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
             if (lph == 16) ss = row16_sum(ss);             // (the same sum, without the LDS crossbar)
             else for (int o = lph >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
             const float rstd = rsqrtf(ss / (float)D + eps);
-            float wa[4], wb[4];
-            Vec4<float>::load(w + 4 * j, wa);
-            Vec4<float>::load(w + half + 4 * j, wb);
 #pragma unroll
             for (int e = 0; e < 4; ++e) { a[e] = a[e] * rstd * wa[e]; b[e] = b[e] * rstd * wb[e]; }
         }
         if (cs) {
-            float c[4], sn[4];
-            Vec4<float>::load(cs + 4 * j, c);
-            Vec4<float>::load(cs + half + 4 * j, sn);
 #pragma unroll
             for (int e = 0; e < 4; ++e) rotate_pair(c[e], sn[e], a[e], b[e]);
         }
@@ -219,7 +265,7 @@ __global__ __launch_bounds__(256) void qk_rope_store_vec_kernel(
             Vec4<TA>::store(dst + half + 4 * j, b);
         }
     }
-    if (packed_out || !slot || blockIdx.y != 0) return;
+    if (packed_out || !slot || (int)blockIdx.y != (value_blocks ? ny : 0)) return;
 
     // ---- values of the 16 tokens t0 .. t0 + n - 1, key/value heads t - t0, t - t0 + n, ... ----
     extern __shared__ __attribute__((aligned(16))) unsigned char vsh[];   // [D][16] elements + 16 bytes a row
@@ -295,11 +341,11 @@ extern "C" int qe_qk_rope_store(const void* qkv, const int* positions, const flo
         if (dt_a == QE_F32)
             qk_rope_store_vec_kernel<float><<<T, 256, (size_t)D * (16 * 4 + 16), stream>>>(
                 QkvSource<float>{(const float*)qkv, nullptr, nullptr, 0, 0}, positions, q_w, k_w, eps, table, slot,
-                (float*)cache, (float*)q_out, (float*)packed_out, Hq, Hkv, D, P);
+                (float*)cache, (float*)q_out, (float*)packed_out, Hq, Hkv, D, P, 0);
         else if (dt_a == QE_BF16)
             qk_rope_store_vec_kernel<bf16_t><<<T, 256, (size_t)D * (16 * 2 + 16), stream>>>(
                 QkvSource<bf16_t>{(const bf16_t*)qkv, nullptr, nullptr, 0, 0}, positions, q_w, k_w, eps, table, slot,
-                (bf16_t*)cache, (bf16_t*)q_out, (bf16_t*)packed_out, Hq, Hkv, D, P);
+                (bf16_t*)cache, (bf16_t*)q_out, (bf16_t*)packed_out, Hq, Hkv, D, P, 0);
         else
             QE_REQUIRE(false, "qk_rope_store: unknown dtype %d", dt_a);
         QE_LAUNCH_CHECK();
@@ -343,10 +389,12 @@ extern "C" int qe_qk_rope_store_parts(const float* parts, int S, const float* bi
     if (T == 0) return 0;
     const long stride = (long)T * (Hq + 2 * Hkv) * D;
     const int passes = qe_cdiv((Hq + Hkv) * (D / 8), 256);      // rounds of 256 lanes over the q and k heads of a token
-    const dim3 grid((unsigned)T, (unsigned)(passes < 4 ? passes : 4));
+    // (few tokens: a block of its own for each token's values)
+    const int value_blocks = (slot && T <= 256) ? 1 : 0;
+    const dim3 grid((unsigned)T, (unsigned)((passes < 4 ? passes : 4) + value_blocks));
     qk_rope_store_vec_kernel<bf16_t><<<grid, 256, (size_t)D * (16 * 2 + 16), stream>>>(
         QkvSource<bf16_t>{nullptr, parts, bias, S, stride}, positions, q_w, k_w, eps, table, slot,
-        (bf16_t*)cache, (bf16_t*)q_out, nullptr, Hq, Hkv, D, P);
+        (bf16_t*)cache, (bf16_t*)q_out, nullptr, Hq, Hkv, D, P, value_blocks);
     QE_LAUNCH_CHECK();
     return 0;
 }
