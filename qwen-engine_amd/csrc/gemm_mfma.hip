@@ -59,7 +59,7 @@ template <typename TO, int BM, int BN, int BK, int NW, int MINB, bool SILU, bool
 __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n, int k_per_split, int xcd_m, int xcd_n,
-    QkvTail tail) {
+    int rotate, QkvTail tail) {
     constexpr int ROWB = BK * 2 + 16;       // bytes of a staged row
     constexpr int PPR = BK / 8;             // 16-byte pieces per row
     constexpr int RPI = 64 * NW / PPR;      // rows the block stages with one piece per thread
@@ -109,6 +109,15 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const int k0 = blockIdx.y * k_per_split;
     const int klen = K - k0 < k_per_split ? K - k0 : k_per_split;
     const int nk = (klen + BK - 1) / BK;
+    // rotate: the block walks its k steps from another start than its neighbours (and wraps round).  Few rows
+    // of x against a large matrix: the blocks stream their rows of W in step, and with a row stride that is a
+    // power of two all their loads of a moment have the same address bits below the stride, which land on the
+    // same few memory channels (the logits' matrix of 151936 x 4096 against 64 rows: 4.4 TB/s, and 5.1 with a
+    // row of 4160; where the stride is no such power, walking in step is the quicker: the blocks then share
+    // their rows of x through the caches).  The order of a tile's sum is then a function of its place, not of
+    // the batch.
+    const int rot = rotate ? (tile_n * 5 + (int)blockIdx.y * 3) % nk : 0;
+#define QE_KK(kt_) ((kt_) < nk ? ((kt_) + rot < nk ? (kt_) + rot : (kt_) + rot - nk) : (kt_))
     // Two sets of staging registers in turn: a step's loads are issued two steps ahead and go to
     // shared memory one step ahead, so a load has a whole step of MFMAs to arrive.
     uint4_t stage[2][LD];
@@ -144,8 +153,9 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     const int dst = lrow * ROWB + pc * 16;                 // where piece 0 goes in a buffer; piece i: + i RPI ROWB
 #define LOAD_GLOBAL(set_, kt_)                                                           \
     {                                                                                    \
-        const bool k_ok = (kt_) * BK + pc * 8 < klen;                                    \
-        const int soff = (kt_) * BK * 2;                                                 \
+        const int kk = QE_KK(kt_);                                                       \
+        const bool k_ok = kk * BK + pc * 8 < klen;                                       \
+        const int soff = kk * BK * 2;                                                    \
         _Pragma("unroll") for (int i = 0; i < LD; ++i) {                                 \
             const int vo = k_ok ? voff[i] : 0x7fffffff;                                  \
             if constexpr (BIG) {                                                         \
@@ -227,8 +237,9 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
         b_[j] = *(const bf16x8*)(b_frag + (buf_) * BUF + j * 32 * ROWB + (ks_) * 32);
 #define LOAD_PIECE(set_, kt_, i_)                                                        \
     {                                                                                    \
-        const int vo = (kt_) * BK + pc * 8 < klen ? voff[i_] : 0x7fffffff;               \
-        const int soff = (kt_) * BK * 2;                                                 \
+        const int kk = QE_KK(kt_);                                                       \
+        const int vo = kk * BK + pc * 8 < klen ? voff[i_] : 0x7fffffff;                  \
+        const int soff = kk * BK * 2;                                                    \
         if constexpr (BIG) {                                                             \
             if ((i_) < LDA)                                                              \
                 asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                  \
@@ -296,6 +307,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     WAIT_LOADS(0, 0)
     WAIT_LOADS(1, 0)
 #undef K_STEP
+#undef QE_KK
 #undef LOAD_PIECE
 #undef READ_FRAGS
 #undef LOAD_GLOBAL
@@ -551,7 +563,8 @@ static int launch_mfma(const void* x, const void* w, const float* bias, void* ou
         if (xcd_m == 0 || rows < fewest) { xcd_m = a; xcd_n = b; fewest = rows; }
     }
     gemm_mfma_kernel<TO, BM, BN, BK, NW, MINB, SILU, QKV><<<dim3((unsigned)blocks, (unsigned)splits), 64 * NW, shmem, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n, k_per_split, xcd_m, xcd_n, tail);
+        (const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n, k_per_split, xcd_m, xcd_n,
+        (!QKV && M <= 64 && (K * 2) % 8192 == 0) ? 1 : 0, tail);
     QE_LAUNCH_CHECK();
     return 0;
 }
