@@ -24,6 +24,7 @@ request's pages the last before the first, so that no kept page outlives the pag
 from __future__ import annotations
 
 import hashlib
+import random
 from collections import OrderedDict
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
@@ -47,13 +48,28 @@ class GroupSpec:
 
 
 class PagePool:
-    """Pages of one group: LIFO free list and reference counts."""
+    """Pages of one group: LIFO free list and reference counts.
 
-    def __init__(self, num_pages: int):
+    scatter: the pages are first handed out in a fixed pseudo-random order instead of 0, 1, 2, ...:
+    aligned runs of SCATTER_RUN neighbouring pages stay together and in order, the runs are shuffled.
+    Handed out in order, the pages that a decode step reads together (the same place of every
+    request and of every split of its keys) lie at regular distances in memory, and how well the
+    memory serves them then depends on those distances: eight requests of 4096 tokens decoded in
+    1.75 to 1.94 ms a step depending on how many pages each prompt had taken (248 or 250), against
+    1.76 to 1.78 ms whatever the prompts' lengths with the pages scattered.  A pool that has served
+    requests for a while is scattered anyway; this makes a fresh one behave the same."""
+
+    SCATTER_RUN = 8
+
+    def __init__(self, num_pages: int, scatter: bool = False):
         if num_pages <= 0:
             raise CacheError("a page pool needs at least one page")
         self.num_pages = num_pages
         self.free: List[int] = list(range(num_pages - 1, -1, -1))  # pop() hands out 0 first
+        if scatter:
+            groups = [list(range(a, min(a + self.SCATTER_RUN, num_pages))) for a in range(0, num_pages, self.SCATTER_RUN)]
+            random.Random(0x5ca77e6).shuffle(groups)
+            self.free = [p for grp in groups for p in grp][::-1]
         self.refcount: List[int] = [0] * num_pages
 
     @property
@@ -168,7 +184,7 @@ class _SharedEntry:
 
 class CacheManager:
     def __init__(self, groups: Sequence[GroupSpec], num_pages, page_size: int, max_requests: int,
-                 prefix_sharing: bool = False, keep_freed_prefixes: bool = False):
+                 prefix_sharing: bool = False, keep_freed_prefixes: bool = False, scatter_pages: bool = False):
         if page_size <= 0:
             raise CacheError("page_size must be positive")
         self.groups = list(groups)
@@ -180,7 +196,7 @@ class CacheManager:
             if g.window is not None and g.window <= 0:
                 raise CacheError("a window must be positive")
         self.page_size = page_size
-        self.pools = [PagePool(n) for n in num_pages]
+        self.pools = [PagePool(n, scatter=scatter_pages) for n in num_pages]
         self.slots = StateSlots(max_requests)
         self.requests: Dict[Hashable, RequestCache] = {}
         # a prefix can only be shared when every group keeps all keys

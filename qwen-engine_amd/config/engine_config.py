@@ -18,6 +18,7 @@ class EngineConfig:
     prefill_chunk: int = 512         # largest portion of one prompt in a step in which some request decodes
     enable_prefix_sharing: bool = True
     keep_freed_prefixes: bool = True   # shared pages of finished requests stay until their memory is needed
+    scatter_pages: bool = True       # a fresh pool hands its pages out in a scattered order (see cache.manager.PagePool)
     seed: int = 0
     debug_poison: bool = False       # NaN into every cache page when it is handed out and when it goes back
     record_mixed_steps: bool = True  # steps of single new tokens beside one prompt portion are replayed from recorded graphs

@@ -51,7 +51,8 @@ class LLMEngine:
             pages = cfg.pages_per_group()
         self.runner = ModelRunner(model, page_size=cfg.block_size, num_pages=pages,
                                   max_requests=cfg.max_num_seqs, prefix_sharing=cfg.enable_prefix_sharing,
-                                  keep_freed_prefixes=cfg.keep_freed_prefixes, debug_poison=cfg.debug_poison,
+                                  keep_freed_prefixes=cfg.keep_freed_prefixes, scatter_pages=cfg.scatter_pages,
+                                  debug_poison=cfg.debug_poison,
                                   record_mixed_steps=cfg.record_mixed_steps, graph_record_after=cfg.graph_record_after,
                                   graph_memory_bytes=cfg.graph_memory_bytes)
         max_len = min(cfg.max_model_len, model.spec.max_positions)

@@ -91,7 +91,7 @@ class ModelRunner:
                  prefix_sharing: bool = False, use_graphs: Optional[bool] = None,
                  keep_freed_prefixes: bool = False, debug_poison: bool = False,
                  record_mixed_steps: bool = True, graph_record_after: int = 1,
-                 graph_memory_bytes: int = 8 << 30):
+                 graph_memory_bytes: int = 8 << 30, scatter_pages: bool = True):
         if model.rt is None:
             raise RuntimeError("the model has no weights yet")
         self.model = model
@@ -102,7 +102,7 @@ class ModelRunner:
         has_state = any(s is not None for s in self.plan.user_state)
         self.cache = CacheManager(self.plan.groups or [], num_pages, page_size, max_requests,
                                   prefix_sharing=prefix_sharing and not has_state,
-                                  keep_freed_prefixes=keep_freed_prefixes) \
+                                  keep_freed_prefixes=keep_freed_prefixes, scatter_pages=scatter_pages) \
             if self.plan.groups else CacheManager([], [], page_size, max_requests)
         dev, dt = self.rt.device, self.rt.dtype
         # debug_poison: the storage starts as NaN, and every page is filled with NaN again when it

@@ -19,6 +19,35 @@ def test_pages_are_handed_out_from_zero_and_reused_last_in_first_out():
         pool.allocate()
 
 
+def test_a_scattered_pool_hands_out_every_page_once_in_a_fixed_order():
+    """The scattered order is a permutation of the pages, the same in every pool of that size, and not the
+    order 0, 1, 2, ...; pages that come back are reused last in, first out as in the plain pool."""
+    a, b = PagePool(257, scatter=True), PagePool(257, scatter=True)
+    order = [a.allocate() for _ in range(257)]
+    assert sorted(order) == list(range(257)) and order != list(range(257))
+    assert [b.allocate() for _ in range(257)] == order
+    with pytest.raises(OutOfPages):
+        a.allocate()
+    a.release(order[5])
+    a.release(order[9])
+    assert a.allocate() == order[9] and a.allocate() == order[5]
+    # aligned runs of neighbouring pages stay together and in order; the runs lie at no regular distances
+    run = PagePool.SCATTER_RUN
+    c = PagePool(32 * run, scatter=True)
+    order = [c.allocate() for _ in range(32 * run)]
+    starts = order[::run]
+    assert sorted(order) == list(range(32 * run)) and all(s % run == 0 for s in starts)
+    assert all(order[i:i + run] == list(range(order[i], order[i] + run)) for i in range(0, 32 * run, run))
+    assert len({b - a for a, b in zip(starts, starts[1:])}) > 16
+    m = CacheManager([GroupSpec(), GroupSpec(window=8)], [64, 64], page_size=4, max_requests=2, scatter_pages=True)
+    m.add_request("r")
+    m.reserve("r", 40)
+    m.commit("r", list(range(40)))
+    m.check_invariants()
+    m.free_request("r")
+    assert all(pool.num_free == 64 for pool in m.pools)
+
+
 def test_reference_counts_refuse_misuse():
     pool = PagePool(2)
     p = pool.allocate()
