@@ -43,10 +43,12 @@ def test_greedy_generation_equals_the_plain_implementation(folders):
 
 @pytest.mark.parametrize("sizes", [dict(max_num_seqs=1), dict(max_step_tokens=7, prefill_chunk=6),
                                    dict(num_blocks=9, block_size=8), dict(block_size=1, num_blocks=200),
-                                   dict(enable_prefix_sharing=False)])
+                                   dict(enable_prefix_sharing=False), dict(scatter_pages=False),
+                                   dict(scatter_pages=False, num_blocks=9)])
 def test_outputs_do_not_depend_on_the_engine_sizes(folders, sizes):
     """Second tiny configuration: prompts of 1, 7, 16 and 30 tokens, two sharing 16 tokens; portions
-    of 6 mixed with decoding; few pages (preemption); greedy and temperature 0.7 with a fixed seed."""
+    of 6 mixed with decoding; few pages (preemption); pages handed out in a scattered order (the
+    default) and in the order 0, 1, 2, ...; greedy and temperature 0.7 with a fixed seed."""
     cfg, w = P.read_folder(folders["B"])
     p = prompts_for(cfg, (1, 7, 16, 30), 2)
     p[3] = p[2] + p[3][16:]                               # the last two share a prefix of 16 tokens
