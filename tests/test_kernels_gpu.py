@@ -969,21 +969,22 @@ def test_gemm_with_silu_mul_over_interleaved_rows(ops, M, I, K):
     close(ops.silu_mul(gu, interleaved=True), want, bf)
 
 
+@pytest.mark.parametrize("I,K,cuts_wanted", [(4096, 2048, 4), (2048, 4096, 8)])
 @pytest.mark.parametrize("M", [17, 40, 64])
-def test_gemm_of_few_rows_against_a_large_matrix(ops, M):
+def test_gemm_of_few_rows_against_a_large_matrix(ops, M, I, K, cuts_wanted):
     """17 to 64 rows against 16 M weights and more go through the tiled kernel: gate|up with silu.mul in a
-    tile shape of its own, the others as partial products in as many cuts of K as the kernel asks for."""
+    tile shape of its own, the others as partial products in as many cuts of K as the kernel asks for.  With
+    rows of 8192 bytes (K = 4096) every block starts its walk along K at another step."""
     bf = torch.bfloat16
-    I, K = 4096, 2048
     g, u = rand(I, K, seed=180, dtype=bf, scale=0.2), rand(I, K, seed=181, dtype=bf, scale=0.2)
     x = rand(M, K, seed=182, dtype=bf)
     w = ops.interleave_gate_up(g, u).to(DEV)
     want = P.silu_mul(P.linear(x.double(), g.double()), P.linear(x.double(), u.double()))
     close(ops.gemm(x.to(DEV), w, epilogue=ops.EPI_SILU_MUL_IL), want, bf)
     close(ops.gemm(x.to(DEV), w, epilogue=ops.EPI_SILU_MUL_IL, algo=ops.ALGO_TILE + 64), want, bf)
-    wd = torch.cat([g, u]).to(DEV)                           # [8192, 2048]: 64 tile columns, so 4 cuts
+    wd = torch.cat([g, u]).to(DEV)                           # [8192, 2048]: 64 tile columns, so 4 cuts; [4096, 4096]: 32, so 8
     cuts = ops.gemm_branch_splits(x.to(DEV), wd)
-    assert cuts == 4
+    assert cuts == cuts_wanted
     parts = ops.gemm(x.to(DEV), wd, epilogue=ops.EPI_PARTIAL, splits=cuts)
     assert parts.shape == (cuts, M, 2 * I) and parts.dtype == torch.float32
     want = P.linear(x.double(), torch.cat([g, u]).double())
